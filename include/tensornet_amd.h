@@ -1,0 +1,275 @@
+/*
+ * tensornet_amd.h -- C ABI of the MI355X (gfx950) implementation of TensorNet's
+ * sparse parameter-server hot path: the per-batch pull / push a single worker's
+ * SparseTable serves, and the DenseTable flat-array optimizer update.
+ *
+ * Every entry point mirrors one interface of the reference (cited as
+ * path:line relative to the reference tree) and follows these conventions:
+ *   - returns an int status (TN_OK == 0); never aborts, never throws.
+ *     tn_last_error() gives the message of the calling thread's last failure.
+ *     Conditions the reference turns into a fatal CHECK come back as codes.
+ *   - "device" pointers are plain HIP device addresses owned by the caller;
+ *     "host" pointers are ordinary host memory.  The library never frees or
+ *     keeps caller memory, and never copies table rows to the host.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     All work of a call is enqueued on that stream.  Calls on one table are
+ *     serialised by a per-table host mutex; use one stream per table.
+ *   - signs are uint64 carried in int64 tensors, exactly as in
+ *     core/kernels/sparse_table_ops.cc:119,124.
+ */
+#ifndef TENSORNET_AMD_H_
+#define TENSORNET_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ----------------------------------------------------------------- status */
+enum {
+    TN_OK = 0,
+    TN_ERR_INVALID_ARGUMENT = 1, /* errors::InvalidArgument in the ops        */
+    TN_ERR_BAD_HANDLE = 2,       /* CHECK core/ps/table/sparse_table.cc:147   */
+    TN_ERR_DIM_MISMATCH = 3,     /* CHECK_EQ core/kernels/sparse_table_ops.cc:204,340 */
+    TN_ERR_VAR_CAPACITY = 4,     /* CHECK_LT core/kernels/sparse_table_ops.cc:136 */
+    TN_ERR_UNKNOWN_KEY = 5,      /* CHECK core/ps/optimizer/optimizer_kernel.h:315 */
+    TN_ERR_TABLE_FULL = 6,       /* HBM table has no free slot left           */
+    TN_ERR_HIP = 7,              /* a HIP runtime call failed                 */
+    TN_ERR_ALREADY_INIT = 8,     /* CHECK core/ps/table/dense_table.cc:39     */
+    TN_ERR_NOT_INIT = 9,
+    TN_ERR_OUT_OF_MEMORY = 10,
+    TN_ERR_UNSUPPORTED = 11
+};
+
+/* Message of the last failing call made by the calling thread ("" if none). */
+const char* tn_last_error(void);
+
+/* Library version string. */
+const char* tn_version(void);
+
+/* ------------------------------------------------------------- optimizers */
+/*
+ * Hyper-parameter blocks.  Field names, types (all float in the reference's
+ * structs, doubles coming from Python are narrowed) and defaults follow
+ * core/ps/optimizer/optimizer.h:36-144 with the Python-side defaults of
+ * core/main/py_wrapper.cc:94-104 (AdaGrad), :121-127 (Adam), :149-156 (Ftrl).
+ * tn_*_params_default() fills in those defaults.
+ */
+typedef struct tn_adagrad_params {
+    float learning_rate;     /* 0.01 */
+    float show_decay_rate;   /* 0.98 */
+    float show_threshold;    /* 0.0  */
+    float initial_g2sum;     /* 0    */
+    float initial_scale;     /* 1    */
+    float epsilon;           /* 1e-8 */
+    float grad_decay_rate;   /* 1.0  */
+    float mom_decay_rate;    /* 1.0  */
+    int32_t no_show_days;    /* 1000 */
+    int32_t elimination_logic; /* 0 or 1 */
+} tn_adagrad_params;
+
+typedef struct tn_adam_params {
+    float learning_rate;   /* 0.01 */
+    float show_decay_rate; /* 0.98 */
+    float beta1;           /* 0.9  */
+    float beta2;           /* 0.999 */
+    float epsilon;         /* 1e-8 */
+    float initial_scale;   /* 1.0  */
+} tn_adam_params;
+
+typedef struct tn_ftrl_params {
+    float learning_rate;   /* 0.01 */
+    float show_decay_rate; /* 0.98 */
+    float show_threshold;  /* 0.0  */
+    float beta;            /* 1    */
+    float lambda1;         /* 0.1  */
+    float lambda2;         /* 1    */
+    float initial_scale;   /* 1.0  */
+} tn_ftrl_params;
+
+void tn_adagrad_params_default(tn_adagrad_params* p);
+void tn_adam_params_default(tn_adam_params* p);
+void tn_ftrl_params_default(tn_ftrl_params* p);
+
+/* Optimizer objects are immortal and may be shared by several tables
+ * (core/main/py_wrapper.cc:112).  Handles are small ints starting at 0. */
+typedef int32_t tn_opt_t;
+
+/* core/main/py_wrapper.cc:82-116 (AdaGrad factory). elimination_logic must be 0 or 1. */
+int tn_opt_create_adagrad(const tn_adagrad_params* p, tn_opt_t* out);
+/* core/main/py_wrapper.cc:117-133 (Adam factory). */
+int tn_opt_create_adam(const tn_adam_params* p, tn_opt_t* out);
+/* core/main/py_wrapper.cc:146-162 (Ftrl factory). */
+int tn_opt_create_ftrl(const tn_ftrl_params* p, tn_opt_t* out);
+/* OptimizerBase::SetSparseZeroInit, core/ps/optimizer/optimizer.h:49
+ * (py: set_sparse_init_mode(opt, is_training) == set_sparse_zero_init(opt, !is_training)). */
+int tn_opt_set_sparse_zero_init(tn_opt_t opt, int zero_init);
+/* OptimizerBase::SetSchedule(float), core/ps/optimizer/optimizer.h:61. */
+int tn_opt_set_learning_rate(tn_opt_t opt, float lr);
+/* py get_opt_learning_rate, core/main/py_wrapper.cc:134-145 (constant schedule only). */
+int tn_opt_get_learning_rate(tn_opt_t opt, float* lr);
+
+/* ------------------------------------------------------------ sparse table */
+/*
+ * Record of one distinct sign of a push, byte-identical to
+ * SparsePushSignInfo (core/ps_interface/ps_raw_interface.h:22-35): 16 bytes.
+ */
+typedef struct tn_sign_info {
+    uint64_t sign;
+    int32_t batch_show;
+    int32_t batch_click;
+} tn_sign_info;
+
+/*
+ * CreateSparseTable (core/ps/table/sparse_table.cc:169-186) as called from
+ * create_sparse_table (core/main/py_wrapper.cc:169-181): a non-empty
+ * embedding_group that already exists returns the existing table's handle.
+ * use_cvm follows SetUseCvm (optimizer.h:51): rows of an AdaGrad table then
+ * carry two extra floats (show, log(click+1)-log(show+1)) after the weights
+ * and pull/push use dim = dimension + 2.
+ * The table lives in HBM as an open-addressing hash table on the current HIP
+ * device.  It is allocated on first use with room for
+ * tn_sparse_table_reserve()'s key count (default 8 x 15485863 slots, the
+ * reference's own no-rehash bucket count, optimizer_kernel.h:257-263) and
+ * grows by re-insertion when its load factor would pass 0.75
+ * (optimizer_kernel.h:266).
+ */
+int tn_sparse_table_create(tn_opt_t opt, const char* name, int dimension, int use_cvm, int shard_num,
+                           int self_shard_id, const char* embedding_group, uint32_t* handle);
+
+/* Size the HBM table for at least max_keys resident keys at load factor <= 0.75. */
+int tn_sparse_table_reserve(uint32_t handle, uint64_t max_keys);
+
+/* Seed of the on-device row initialiser (the reference seeds from the wall
+ * clock, core/utility/random.h:30-42; here new rows are a pure function of
+ * (seed, sign)). */
+int tn_sparse_table_set_seed(uint32_t handle, uint64_t seed);
+
+/* SparseOptimizerKernelBase::KeyCount, core/ps/optimizer/optimizer_kernel.h:540-547. */
+int tn_sparse_table_key_count(uint32_t handle, uint64_t* count);
+
+/* Number of HBM hash slots currently allocated (0 before first use). */
+int tn_sparse_table_capacity(uint32_t handle, uint64_t* slots);
+
+/* Floats per row: weights (dimension, +2 with cvm) and optimizer state.
+ * State layout (float words; integers stored bitwise):
+ *   AdaGrad: g2sum, show, click, no_show_days(int32)        (ada_grad_kernel.h:76-83)
+ *   Adam:    m[dim], v[dim], show, delta_show(int32)        (adam_kernel.h:72-86, data_struct.h:54-58)
+ *   Ftrl:    z[dim], n[dim], show, delta_show(int32)        (ftrl_kernel.h:73-88) */
+int tn_sparse_table_row_layout(uint32_t handle, int* weight_floats, int* state_floats);
+
+/*
+ * SparseTable::Pull (core/ps/table/sparse_table.cc:52-66): for each of the n
+ * device signs, in request order, look the row up -- inserting and
+ * initialising it if absent (optimizer_kernel.h:299-308) -- and write its
+ * `dim` floats to out[i*dim .. i*dim+dim) (device).  dim must equal the
+ * table's weight_floats.
+ */
+int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream);
+
+/*
+ * SparseTable::Push (core/ps/table/sparse_table.cc:68-83): apply n records
+ * (device infos[n], device grads[n*dim]) in ARRAY ORDER; a sign occurring k
+ * times gets k sequential optimizer Applies.  A sign that was never pulled is
+ * TN_ERR_UNKNOWN_KEY (that record is skipped, the others are applied).
+ */
+int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float* grads, int64_t n, int dim,
+                         void* stream);
+
+/*
+ * Snapshot injection / read-back: what the reference does through the mutable
+ * pointer returned by SparseOptimizerKernelBase::GetWeight
+ * (optimizer_kernel.h:84) and through bin Serialized/DeSerialized
+ * (optimizer_kernel.h:341-351,399-408).  All pointers are device memory.
+ * load_rows inserts (or overwrites) n rows; w is [n, weight_floats], state is
+ * [n, state_floats] or NULL for freshly-constructed state.
+ * export_rows writes the rows of n signs; found[i] = 0 and zeros for absent signs.
+ */
+int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const float* w, const float* state,
+                              int64_t n, void* stream);
+int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t n, float* w, float* state,
+                                uint8_t* found, void* stream);
+
+/*
+ * SparseTablePull op (core/ops/sparse_table_ops.cc:21-43, kernel
+ * core/kernels/sparse_table_ops.cc:170-265).  N slots; slot s has
+ * value_lens[s] int64 signs at device pointer values[s], a device variable
+ * vars[s] of shape [var_rows[s], var_dim] row-major, and a device output
+ * mapped_values[s] of value_lens[s] int64.  values/vars/mapped_values/
+ * value_lens/var_rows are HOST arrays of length N.
+ * Writes mapped_values[s][i] = rank of values[s][i]'s first occurrence among
+ * the distinct signs of slot s (sparse_table_ops.cc:122-131) and copies the
+ * pulled row of the j-th distinct sign into vars[s][j, :]; rows >= U_s are
+ * left untouched.  U_s >= var_rows[s] is TN_ERR_VAR_CAPACITY.
+ * The call returns after the stream work has completed (the reference op
+ * blocks on a semaphore, sparse_table_ops.cc:236).
+ */
+int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                            float* const* vars, const int64_t* var_rows, int var_dim,
+                            int64_t* const* mapped_values, void* stream);
+
+/*
+ * SparseTablePush op (core/ops/sparse_table_ops.cc:45-53, kernel
+ * core/kernels/sparse_table_ops.cc:317-368).  grads[s] is a device matrix
+ * [grad_rows[s], grad_dim] whose row j belongs to the j-th distinct sign of
+ * slot s; feature_labels[s] holds value_lens[s] int64 labels.  Per distinct
+ * sign batch_show = occurrences and batch_click = sum of labels
+ * (sparse_table_ops.cc:283-296); records are applied slot-major, so a sign
+ * present in k slots receives k sequential Applies, slot 0 first.
+ * Enqueues the update and returns without waiting, like the reference op
+ * (sparse_table_ops.cc:363-367); errors of the enqueued work are reported by
+ * the next synchronising call on the table or by tn_sparse_table_sync().
+ */
+int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                            const float* const* grads, const int64_t* grad_rows, int grad_dim,
+                            const int64_t* const* feature_labels, void* stream);
+
+/* Wait for the table's enqueued work and return (and clear) its latched error. */
+int tn_sparse_table_sync(uint32_t handle);
+
+/* U_s of the last pull_op / synchronised push_op on the table (host array of N). */
+int tn_sparse_table_last_unique_counts(uint32_t handle, int N, int64_t* counts);
+
+/* Keep pull_op from waiting on the stream (for callers that order work on the
+ * stream themselves); its errors are then latched like push_op's. */
+int tn_sparse_table_set_async(uint32_t handle, int async_pull);
+
+/* ------------------------------------------------------------- dense table */
+/* CreateDenseTable (core/ps/table/dense_table.cc:180-186); Adam or AdaGrad. */
+int tn_dense_table_create(tn_opt_t opt, int shard_num, int self_shard_id, uint32_t* handle);
+
+/*
+ * DenseTableInit op (core/kernels/dense_table_ops.cc:73-118): concatenates N
+ * device variables (var_lens[s] floats each, host arrays of length N) into
+ * the table: DenseTable::Init(total) + SetWeight (dense_table.cc:37-87).
+ * A second Init with a different total is TN_ERR_ALREADY_INIT.
+ */
+int tn_dense_table_init(uint32_t handle, int N, const float* const* vars, const int64_t* var_lens, void* stream);
+
+/*
+ * DenseTablePushPull op (core/kernels/dense_table_ops.cc:130-252): applies
+ * the concatenated gradient with this step's learning rate
+ * (DenseOptimizerKernel::Apply, optimizer_kernel.h:192-204 ->
+ * DenseAdamValue::Apply adam_kernel.cc:46-55 or DenseAdaGradValue::Apply
+ * ada_grad_kernel.cc:42-48) and writes the new weights back into the
+ * variables.  vars[s] may be NULL to skip the write-back of a variable.
+ */
+int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const float* const* grads,
+                             const int64_t* lens, float learning_rate, void* stream);
+
+/* DenseTable::TotalElements (core/ps/table/dense_table.h:44). */
+int tn_dense_table_total_elements(uint32_t handle, int64_t* total);
+
+/* DenseOptimizerKernelBase::GetWeight / SetWeight (optimizer_kernel.h:63-65)
+ * over the whole single-worker range; device pointers of total floats. */
+int tn_dense_table_get_weight(uint32_t handle, float* w, void* stream);
+int tn_dense_table_set_weight(uint32_t handle, const float* w, void* stream);
+/* Optimizer state read-back for tests: Adam m,v ; AdaGrad d2sum,g2sum,m (device, total floats each; NULL skips). */
+int tn_dense_table_get_state(uint32_t handle, float* s0, float* s1, float* s2, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENSORNET_AMD_H_ */

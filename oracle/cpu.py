@@ -1,0 +1,231 @@
+"""ctypes front end of oracle/liboracle.so (see oracle/oracle.cc).
+
+TEST INFRASTRUCTURE: the checker the HIP path is compared with, and the timed
+CPU baseline of bench.py.  Works on numpy arrays.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+ADAGRAD, ADAM, FTRL = 0, 1, 2
+
+sign_info_dtype = np.dtype([("sign", "<u8"), ("batch_show", "<i4"), ("batch_click", "<i4")])
+
+_lib = None
+
+
+def build():
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        build()
+    lib = C.CDLL(LIB_PATH)
+    P = C.c_void_p
+    lib.orc_table_create.restype = P
+    lib.orc_table_create.argtypes = [C.c_int, P, C.c_int, C.c_int, C.c_int, C.c_uint64, C.c_uint64]
+    lib.orc_table_destroy.argtypes = [P]
+    lib.orc_table_weight_floats.argtypes = [P]
+    lib.orc_table_state_floats.argtypes = [P]
+    lib.orc_table_key_count.restype = C.c_uint64
+    lib.orc_table_key_count.argtypes = [P]
+    lib.orc_table_set_rows.argtypes = [P, P, P, P, C.c_int64]
+    lib.orc_table_get_rows.argtypes = [P, P, C.c_int64, P, P, P]
+    lib.orc_table_pull.argtypes = [P, P, C.c_int64, C.c_int, P]
+    lib.orc_table_push.argtypes = [P, P, P, C.c_int64, C.c_int]
+    lib.orc_pull_remap.restype = C.c_int64
+    lib.orc_pull_remap.argtypes = [P, C.c_int64, P, P]
+    lib.orc_push_remap.restype = C.c_int64
+    lib.orc_push_remap.argtypes = [P, P, C.c_int64, P]
+    lib.orc_pull_op.argtypes = [P, C.c_int, P, P, P, P, C.c_int, P, P]
+    lib.orc_push_op.argtypes = [P, C.c_int, P, P, P, C.c_int, P, P]
+    lib.orc_dense_create.restype = P
+    lib.orc_dense_create.argtypes = [C.c_int, P, C.c_int64]
+    lib.orc_dense_destroy.argtypes = [P]
+    lib.orc_dense_set_weight.argtypes = [P, P]
+    lib.orc_dense_get_weight.argtypes = [P, P]
+    lib.orc_dense_apply.argtypes = [P, P, C.c_float]
+    lib.orc_dense_num_blocks.argtypes = [P]
+    lib.orc_dense_get_state.argtypes = [P, C.c_int, P]
+    _lib = lib
+    return lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _ptrs(arrays):
+    arr = (C.c_void_p * len(arrays))()
+    for i, a in enumerate(arrays):
+        arr[i] = a.ctypes.data
+    return arr
+
+
+def _params(kind, **kw):
+    """Packs hyper-parameters in the order oracle.cc's FillOpt reads them."""
+    if kind == ADAGRAD:
+        vals = [
+            kw.get("learning_rate", 0.01),
+            kw.get("initial_g2sum", 0.0),
+            kw.get("initial_scale", 1.0),
+            kw.get("epsilon", 1e-8),
+            kw.get("grad_decay_rate", 1.0),
+            kw.get("mom_decay_rate", 1.0),
+        ]
+    elif kind == ADAM:
+        vals = [
+            kw.get("learning_rate", 0.01),
+            kw.get("beta1", 0.9),
+            kw.get("beta2", 0.999),
+            kw.get("epsilon", 1e-8),
+            kw.get("initial_scale", 1.0),
+        ]
+    else:
+        vals = [
+            kw.get("learning_rate", 0.01),
+            kw.get("beta", 1.0),
+            kw.get("lambda1", 0.1),
+            kw.get("lambda2", 1.0),
+            kw.get("initial_scale", 1.0),
+        ]
+    return np.asarray(vals + [0.0] * (8 - len(vals)), dtype=np.float32)
+
+
+def pull_remap(values):
+    """SparsePullVarInfo: (mapped ids int64[L], distinct signs uint64[U])."""
+    values = np.ascontiguousarray(values, dtype=np.int64)
+    mapped = np.empty_like(values)
+    signs = np.empty(values.shape[0], dtype=np.uint64)
+    u = load().orc_pull_remap(_p(values), values.shape[0], _p(mapped), _p(signs))
+    return mapped, signs[:u].copy()
+
+
+def push_remap(values, labels):
+    """SparsePushVarInfo: structured array (sign, batch_show, batch_click)[U]."""
+    values = np.ascontiguousarray(values, dtype=np.int64)
+    labels = np.ascontiguousarray(labels, dtype=np.int64)
+    infos = np.empty(values.shape[0], dtype=sign_info_dtype)
+    u = load().orc_push_remap(_p(values), _p(labels), values.shape[0], _p(infos))
+    return infos[:u].copy()
+
+
+class Table(object):
+    """One SparseTable of the reference with its 8-block optimizer kernel."""
+
+    def __init__(self, kind, dim, use_cvm=False, zero_init=False, seed=1, buckets=15485863, **hyper):
+        self.kind = kind
+        self.dim = dim
+        self._params = _params(kind, **hyper)
+        self._h = load().orc_table_create(
+            kind, _p(self._params), dim, int(use_cvm), int(zero_init), seed, buckets
+        )
+        self.wf = load().orc_table_weight_floats(self._h)
+        self.sf = load().orc_table_state_floats(self._h)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            load().orc_table_destroy(self._h)
+            self._h = None
+
+    def key_count(self):
+        return int(load().orc_table_key_count(self._h))
+
+    def set_rows(self, signs, w, state=None):
+        signs = np.ascontiguousarray(signs, dtype=np.uint64)
+        w = np.ascontiguousarray(w, dtype=np.float32).reshape(len(signs), self.wf)
+        if state is not None:
+            state = np.ascontiguousarray(state, dtype=np.float32).reshape(len(signs), self.sf)
+        load().orc_table_set_rows(self._h, _p(signs), _p(w), _p(state), len(signs))
+
+    def get_rows(self, signs):
+        signs = np.ascontiguousarray(signs, dtype=np.uint64)
+        w = np.zeros((len(signs), self.wf), dtype=np.float32)
+        st = np.zeros((len(signs), self.sf), dtype=np.float32)
+        found = np.zeros(len(signs), dtype=np.uint8)
+        load().orc_table_get_rows(self._h, _p(signs), len(signs), _p(w), _p(st), _p(found))
+        return w, st, found
+
+    def pull(self, signs, dim=None):
+        signs = np.ascontiguousarray(signs, dtype=np.uint64)
+        dim = self.wf if dim is None else dim
+        out = np.empty((len(signs), dim), dtype=np.float32)
+        load().orc_table_pull(self._h, _p(signs), len(signs), dim, _p(out))
+        return out
+
+    def push(self, infos, grads):
+        infos = np.ascontiguousarray(infos, dtype=sign_info_dtype)
+        grads = np.ascontiguousarray(grads, dtype=np.float32)
+        return load().orc_table_push(self._h, _p(infos), _p(grads), len(infos), grads.shape[1])
+
+    def pull_op(self, values, vars):
+        """values: list of int64 arrays; vars: list of float32 [rows, dim] arrays (written
+        in place).  Returns (status, mapped list, distinct counts)."""
+        n = len(values)
+        values = [np.ascontiguousarray(v, dtype=np.int64) for v in values]
+        mapped = [np.empty_like(v) for v in values]
+        lens = np.asarray([len(v) for v in values], dtype=np.int64)
+        rows = np.asarray([v.shape[0] for v in vars], dtype=np.int64)
+        counts = np.zeros(n, dtype=np.int64)
+        rc = load().orc_pull_op(
+            self._h, n, _ptrs(values), _p(lens), _ptrs(vars), _p(rows), vars[0].shape[1], _ptrs(mapped), _p(counts)
+        )
+        return rc, mapped, counts
+
+    def push_op(self, values, grads, labels):
+        n = len(values)
+        values = [np.ascontiguousarray(v, dtype=np.int64) for v in values]
+        labels = [np.ascontiguousarray(l, dtype=np.int64) for l in labels]
+        grads = [np.ascontiguousarray(g, dtype=np.float32) for g in grads]
+        lens = np.asarray([len(v) for v in values], dtype=np.int64)
+        counts = np.zeros(n, dtype=np.int64)
+        rc = load().orc_push_op(
+            self._h, n, _ptrs(values), _p(lens), _ptrs(grads), grads[0].shape[1], _ptrs(labels), _p(counts)
+        )
+        return rc, counts
+
+
+class Dense(object):
+    """DenseTable of one worker: 8 optimizer blocks over a flat array."""
+
+    def __init__(self, kind, total, **hyper):
+        self.total = total
+        self._params = _params(kind, **hyper)
+        self._h = load().orc_dense_create(kind, _p(self._params), total)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            load().orc_dense_destroy(self._h)
+            self._h = None
+
+    def num_blocks(self):
+        return load().orc_dense_num_blocks(self._h)
+
+    def set_weight(self, w):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        assert w.size == self.total
+        load().orc_dense_set_weight(self._h, _p(w))
+
+    def get_weight(self):
+        w = np.empty(self.total, dtype=np.float32)
+        load().orc_dense_get_weight(self._h, _p(w))
+        return w
+
+    def apply(self, grad, lr):
+        grad = np.ascontiguousarray(grad, dtype=np.float32)
+        assert grad.size == self.total
+        load().orc_dense_apply(self._h, _p(grad), lr)
+
+    def get_state(self, which):
+        out = np.zeros(self.total, dtype=np.float32)
+        load().orc_dense_get_state(self._h, which, _p(out))
+        return out

@@ -1,0 +1,134 @@
+"""Configuration surface of the hot path, mirroring the reference's
+`tensornet.core` (pybind module `_pywrap_tn`, core/main/py_wrapper.cc:61-263):
+optimizer factories taking keyword arguments with the reference's names and
+defaults, and table factories returning integer handles.
+"""
+import ctypes as C
+
+from . import _lib
+
+
+class _Opt(object):
+    """Opaque optimizer object (the reference returns a PyCapsule)."""
+
+    def __init__(self, handle, name):
+        self.handle = handle
+        self.name = name
+
+    def __repr__(self):
+        return "<tensornet_amd %s optimizer #%d>" % (self.name, self.handle)
+
+
+def _fill(params, kwargs, allowed):
+    for key, value in kwargs.items():
+        if key not in allowed:
+            # PYDICT_PARSE_KWARGS ignores unknown names (py_wrapper.cc:38-45)
+            continue
+        if key in ("no_show_days", "elimination_logic"):
+            setattr(params, key, int(value))
+        else:
+            setattr(params, key, float(value))
+
+
+def AdaGrad(**kwargs):
+    """py_wrapper.cc:82-116.  learning_rate must be a float here (schedules
+    are only evaluated for the dense path in the reference)."""
+    lib = _lib.load()
+    p = _lib.AdaGradParams()
+    lib.tn_adagrad_params_default(C.byref(p))
+    _fill(p, kwargs, [f for f, _ in _lib.AdaGradParams._fields_])
+    if p.elimination_logic not in (0, 1):
+        raise ValueError(
+            "elimination_logic must be in the set of valid values {0, 1}, but got: %d" % p.elimination_logic
+        )
+    h = C.c_int32()
+    _lib.check(lib.tn_opt_create_adagrad(C.byref(p), C.byref(h)))
+    return _Opt(h.value, "AdaGrad")
+
+
+def Adam(**kwargs):
+    """py_wrapper.cc:117-133."""
+    lib = _lib.load()
+    p = _lib.AdamParams()
+    lib.tn_adam_params_default(C.byref(p))
+    _fill(p, kwargs, [f for f, _ in _lib.AdamParams._fields_])
+    h = C.c_int32()
+    _lib.check(lib.tn_opt_create_adam(C.byref(p), C.byref(h)))
+    return _Opt(h.value, "Adam")
+
+
+def Ftrl(**kwargs):
+    """py_wrapper.cc:146-162."""
+    lib = _lib.load()
+    p = _lib.FtrlParams()
+    lib.tn_ftrl_params_default(C.byref(p))
+    _fill(p, kwargs, [f for f, _ in _lib.FtrlParams._fields_])
+    h = C.c_int32()
+    _lib.check(lib.tn_opt_create_ftrl(C.byref(p), C.byref(h)))
+    return _Opt(h.value, "Ftrl")
+
+
+def get_opt_learning_rate(opt):
+    """py_wrapper.cc:134-145 (constant learning rate)."""
+    lr = C.c_float()
+    _lib.check(_lib.load().tn_opt_get_learning_rate(opt.handle, C.byref(lr)))
+    return lr.value
+
+
+def set_sparse_init_mode(opt, is_training):
+    """py_wrapper.cc:163-168: zero-initialise new rows when not training."""
+    _lib.check(_lib.load().tn_opt_set_sparse_zero_init(opt.handle, 0 if is_training else 1))
+
+
+def create_sparse_table(opt, name, dimension, use_cvm=False, embedding_group=""):
+    """py_wrapper.cc:169-181 -> CreateSparseTable (sparse_table.cc:169-186)."""
+    h = C.c_uint32()
+    _lib.check(
+        _lib.load().tn_sparse_table_create(
+            opt.handle,
+            (name or "").encode(),
+            int(dimension),
+            1 if use_cvm else 0,
+            1,
+            0,
+            (embedding_group or "").encode(),
+            C.byref(h),
+        )
+    )
+    return h.value
+
+
+def create_dense_table(opt):
+    """py_wrapper.cc:182-191 -> CreateDenseTable (dense_table.cc:180-186)."""
+    h = C.c_uint32()
+    _lib.check(_lib.load().tn_dense_table_create(opt.handle, 1, 0, C.byref(h)))
+    return h.value
+
+
+def reserve_sparse_table(table_handle, max_keys):
+    """Sizes the HBM hash table for max_keys resident signs (no counterpart in
+    the reference, whose host hash maps grow by themselves)."""
+    _lib.check(_lib.load().tn_sparse_table_reserve(table_handle, int(max_keys)))
+
+
+def set_sparse_table_seed(table_handle, seed):
+    _lib.check(_lib.load().tn_sparse_table_set_seed(table_handle, int(seed) & 0xFFFFFFFFFFFFFFFF))
+
+
+def sparse_table_key_count(table_handle):
+    n = C.c_uint64()
+    _lib.check(_lib.load().tn_sparse_table_key_count(table_handle, C.byref(n)))
+    return n.value
+
+
+def sparse_table_capacity(table_handle):
+    n = C.c_uint64()
+    _lib.check(_lib.load().tn_sparse_table_capacity(table_handle, C.byref(n)))
+    return n.value
+
+
+def sparse_table_row_layout(table_handle):
+    w = C.c_int()
+    s = C.c_int()
+    _lib.check(_lib.load().tn_sparse_table_row_layout(table_handle, C.byref(w), C.byref(s)))
+    return w.value, s.value

@@ -1,0 +1,890 @@
+// Device code of the sparse pull / push path.  Included by sparse_table.hip only.
+//
+// HBM layout of one table (structure of arrays, all indexed by the slot number
+// of an open-addressing hash table with linear probing):
+//     keys[cap + 1]              uint64 sign, EMPTY_KEY where free
+//     w   [cap + 1][wstride]     embedding weights (+2 cvm columns)
+//     st  [cap + 1][sstride]     optimizer state
+// Slot `cap` is reserved for the one sign whose value equals EMPTY_KEY.
+// A pull touches keys and w only (one 64-byte granule each for dim 16); the
+// optimizer state is touched by push alone.
+//
+// Per-call scratch (all sized by the number of lookups L of the call):
+//     dedup table   per slot of the op, open addressing over the slot's signs,
+//                   entry {sign, position of first occurrence, rank}
+//     group table   open addressing over the distinct signs of all slots of a
+//                   push, entry {sign, count, list offset}
+// Both are filled with 0xFF bytes before use, which is EMPTY_KEY / "no
+// position yet" / "count -1" at once.
+#ifndef TN_SPARSE_KERNELS_H_
+#define TN_SPARSE_KERNELS_H_
+
+#include "tn_common.h"
+
+namespace tn {
+
+struct Store {
+    uint64_t cap;
+    uint64_t* keys;
+    float* w;
+    float* st;
+    uint32_t* special;            // 1 when the sign EMPTY_KEY itself is resident
+    unsigned long long* count;    // resident keys
+    int D, wdim, wstride, sstride;
+};
+
+// One slot (input tensor pair) of a pull / push op.  64 bytes.
+struct SlotDesc {
+    const int64_t* values;
+    int64_t* mapped;        // pull
+    const int64_t* labels;  // push
+    float* var;             // pull
+    const float* grads;     // push
+    int64_t rows;           // rows of var (pull) / of grads (push)
+    uint32_t len;
+    uint32_t lbase;         // first lookup of the slot in the concatenated order
+    uint32_t tbase;         // first entry of the slot's dedup table
+    uint32_t tcap;          // entries of the slot's dedup table (+1 special)
+};
+
+struct DedupEntry {
+    uint64_t key;
+    uint32_t minpos;  // smallest in-slot position of the sign
+    uint32_t rank;    // index of the sign in the compact distinct list of the call
+};
+
+struct GroupEntry {
+    uint64_t key;
+    uint32_t cnt;  // occurrences - 1 (starts at 0xFFFFFFFF)
+    uint32_t off;  // start of the group's member list
+};
+
+constexpr int REMAP_ITEMS = 8;
+constexpr int REMAP_THREADS = 256;
+constexpr int REMAP_TILE = REMAP_ITEMS * REMAP_THREADS;
+constexpr int MAX_SLOTS = 4096;
+
+__device__ __forceinline__ unsigned long long* ull(uint64_t* p) { return reinterpret_cast<unsigned long long*>(p); }
+
+// Hands out consecutive indices from *counter to the lanes whose flag is set,
+// with one atomic per wavefront.
+__device__ __forceinline__ uint32_t wave_alloc(bool flag, uint32_t* counter) {
+    unsigned long long mask = __ballot(flag);
+    if (mask == 0) return 0;
+    int leader = __ffsll((long long)mask) - 1;
+    int lane = (int)__lane_id();
+    uint32_t base = 0;
+    if (lane == leader) base = atomicAdd(counter, (uint32_t)__popcll(mask));
+    base = __shfl(base, leader);
+    return base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+}
+
+// ------------------------------------------------------------------ fills
+__global__ __launch_bounds__(256) void k_fill_ff(uint4* p, size_t n16) {
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4 v = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) p[i] = v;
+}
+
+// fills the first (status->gcap + 1) group entries
+__global__ __launch_bounds__(256) void k_fill_groups(GroupEntry* gt, const DevStatus* status) {
+    size_t n16 = (size_t)status->gcap + 1;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4 v = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+    uint4* p = reinterpret_cast<uint4*>(gt);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) p[i] = v;
+}
+
+__global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gcap) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        status->err = 0;
+        status->n_unique = n_unique;
+        status->n_groups = 0;
+        status->n_new = 0;
+        status->gcap = gcap;
+        status->list_cursor = 0;
+    }
+}
+
+__global__ void k_finish_insert(Store s, const DevStatus* status) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *s.count += status->n_new;
+}
+
+// ------------------------------------------------------- table probe/insert
+// One thread per sign.  rows[i] = slot of signs[i] (NO_ROW if absent / full).
+// With INSERT an absent sign claims the first free slot of its probe sequence
+// (SparseKernelBlock::GetWeight's insert, optimizer_kernel.h:299-308) and the
+// index i of every claim is appended to newlist.
+template <bool INSERT>
+__global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restrict__ signs, int64_t n_host,
+                                               const uint32_t* n_dev, uint32_t* __restrict__ rows,
+                                               uint32_t* __restrict__ newlist, DevStatus* status, uint32_t miss_err) {
+    const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint64_t sign = signs[i];
+        uint32_t row = NO_ROW;
+        bool is_new = false;
+        if (sign == EMPTY_KEY) {
+            if (INSERT) {
+                is_new = atomicCAS(s.special, 0u, 1u) == 0u;
+                row = (uint32_t)s.cap;
+            } else if (ld_relaxed(s.special)) {
+                row = (uint32_t)s.cap;
+            }
+        } else {
+            uint64_t idx = slot_of(sign, s.cap);
+            for (uint64_t p = 0; p < s.cap; ++p) {
+                uint64_t k = ld_relaxed(&s.keys[idx]);
+                if (k == sign) {
+                    row = (uint32_t)idx;
+                    break;
+                }
+                if (k == EMPTY_KEY) {
+                    if (!INSERT) break;
+                    uint64_t old = atomicCAS(ull(&s.keys[idx]), EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY) {
+                        row = (uint32_t)idx;
+                        is_new = true;
+                        break;
+                    }
+                    if (old == sign) {
+                        row = (uint32_t)idx;
+                        break;
+                    }
+                }
+                idx = (idx + 1 == s.cap) ? 0 : idx + 1;
+            }
+        }
+        rows[i] = row;
+        if (row == NO_ROW && miss_err) atomicOr(&status->err, miss_err);
+        if (INSERT) {
+            uint32_t j = wave_alloc(is_new, &status->n_new);
+            if (is_new) newlist[j] = (uint32_t)i;
+        }
+    }
+}
+
+// ---------------------------------------------------------- row initialiser
+__device__ __forceinline__ uint64_t rnd64(uint64_t seed, uint64_t sign, uint64_t ctr) {
+    return mix64(mix64(sign ^ seed) + (ctr + 1) * 0x9E3779B97F4A7C15ull);
+}
+
+// Two independent N(0,1) draws from 64 random bits (Box-Muller).
+__device__ __forceinline__ float2 normal_pair(uint64_t bits) {
+    float u1 = ((float)(uint32_t)(bits >> 32) + 1.0f) * 2.3283064365386963e-10f;  // (0, 1]
+    float u2 = (float)(uint32_t)bits * 2.3283064365386963e-10f;                   // [0, 1)
+    float r = sqrtf(-2.0f * logf(u1));
+    float sn, cs;
+    sincosf(6.283185307179586f * u2, &sn, &cs);
+    return make_float2(r * cs, r * sn);
+}
+
+__device__ __forceinline__ void init_state(const Store& s, const OptDev& o, float* st) {
+    if (o.kind == OPT_ADAGRAD) {
+        st[0] = o.initial_g2sum;  // ada_grad_kernel.cc:94-98
+        st[1] = 0.f;
+        st[2] = 0.f;
+        st[3] = 0.f;  // no_show_days = 0 (int bits)
+    } else {
+        for (int i = 0; i < s.sstride; i++) st[i] = 0.f;  // m=v=0 / z=n=0, show, delta_show
+    }
+}
+
+// New rows: w[i] = N(0, 1/sqrt(D)) * initial_scale, or zeros under
+// sparse_zero_init; fresh optimizer state (ada_grad_kernel.cc:78-103,
+// adam_kernel.cc:89-110, ftrl_kernel.cc:34-55).  The draw is a pure function
+// of (seed, sign, element).  One thread per new row.
+__global__ __launch_bounds__(256) void k_init_rows(Store s, OptDev o, uint64_t seed, const uint64_t* __restrict__ signs,
+                                                   const uint32_t* __restrict__ rows,
+                                                   const uint32_t* __restrict__ newlist, const DevStatus* status) {
+    const uint32_t n_new = status->n_new;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    const float stddev = (float)(1.0 / sqrt((double)s.D));
+    for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < n_new; j += stride) {
+        const uint32_t i = newlist[j];
+        const uint64_t sign = signs[i];
+        const uint64_t row = rows[i];
+        float* w = s.w + row * s.wstride;
+        if (o.zero_init) {
+            for (int c = 0; c < s.D; c++) w[c] = 0.f;
+        } else {
+            for (int c = 0; c < s.D; c += 2) {
+                float2 z = normal_pair(rnd64(seed, sign, (uint64_t)(c >> 1)));
+                w[c] = (z.x * stddev) * o.initial_scale;
+                if (c + 1 < s.D) w[c + 1] = (z.y * stddev) * o.initial_scale;
+            }
+        }
+        for (int c = s.D; c < s.wstride; c++) w[c] = 0.f;  // cvm columns / padding
+        init_state(s, o, s.st + row * s.sstride);
+    }
+}
+
+// ------------------------------------------------------------------ gathers
+// out[i, :] = w[rows[i], 0:wdim]   (SparseTable::Pull's append, sparse_table.cc:64)
+template <int VEC>
+__global__ __launch_bounds__(256) void k_gather_rows(Store s, const uint32_t* __restrict__ rows, int64_t n,
+                                                     float* __restrict__ out) {
+    const int chunks = s.wdim / VEC;
+    const int64_t total = n * chunks;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int64_t i = t / chunks;
+        const int c = (int)(t - i * chunks);
+        const uint32_t row = rows[i];
+        if (VEC == 4) {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row != NO_ROW) v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
+            *reinterpret_cast<float4*>(out + i * s.wdim + c * 4) = v;
+        } else {
+            out[i * s.wdim + c] = (row != NO_ROW) ? s.w[(uint64_t)row * s.wstride + c] : 0.f;
+        }
+    }
+}
+
+// vars[slot][rank, :] = w[rows[u], :] for every distinct sign u of the op
+// (PopulatePulledVariable_, sparse_table_ops.cc:244-265).
+template <int VEC>
+__global__ __launch_bounds__(256) void k_gather_vars(Store s, const uint32_t* __restrict__ rows,
+                                                     const uint32_t* __restrict__ uniq_slot,
+                                                     const uint32_t* __restrict__ ubase,
+                                                     const SlotDesc* __restrict__ descs, DevStatus* status) {
+    const int chunks = s.wdim / VEC;
+    const int64_t total = (int64_t)status->n_unique * chunks;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int64_t u = t / chunks;
+        const int c = (int)(t - u * chunks);
+        const uint32_t row = rows[u];
+        const uint32_t sl = uniq_slot[u];
+        const int64_t r = (int64_t)u - (int64_t)ubase[sl];
+        const SlotDesc& d = descs[sl];
+        if (r >= d.rows) {
+            if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
+            continue;
+        }
+        if (row == NO_ROW) continue;
+        if (VEC == 4) {
+            float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
+            *reinterpret_cast<float4*>(d.var + r * s.wdim + c * 4) = v;
+        } else {
+            d.var[r * s.wdim + c] = s.w[(uint64_t)row * s.wstride + c];
+        }
+    }
+}
+
+// Snapshot load: table row <- caller row (+ given or fresh state).
+__global__ __launch_bounds__(256) void k_load_rows(Store s, OptDev o, const uint32_t* __restrict__ rows, int64_t n,
+                                                   const float* __restrict__ w, const float* __restrict__ state) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint32_t row = rows[i];
+        if (row == NO_ROW) continue;
+        float* dw = s.w + (uint64_t)row * s.wstride;
+        for (int c = 0; c < s.wdim; c++) dw[c] = w[i * s.wdim + c];
+        for (int c = s.wdim; c < s.wstride; c++) dw[c] = 0.f;
+        float* ds = s.st + (uint64_t)row * s.sstride;
+        if (state) {
+            const int sf = (o.kind == OPT_ADAGRAD) ? 4 : 2 * s.D + 2;
+            for (int c = 0; c < sf; c++) ds[c] = state[i * sf + c];
+            for (int c = sf; c < s.sstride; c++) ds[c] = 0.f;
+        } else {
+            init_state(s, o, ds);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void k_export_rows(Store s, OptDev o, const uint32_t* __restrict__ rows, int64_t n,
+                                                     float* __restrict__ w, float* __restrict__ state,
+                                                     uint8_t* __restrict__ found) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int sf = (o.kind == OPT_ADAGRAD) ? 4 : 2 * s.D + 2;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint32_t row = rows[i];
+        if (found) found[i] = row != NO_ROW;
+        const float* sw = s.w + (uint64_t)row * s.wstride;
+        const float* ss = s.st + (uint64_t)row * s.sstride;
+        if (w)
+            for (int c = 0; c < s.wdim; c++) w[i * s.wdim + c] = (row != NO_ROW) ? sw[c] : 0.f;
+        if (state)
+            for (int c = 0; c < sf; c++) state[i * sf + c] = (row != NO_ROW) ? ss[c] : 0.f;
+    }
+}
+
+// Re-insertion of every resident row into a larger table.
+__global__ __launch_bounds__(256) void k_rehash(Store from, Store to, DevStatus* status) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i <= from.cap; i += stride) {
+        uint64_t dst;
+        if (i == from.cap) {
+            if (*from.special == 0) continue;
+            *to.special = 1;
+            dst = to.cap;
+        } else {
+            const uint64_t sign = from.keys[i];
+            if (sign == EMPTY_KEY) continue;
+            uint64_t idx = slot_of(sign, to.cap);
+            dst = EMPTY_KEY;
+            for (uint64_t p = 0; p < to.cap; ++p) {
+                uint64_t old = atomicCAS(ull(&to.keys[idx]), EMPTY_KEY, sign);
+                if (old == EMPTY_KEY) {
+                    dst = idx;
+                    break;
+                }
+                idx = (idx + 1 == to.cap) ? 0 : idx + 1;
+            }
+            if (dst == EMPTY_KEY) {
+                atomicOr(&status->err, DEV_ERR_TABLE_FULL);
+                continue;
+            }
+        }
+        const float* sw = from.w + i * from.wstride;
+        float* dw = to.w + dst * to.wstride;
+        for (int c = 0; c < from.wstride; c++) dw[c] = sw[c];
+        const float* ss = from.st + i * from.sstride;
+        float* ds = to.st + dst * to.sstride;
+        for (int c = 0; c < from.sstride; c++) ds[c] = ss[c];
+    }
+}
+
+// -------------------------------------------------------------------- remap
+// Slot of a lookup: last s with lbase[s] <= gi (lbase[N] = L), skipping empty slots.
+__device__ __forceinline__ int find_slot(const uint32_t* lb, int N, uint32_t gi) {
+    int lo = 0, hi = N;  // invariant: lb[lo] <= gi < lb[hi]
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (lb[mid] <= gi)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ void load_lbase(uint32_t* sh, const uint32_t* lbase, int N) {
+    for (int i = threadIdx.x; i <= N; i += blockDim.x) sh[i] = lbase[i];
+    __syncthreads();
+}
+
+// Step 1: every lookup finds or claims the entry of its sign in its slot's
+// dedup table, remembers the entry (tidx) and lowers the entry's minpos to its
+// own in-slot position.  After the kernel, minpos is the position of the
+// sign's first occurrence: exactly the lookup on which the reference's
+// std::map insert succeeds (sparse_table_ops.cc:122-131).
+__global__ __launch_bounds__(256) void k_remap_insert(const SlotDesc* __restrict__ descs,
+                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                      DedupEntry* dt, uint32_t* __restrict__ tidx) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        const int sl = find_slot(lb, N, gi);
+        const SlotDesc& d = descs[sl];
+        const uint32_t li = gi - lb[sl];
+        const uint64_t sign = (uint64_t)d.values[li];
+        const uint32_t tbase = d.tbase, tcap = d.tcap;
+        uint32_t e;
+        if (sign == EMPTY_KEY) {
+            e = tbase + tcap;
+        } else {
+            uint32_t idx = (uint32_t)slot_of(sign, tcap);
+            for (;;) {
+                e = tbase + idx;
+                uint64_t k = ld_relaxed(&dt[e].key);
+                if (k == sign) break;
+                if (k == EMPTY_KEY) {
+                    uint64_t old = atomicCAS(ull(&dt[e].key), EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                }
+                idx = (idx + 1 == tcap) ? 0 : idx + 1;
+            }
+        }
+        tidx[gi] = e;
+        if (ld_relaxed(&dt[e].minpos) > li) atomicMin(&dt[e].minpos, li);
+    }
+}
+
+__device__ __forceinline__ uint32_t block_sum_256(uint32_t v, uint32_t* sh /*4*/) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) sh[wave] = v;
+    __syncthreads();
+    uint32_t t = sh[0] + sh[1] + sh[2] + sh[3];
+    __syncthreads();
+    return t;
+}
+
+// exclusive prefix of v over the 256 threads of the block
+__device__ __forceinline__ uint32_t block_excl_scan_256(uint32_t v, uint32_t* sh /*4*/) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+    for (int o = 1; o < 64; o <<= 1) {
+        uint32_t t = __shfl_up(inc, o);
+        if (lane >= o) inc += t;
+    }
+    if (lane == 63) sh[wave] = inc;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int wv = 0; wv < wave; wv++) base += sh[wv];
+    __syncthreads();
+    return base + inc - v;
+}
+
+// Step 2: a lookup is a first occurrence iff its position equals its entry's
+// minpos.  One flag bit per lookup (8 per thread), one count per tile.
+__global__ __launch_bounds__(REMAP_THREADS) void k_flag_count(const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                              const DedupEntry* __restrict__ dt,
+                                                              const uint32_t* __restrict__ tidx,
+                                                              uint8_t* __restrict__ flag8,
+                                                              uint32_t* __restrict__ tilesum) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t red[4];
+    load_lbase(lb, lbase, N);
+    const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
+    uint32_t bits = 0;
+    if (base < L) {
+        int sl = find_slot(lb, N, base);
+        for (int j = 0; j < REMAP_ITEMS; j++) {
+            const uint32_t gi = base + j;
+            if (gi >= L) break;
+            while (gi >= lb[sl + 1]) sl++;
+            const uint32_t li = gi - lb[sl];
+            if (dt[tidx[gi]].minpos == li) bits |= 1u << j;
+        }
+        flag8[base / REMAP_ITEMS] = (uint8_t)bits;
+    }
+    uint32_t total = block_sum_256(__popc(bits), red);
+    if (threadIdx.x == 0) tilesum[blockIdx.x] = total;
+}
+
+// Step 3 (one workgroup): exclusive scan of the tile counts; total distinct
+// count U; size of the push's group table; ubase of trailing empty slots.
+__global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict__ tilesum,
+                                                     uint32_t* __restrict__ tileoff, uint32_t ntiles,
+                                                     const uint32_t* __restrict__ lbase, uint32_t* __restrict__ ubase,
+                                                     int N, uint32_t L, DevStatus* status) {
+    __shared__ uint32_t wsum[16];
+    __shared__ uint32_t carry_sh;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) carry_sh = 0;
+    __syncthreads();
+    for (uint32_t start = 0; start < ntiles; start += 1024) {
+        const uint32_t i = start + threadIdx.x;
+        const uint32_t v = (i < ntiles) ? tilesum[i] : 0;
+        uint32_t inc = v;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t t = __shfl_up(inc, o);
+            if (lane >= o) inc += t;
+        }
+        if (lane == 63) wsum[wave] = inc;
+        __syncthreads();
+        uint32_t base = carry_sh;
+        for (int wv = 0; wv < wave; wv++) base += wsum[wv];
+        if (i < ntiles) tileoff[i] = base + inc - v;
+        __syncthreads();
+        if (threadIdx.x == 1023) carry_sh = base + inc;
+        __syncthreads();
+    }
+    const uint32_t U = carry_sh;
+    if (threadIdx.x == 0) {
+        status->n_unique = U;
+        uint32_t g = 2 * U;
+        status->gcap = g < 16 ? 16 : g;
+    }
+    for (int sl = threadIdx.x; sl <= N; sl += blockDim.x)
+        if (lbase[sl] >= L) ubase[sl] = U;
+}
+
+// Step 4: rank of every first occurrence = number of first occurrences before
+// it in the concatenated order; the compact lists of distinct signs follow.
+__global__ __launch_bounds__(REMAP_THREADS) void k_assign_rank(
+    const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L, DedupEntry* dt,
+    const uint32_t* __restrict__ tidx, const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff,
+    uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign, uint32_t* __restrict__ uniq_slot,
+    int32_t* __restrict__ ushow, int32_t* __restrict__ uclick) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t red[4];
+    load_lbase(lb, lbase, N);
+    const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
+    uint32_t bits = 0;
+    if (base < L) bits = flag8[base / REMAP_ITEMS];
+    uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256(__popc(bits), red);
+    if (base >= L) return;
+    int sl = find_slot(lb, N, base);
+    for (int j = 0; j < REMAP_ITEMS; j++) {
+        const uint32_t gi = base + j;
+        if (gi >= L) break;
+        while (gi >= lb[sl + 1]) sl++;
+        if (gi == lb[sl]) {
+            // first lookup of slot sl: u distinct signs precede it; empty slots just before share the value
+            ubase[sl] = u;
+            for (int e = sl - 1; e >= 0 && lb[e] == gi; e--) ubase[e] = u;
+        }
+        if (bits & (1u << j)) {
+            const SlotDesc& d = descs[sl];
+            dt[tidx[gi]].rank = u;
+            uniq_sign[u] = (uint64_t)d.values[gi - lb[sl]];
+            uniq_slot[u] = (uint32_t)sl;
+            if (ushow) {
+                ushow[u] = 0;
+                uclick[u] = 0;
+            }
+            u++;
+        }
+    }
+}
+
+// Step 5 (pull): mapped id = rank within the slot (sparse_table_ops.cc:130).
+__global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict__ descs,
+                                                      const uint32_t* __restrict__ lbase,
+                                                      const uint32_t* __restrict__ ubase, int N, uint32_t L,
+                                                      const DedupEntry* __restrict__ dt,
+                                                      const uint32_t* __restrict__ tidx) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        const int sl = find_slot(lb, N, gi);
+        const uint32_t u = dt[tidx[gi]].rank;
+        descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+    }
+}
+
+// Step 5 (push): batch_show = occurrences, batch_click = sum of labels
+// (sparse_table_ops.cc:283-296; labels are narrowed to int as there).
+__global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
+                                                    const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                    const DedupEntry* __restrict__ dt,
+                                                    const uint32_t* __restrict__ tidx, int32_t* ushow,
+                                                    int32_t* uclick) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        const int sl = find_slot(lb, N, gi);
+        const uint32_t u = dt[tidx[gi]].rank;
+        atomicAdd(&ushow[u], 1);
+        const int label = (int)descs[sl].labels[gi - lb[sl]];
+        if (label != 0) atomicAdd(&uclick[u], label);
+    }
+}
+
+// ------------------------------------------------------------ push grouping
+// Where the sign / gradient / counts of record u of a push come from.
+struct PushSrc {
+    // table-level push (SparseTable::Push): records in one array
+    const tn_sign_info* infos;
+    const float* grads;
+    // op-level push: compact distinct lists of the remap + per-slot gradient matrices
+    const uint64_t* uniq_sign;
+    const uint32_t* uniq_slot;
+    const uint32_t* ubase;
+    const int32_t* ushow;
+    const int32_t* uclick;
+    const SlotDesc* descs;
+    int dim;
+};
+
+__device__ __forceinline__ uint64_t src_sign(const PushSrc& p, uint32_t u) {
+    return p.infos ? p.infos[u].sign : p.uniq_sign[u];
+}
+
+// Records with the same sign must be applied one after the other in record
+// order (sparse_table.cc:72-82).  Every record joins the group of its sign...
+__global__ __launch_bounds__(256) void k_group_insert(PushSrc src, int64_t n_host, DevStatus* status, GroupEntry* gt,
+                                                      uint32_t* __restrict__ gidx, uint32_t* __restrict__ ord) {
+    const int64_t n = src.infos ? n_host : (int64_t)status->n_unique;
+    const uint32_t gcap = status->gcap;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
+        const uint64_t sign = src_sign(src, (uint32_t)u);
+        uint32_t e;
+        if (sign == EMPTY_KEY) {
+            e = gcap;
+        } else {
+            uint32_t idx = (uint32_t)slot_of(sign, gcap);
+            for (;;) {
+                e = idx;
+                uint64_t k = ld_relaxed(&gt[e].key);
+                if (k == sign) break;
+                if (k == EMPTY_KEY) {
+                    uint64_t old = atomicCAS(ull(&gt[e].key), EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                }
+                idx = (idx + 1 == gcap) ? 0 : idx + 1;
+            }
+        }
+        gidx[u] = e;
+        ord[u] = atomicAdd(&gt[e].cnt, 1u) + 1u;  // arrival number inside the group
+    }
+}
+
+// ...every group gets a slice of the member list...
+__global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupEntry* gt,
+                                                       uint64_t* __restrict__ grp_sign,
+                                                       uint32_t* __restrict__ grp_off,
+                                                       uint32_t* __restrict__ grp_cnt) {
+    const uint32_t n = status->gcap + 1;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+        const uint32_t c = gt[e].cnt;
+        const bool used = c != 0xFFFFFFFFu;
+        const uint32_t g = wave_alloc(used, &status->n_groups);
+        if (!used) continue;
+        const uint32_t k = c + 1;
+        const uint32_t off = atomicAdd(&status->list_cursor, k);
+        gt[e].off = off;
+        grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
+        grp_off[g] = off;
+        grp_cnt[g] = k;
+    }
+}
+
+// ...and the members are written into it (in arrival order; the apply kernel
+// walks them in ascending record order).
+__global__ __launch_bounds__(256) void k_group_fill(int64_t n_host, const uint32_t* n_dev, const GroupEntry* gt,
+                                                    const uint32_t* __restrict__ gidx,
+                                                    const uint32_t* __restrict__ ord, uint32_t* __restrict__ list) {
+    const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride)
+        list[gt[gidx[u]].off + ord[u]] = (uint32_t)u;
+}
+
+// -------------------------------------------------------------------- apply
+// smallest member of the group's list that is larger than prev (prev = -1 first)
+__device__ __forceinline__ uint32_t next_member(const uint32_t* list, uint32_t k, int64_t prev) {
+    uint32_t best = 0xFFFFFFFFu;
+    for (uint32_t t = 0; t < k; t++) {
+        uint32_t v = list[t];
+        if ((int64_t)v > prev && v < best) best = v;
+    }
+    return best;
+}
+
+// Resolves record u to its gradient row and counts; false if the op's gradient
+// matrix has no such row.
+__device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, const float*& g, int& show, int& click) {
+    if (p.infos) {
+        g = p.grads + (uint64_t)u * p.dim;
+        show = p.infos[u].batch_show;
+        click = p.infos[u].batch_click;
+        return true;
+    }
+    const uint32_t sl = p.uniq_slot[u];
+    const int64_t r = (int64_t)u - (int64_t)p.ubase[sl];
+    const SlotDesc& d = p.descs[sl];
+    if (r >= d.rows) return false;
+    g = d.grads + (uint64_t)r * p.dim;
+    show = p.ushow[u];
+    click = p.uclick[u];
+    return true;
+}
+
+// One group of LPG lanes owns one distinct sign: it loads the row once, applies
+// the sign's records in ascending record order (slot 0 first) and stores the
+// row once.  Each lane holds one float4 of every per-element array.
+//   AdaGrad  ada_grad_kernel.cc:105-129     Adam  adam_kernel.cc:112-125
+//   Ftrl     ftrl_kernel.cc:57-80
+template <int KIND, int LPG>
+__global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                   const uint32_t* __restrict__ grp_row,
+                                                   const uint32_t* __restrict__ grp_off,
+                                                   const uint32_t* __restrict__ grp_cnt,
+                                                   const uint32_t* __restrict__ list) {
+    const uint32_t n_groups = status->n_groups;
+    const int D = s.D;
+    const int sub = threadIdx.x % LPG;                       // my float4 inside the row
+    const int lane = (int)__lane_id();
+    const int lane0 = lane - sub;                            // first lane of my group in the wavefront
+    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    for (uint32_t g = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; g < n_groups; g += gstride) {
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
+        const uint32_t k = grp_cnt[g];
+        const uint32_t* mem = list + grp_off[g];
+        float* wp = s.w + (uint64_t)row * s.wstride;
+        float* sp = s.st + (uint64_t)row * s.sstride;
+        float4 w = reinterpret_cast<float4*>(wp)[sub];
+        float4 a, b;          // Adam m,v / Ftrl z,n
+        float g2sum = 0.f, show = 0.f, click = 0.f;
+        int delta_show = 0;
+        if (KIND == OPT_ADAGRAD) {
+            float4 h = *reinterpret_cast<const float4*>(sp);
+            g2sum = h.x;
+            show = h.y;
+            click = h.z;
+        } else {
+            a = reinterpret_cast<float4*>(sp)[sub];
+            b = reinterpret_cast<float4*>(sp + D)[sub];
+            delta_show = __float_as_int(sp[2 * D + 1]);
+        }
+        int64_t prev = -1;
+        bool any = false;
+        for (uint32_t j = 0; j < k; j++) {
+            const uint32_t u = (k == 1) ? mem[0] : next_member(mem, k, prev);
+            prev = u;
+            const float* gp;
+            int bshow, bclick;
+            if (!src_record(src, u, gp, bshow, bclick)) {
+                if (sub == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+                continue;
+            }
+            any = true;
+            const float4 gr = reinterpret_cast<const float4*>(gp)[sub];
+            if (KIND == OPT_ADAGRAD) {
+                show += (float)bshow;
+                click += (float)bclick;
+                const float p0 = gr.x * gr.x, p1 = gr.y * gr.y, p2 = gr.z * gr.z, p3 = gr.w * gr.w;
+                // add_g2sum: double accumulator over the float products, element order 0..D-1
+                double tot = 0.0;
+                for (int l = 0; l < LPG; l++) {
+                    double cand = tot;
+                    cand += (double)p0;
+                    cand += (double)p1;
+                    cand += (double)p2;
+                    cand += (double)p3;
+                    tot = __shfl(cand, lane0 + l);
+                }
+                g2sum = (float)((double)g2sum + tot / (double)D);
+                const float den = o.eps + sqrtf(g2sum);
+                w.x -= o.lr * gr.x / den;
+                w.y -= o.lr * gr.y / den;
+                w.z -= o.lr * gr.z / den;
+                w.w -= o.lr * gr.w / den;
+            } else if (KIND == OPT_ADAM) {
+                delta_show += bshow;
+                const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+#define TN_ADAM_E(W, M, V, G)                    \
+    M = o.beta1 * M + c1 * G;                    \
+    V = o.beta2 * V + c2 * G * G;                \
+    W -= o.lr * M / (o.eps + sqrtf(V));
+                TN_ADAM_E(w.x, a.x, b.x, gr.x)
+                TN_ADAM_E(w.y, a.y, b.y, gr.y)
+                TN_ADAM_E(w.z, a.z, b.z, gr.z)
+                TN_ADAM_E(w.w, a.w, b.w, gr.w)
+#undef TN_ADAM_E
+            } else {
+                delta_show += bshow;
+#define TN_FTRL_E(W, Z, NN, G)                                                   \
+    {                                                                            \
+        const float g2 = G * G;                                                  \
+        Z += G - o.lr * (sqrtf(NN + g2) - sqrtf(NN)) * W;                        \
+        NN += g2;                                                                \
+        if (fabsf(Z) <= o.lambda1) {                                             \
+            W = 0.f;                                                             \
+        } else {                                                                 \
+            W = -1 / ((o.beta + sqrtf(NN)) * o.lr + o.lambda2);                  \
+            if (Z > 0)                                                           \
+                W *= Z - o.lambda1;                                              \
+            else                                                                 \
+                W *= Z + o.lambda1;                                              \
+        }                                                                        \
+    }
+                TN_FTRL_E(w.x, a.x, b.x, gr.x)
+                TN_FTRL_E(w.y, a.y, b.y, gr.y)
+                TN_FTRL_E(w.z, a.z, b.z, gr.z)
+                TN_FTRL_E(w.w, a.w, b.w, gr.w)
+#undef TN_FTRL_E
+            }
+        }
+        if (!any) continue;
+        reinterpret_cast<float4*>(wp)[sub] = w;
+        if (KIND == OPT_ADAGRAD) {
+            if (sub == 0) {
+                *reinterpret_cast<float4*>(sp) = make_float4(g2sum, show, click, 0.f);  // no_show_days = 0
+                if (o.use_cvm) {
+                    wp[D] = show;
+                    wp[D + 1] = logf(click + 1) - logf(show + 1);
+                }
+            }
+        } else {
+            reinterpret_cast<float4*>(sp)[sub] = a;
+            reinterpret_cast<float4*>(sp + D)[sub] = b;
+            if (sub == 0) sp[2 * D + 1] = __int_as_float(delta_show);
+        }
+    }
+}
+
+// Any dim / alignment: one thread per distinct sign, scalar loops.
+template <int KIND>
+__global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                      const uint32_t* __restrict__ grp_row,
+                                                      const uint32_t* __restrict__ grp_off,
+                                                      const uint32_t* __restrict__ grp_cnt,
+                                                      const uint32_t* __restrict__ list) {
+    const uint32_t n_groups = status->n_groups;
+    const int D = s.D;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < n_groups; g += stride) {
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;
+        const uint32_t k = grp_cnt[g];
+        const uint32_t* mem = list + grp_off[g];
+        float* w = s.w + (uint64_t)row * s.wstride;
+        float* sp = s.st + (uint64_t)row * s.sstride;
+        int64_t prev = -1;
+        for (uint32_t j = 0; j < k; j++) {
+            const uint32_t u = (k == 1) ? mem[0] : next_member(mem, k, prev);
+            prev = u;
+            const float* gp;
+            int bshow, bclick;
+            if (!src_record(src, u, gp, bshow, bclick)) {
+                atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+                continue;
+            }
+            if (KIND == OPT_ADAGRAD) {
+                float show = sp[1] + (float)bshow;
+                float click = sp[2] + (float)bclick;
+                double add = 0.0;
+                for (int i = 0; i < D; i++) add += (double)(gp[i] * gp[i]);
+                float g2sum = (float)((double)sp[0] + add / (double)D);
+                const float den = o.eps + sqrtf(g2sum);
+                for (int i = 0; i < D; i++) w[i] -= o.lr * gp[i] / den;
+                sp[0] = g2sum;
+                sp[1] = show;
+                sp[2] = click;
+                sp[3] = 0.f;
+                if (o.use_cvm) {
+                    w[D] = show;
+                    w[D + 1] = logf(click + 1) - logf(show + 1);
+                }
+            } else if (KIND == OPT_ADAM) {
+                sp[2 * D + 1] = __int_as_float(__float_as_int(sp[2 * D + 1]) + bshow);
+                float* m = sp;
+                float* v = sp + D;
+                const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+                for (int i = 0; i < D; i++) {
+                    const float gi = gp[i];
+                    m[i] = o.beta1 * m[i] + c1 * gi;
+                    v[i] = o.beta2 * v[i] + c2 * gi * gi;
+                    w[i] -= o.lr * m[i] / (o.eps + sqrtf(v[i]));
+                }
+            } else {
+                sp[2 * D + 1] = __int_as_float(__float_as_int(sp[2 * D + 1]) + bshow);
+                float* z = sp;
+                float* nn = sp + D;
+                for (int i = 0; i < D; i++) {
+                    const float gi = gp[i];
+                    const float g2 = gi * gi;
+                    z[i] += gi - o.lr * (sqrtf(nn[i] + g2) - sqrtf(nn[i])) * w[i];
+                    nn[i] += g2;
+                    if (fabsf(z[i]) <= o.lambda1) {
+                        w[i] = 0.f;
+                    } else {
+                        float nw = -1 / ((o.beta + sqrtf(nn[i])) * o.lr + o.lambda2);
+                        if (z[i] > 0)
+                            nw *= z[i] - o.lambda1;
+                        else
+                            nw *= z[i] + o.lambda1;
+                        w[i] = nw;
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace tn
+
+#endif  // TN_SPARSE_KERNELS_H_

@@ -1,0 +1,875 @@
+// SparseTable host side: registry, HBM storage management and the launch
+// sequences of pull / push at table level (core/ps/table/sparse_table.cc:52-83)
+// and at operator level (core/kernels/sparse_table_ops.cc:170-265,317-368).
+#include "sparse_kernels.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace tn {
+
+namespace {
+
+constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:266
+constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
+constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
+constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
+
+struct HostStatus {
+    DevStatus st;
+    uint32_t ubase[MAX_SLOTS + 1];
+};
+
+struct SparseTable {
+    std::shared_ptr<OptConf> opt;
+    std::string name, group;
+    int dim = 0, use_cvm = 0, shard_num = 1, self_shard_id = 0;
+    uint32_t handle = 0;
+    int device = 0;
+    uint64_t seed = 0x243F6A8885A308D3ull;
+    uint64_t reserve_keys = 0;
+    bool allocated = false;
+    Store store{};
+    uint64_t count_upper = 0;  // upper bound of resident keys known without a device read
+    uint64_t booked = 0;       // part of count_upper booked for the inserts of the pending call
+
+    DevBuf ws;                      // per-call scratch
+    DevStatus* dstatus = nullptr;   // device
+    HostStatus* hpull = nullptr;    // pinned
+    HostStatus* hpush = nullptr;    // pinned
+    char* hstage = nullptr;         // pinned staging of slot descriptors
+    size_t hstage_bytes = 0;
+    hipEvent_t stage_ev = nullptr;  // staging buffer free again
+    bool stage_pending = false;
+    bool push_pending = false;      // hpush holds an unchecked status
+    bool pull_pending = false;
+    int pending_slots = 0;          // N of the pending calls
+    std::vector<int64_t> pending_rows;  // var rows of a pending async pull
+    int async_pull = 0;
+    int latched = TN_OK;
+    std::string latched_msg;
+    std::vector<int64_t> last_counts;
+    hipStream_t last_stream = nullptr;
+    std::mutex mu;
+};
+
+std::mutex g_tables_mu;
+std::vector<SparseTable*> g_tables;
+
+SparseTable* get_table(uint32_t h) {
+    std::lock_guard<std::mutex> lk(g_tables_mu);
+    if (h >= g_tables.size()) return nullptr;
+    return g_tables[h];
+}
+
+OptDev make_optdev(const SparseTable* t) {
+    const OptConf& c = *t->opt;
+    OptDev o{};
+    o.kind = c.kind;
+    o.zero_init = c.sparse_zero_init;
+    o.use_cvm = t->use_cvm;
+    o.lr = c.learning_rate;
+    o.eps = c.epsilon;
+    o.initial_g2sum = c.initial_g2sum;
+    o.initial_scale = c.initial_scale;
+    o.beta1 = c.beta1;
+    o.beta2 = c.beta2;
+    o.beta = c.beta;
+    o.lambda1 = c.lambda1;
+    o.lambda2 = c.lambda2;
+    return o;
+}
+
+int round4(int x) { return (x + 3) & ~3; }
+
+void layout(const SparseTable* t, Store& s) {
+    s.D = t->dim;
+    s.wdim = t->dim + (t->use_cvm ? 2 : 0);
+    bool vec = (t->dim % 4) == 0;
+    s.wstride = vec ? round4(s.wdim) : s.wdim;
+    int sf = (t->opt->kind == OPT_ADAGRAD) ? 4 : 2 * t->dim + 2;
+    s.sstride = vec ? round4(sf) : sf;
+}
+
+int state_floats(const SparseTable* t) { return (t->opt->kind == OPT_ADAGRAD) ? 4 : 2 * t->dim + 2; }
+
+int alloc_store(const SparseTable* t, uint64_t cap, Store& s, hipStream_t st) {
+    layout(t, s);
+    if (cap < 64) cap = 64;
+    if (cap > MAX_SLOTS_PER_TABLE) return fail(TN_ERR_UNSUPPORTED, "sparse table: more than 2^32 slots");
+    s.cap = cap;
+    const size_t rows = (size_t)cap + 1;
+    hipError_t e;
+    e = hipMalloc((void**)&s.keys, rows * sizeof(uint64_t) + 64);
+    if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc keys: ") + hipGetErrorString(e));
+    e = hipMalloc((void**)&s.w, rows * s.wstride * sizeof(float));
+    if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc weights: ") + hipGetErrorString(e));
+    e = hipMalloc((void**)&s.st, rows * s.sstride * sizeof(float));
+    if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc state: ") + hipGetErrorString(e));
+    void* small = nullptr;
+    TN_HIP(hipMalloc(&small, 64));
+    s.count = (unsigned long long*)small;
+    s.special = (uint32_t*)((char*)small + 8);
+    TN_HIP(hipMemsetAsync(small, 0, 64, st));
+    TN_HIP(hipMemsetAsync(s.keys, 0xFF, rows * sizeof(uint64_t), st));
+    return TN_OK;
+}
+
+void free_store(Store& s) {
+    if (s.keys) (void)hipFree(s.keys);
+    if (s.w) (void)hipFree(s.w);
+    if (s.st) (void)hipFree(s.st);
+    if (s.count) (void)hipFree(s.count);
+    s = Store{};
+}
+
+int ensure_side_buffers(SparseTable* t) {
+    if (t->dstatus) return TN_OK;
+    TN_HIP(hipMalloc((void**)&t->dstatus, sizeof(DevStatus)));
+    TN_HIP(hipMemset(t->dstatus, 0, sizeof(DevStatus)));
+    TN_HIP(hipHostMalloc((void**)&t->hpull, sizeof(HostStatus), hipHostMallocDefault));
+    TN_HIP(hipHostMalloc((void**)&t->hpush, sizeof(HostStatus), hipHostMallocDefault));
+    std::memset(t->hpull, 0, sizeof(HostStatus));
+    std::memset(t->hpush, 0, sizeof(HostStatus));
+    t->hstage_bytes = (size_t)MAX_SLOTS * sizeof(SlotDesc) + (MAX_SLOTS + 1) * sizeof(uint32_t);
+    TN_HIP(hipHostMalloc((void**)&t->hstage, t->hstage_bytes, hipHostMallocDefault));
+    TN_HIP(hipEventCreateWithFlags(&t->stage_ev, hipEventDisableTiming));
+    return TN_OK;
+}
+
+int ensure_allocated(SparseTable* t, hipStream_t st) {
+    TN_TRY(ensure_side_buffers(t));
+    if (t->allocated) return TN_OK;
+    uint64_t cap = DEFAULT_SLOTS;
+    if (t->reserve_keys) cap = (uint64_t)((double)t->reserve_keys / MAX_LOAD) + 64;
+    TN_TRY(alloc_store(t, cap, t->store, st));
+    t->allocated = true;
+    t->count_upper = 0;
+    return TN_OK;
+}
+
+const char* dev_err_text(uint32_t err) {
+    if (err & DEV_ERR_TABLE_FULL) return "sparse table is full";
+    if (err & DEV_ERR_UNKNOWN_KEY) return "embedding of a pushed sign not created yet (push before pull)";
+    if (err & DEV_ERR_VAR_CAPACITY) return "distinct signs of a slot exceed the rows of its variable";
+    if (err & DEV_ERR_GRAD_ROWS) return "gradient matrix of a slot has fewer rows than the slot has distinct signs";
+    return "";
+}
+
+int dev_err_code(uint32_t err) {
+    if (err & DEV_ERR_TABLE_FULL) return TN_ERR_TABLE_FULL;
+    if (err & DEV_ERR_UNKNOWN_KEY) return TN_ERR_UNKNOWN_KEY;
+    if (err & DEV_ERR_VAR_CAPACITY) return TN_ERR_VAR_CAPACITY;
+    if (err & DEV_ERR_GRAD_ROWS) return TN_ERR_INVALID_ARGUMENT;
+    return TN_OK;
+}
+
+void latch(SparseTable* t, int code, const std::string& msg) {
+    if (code != TN_OK && t->latched == TN_OK) {
+        t->latched = code;
+        t->latched_msg = msg;
+    }
+}
+
+// Examines the status blocks of finished calls (the stream must have been synchronised).
+void harvest(SparseTable* t) {
+    if (t->pull_pending) {
+        t->pull_pending = false;
+        const HostStatus& h = *t->hpull;
+        int N = t->pending_slots;
+        // the call booked room for every sign it could have inserted; keep what it did insert
+        if (t->booked >= h.st.n_new) t->count_upper -= t->booked - h.st.n_new;
+        t->booked = 0;
+        t->last_counts.assign(N, 0);
+        for (int s = 0; s < N; s++) t->last_counts[s] = (int64_t)h.ubase[s + 1] - (int64_t)h.ubase[s];
+        latch(t, dev_err_code(h.st.err), std::string("sparse pull: ") + dev_err_text(h.st.err));
+        for (int s = 0; s < N && s < (int)t->pending_rows.size(); s++)
+            if (t->last_counts[s] >= t->pending_rows[s])  // CHECK_LT(signs.size(), max_var_count)
+                latch(t, TN_ERR_VAR_CAPACITY,
+                      "sparse pull: slot " + std::to_string(s) + " has " + std::to_string(t->last_counts[s]) +
+                          " distinct signs, its variable only " + std::to_string(t->pending_rows[s]) + " rows");
+    }
+    if (t->push_pending) {
+        t->push_pending = false;
+        const HostStatus& h = *t->hpush;
+        int N = t->pending_slots;
+        if (N > 0) {
+            t->last_counts.assign(N, 0);
+            for (int s = 0; s < N; s++) t->last_counts[s] = (int64_t)h.ubase[s + 1] - (int64_t)h.ubase[s];
+        }
+        latch(t, dev_err_code(h.st.err), std::string("sparse push: ") + dev_err_text(h.st.err));
+    }
+}
+
+int take_latched(SparseTable* t) {
+    int code = t->latched;
+    if (code != TN_OK) {
+        set_error(t->latched_msg);
+        t->latched = TN_OK;
+        t->latched_msg.clear();
+    }
+    return code;
+}
+
+int sync_table(SparseTable* t, hipStream_t st) {
+    TN_HIP(hipStreamSynchronize(st));
+    if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
+    harvest(t);
+    return take_latched(t);
+}
+
+// Moves every resident row into a freshly allocated table of `cap` slots.
+int grow_to(SparseTable* t, uint64_t cap, hipStream_t st) {
+    Store& s = t->store;
+    if (cap > MAX_SLOTS_PER_TABLE) cap = MAX_SLOTS_PER_TABLE;
+    if (cap <= s.cap) return fail(TN_ERR_TABLE_FULL, "sparse table cannot grow beyond 2^32 slots");
+    Store bigger{};
+    int rc = alloc_store(t, cap, bigger, st);
+    if (rc != TN_OK) {
+        free_store(bigger);
+        return rc;
+    }
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
+    hipLaunchKernelGGL(k_rehash, dim3(launch_grid((int64_t)s.cap + 1, 256, GRID_CAP * 4)), dim3(256), 0, st, s, bigger,
+                       t->dstatus);
+    TN_HIP(hipMemcpyAsync(bigger.count, s.count, sizeof(unsigned long long), hipMemcpyDeviceToDevice, st));
+    TN_HIP(hipStreamSynchronize(st));
+    free_store(s);
+    s = bigger;
+    return TN_OK;
+}
+
+int read_count(SparseTable* t, hipStream_t st, uint64_t* out) {
+    TN_HIP(hipStreamSynchronize(st));
+    unsigned long long cnt = 0;
+    TN_HIP(hipMemcpy(&cnt, t->store.count, sizeof(cnt), hipMemcpyDeviceToHost));
+    t->count_upper = cnt;
+    *out = cnt;
+    return TN_OK;
+}
+
+// Makes room for up to `incoming` new keys: grows (re-inserts into a larger
+// table) when the load factor could pass MAX_LOAD (optimizer_kernel.h:266).
+// Callers have collected the status of earlier calls (t->booked == 0).
+int ensure_room(SparseTable* t, uint64_t incoming, hipStream_t st) {
+    Store& s = t->store;
+    if ((double)(t->count_upper + incoming) > MAX_LOAD * (double)s.cap) {
+        uint64_t cnt = 0;  // the bound may be loose: read the true count
+        TN_TRY(read_count(t, st, &cnt));
+        if ((double)(cnt + incoming) > MAX_LOAD * (double)s.cap) {
+            uint64_t need = (uint64_t)((double)(cnt + incoming) / MAX_LOAD) + 64;
+            TN_TRY(grow_to(t, std::max<uint64_t>(need, s.cap * 2), st));
+        }
+    }
+    t->count_upper += incoming;
+    t->booked = incoming;
+    return TN_OK;
+}
+
+// ---------------------------------------------------------------- workspace
+struct Carver {
+    char* base;
+    size_t off = 0;
+    template <typename T>
+    T* take(size_t n) {
+        off = align_up(off, 256);
+        T* p = reinterpret_cast<T*>(base + off);
+        off += n * sizeof(T);
+        return p;
+    }
+};
+
+// Scratch of one op call, carved from the table's workspace buffer.
+struct OpScratch {
+    SlotDesc* descs;
+    uint32_t* lbase;
+    uint32_t* ubase;
+    DedupEntry* dt;
+    size_t dt_entries;
+    uint32_t* tidx;
+    uint8_t* flag8;
+    uint32_t* tilesum;
+    uint32_t* tileoff;
+    uint32_t ntiles;
+    uint64_t* uniq_sign;
+    uint32_t* uniq_slot;
+    int32_t* ushow;
+    int32_t* uclick;
+    uint32_t* rows;
+    uint32_t* newlist;
+    // push grouping
+    GroupEntry* gt;
+    uint32_t* gidx;
+    uint32_t* ord;
+    uint32_t* list;
+    uint64_t* grp_sign;
+    uint32_t* grp_off;
+    uint32_t* grp_cnt;
+    uint32_t* grp_row;
+};
+
+void carve_group(Carver& c, OpScratch& w, size_t n) {
+    size_t gcap = std::max<size_t>(16, 2 * n);
+    w.gt = c.take<GroupEntry>(gcap + 1);
+    w.gidx = c.take<uint32_t>(n);
+    w.ord = c.take<uint32_t>(n);
+    w.list = c.take<uint32_t>(n);
+    w.grp_sign = c.take<uint64_t>(n);
+    w.grp_off = c.take<uint32_t>(n);
+    w.grp_cnt = c.take<uint32_t>(n);
+    w.grp_row = c.take<uint32_t>(n);
+}
+
+size_t carve_op(char* base, OpScratch& w, int N, size_t L, size_t dt_entries, bool push) {
+    Carver c{base};
+    w.descs = c.take<SlotDesc>(N);
+    w.lbase = c.take<uint32_t>(N + 1);
+    w.ubase = c.take<uint32_t>(N + 1);
+    w.dt = c.take<DedupEntry>(dt_entries);
+    w.dt_entries = dt_entries;
+    w.tidx = c.take<uint32_t>(L);
+    w.flag8 = c.take<uint8_t>(L / REMAP_ITEMS + REMAP_THREADS);
+    w.ntiles = (uint32_t)((L + REMAP_TILE - 1) / REMAP_TILE);
+    w.tilesum = c.take<uint32_t>(w.ntiles + 1);
+    w.tileoff = c.take<uint32_t>(w.ntiles + 1);
+    w.uniq_sign = c.take<uint64_t>(L);
+    w.uniq_slot = c.take<uint32_t>(L);
+    if (push) {
+        w.ushow = c.take<int32_t>(L);
+        w.uclick = c.take<int32_t>(L);
+        carve_group(c, w, L);
+        w.rows = nullptr;
+        w.newlist = nullptr;
+    } else {
+        w.ushow = w.uclick = nullptr;
+        w.rows = c.take<uint32_t>(L);
+        w.newlist = c.take<uint32_t>(L);
+    }
+    return align_up(c.off, 256);
+}
+
+// Validates the slot arrays of an op and stages descriptors; returns L.
+int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64_t* lens, std::vector<SlotDesc>& descs,
+                std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what) {
+    if (N <= 0 || !values || !lens) return fail(TN_ERR_INVALID_ARGUMENT, std::string(what) + ": no slots");
+    if (N > MAX_SLOTS)
+        return fail(TN_ERR_UNSUPPORTED, std::string(what) + ": more than " + std::to_string(MAX_SLOTS) + " slots");
+    descs.assign(N, SlotDesc{});
+    lbase.assign(N + 1, 0);
+    size_t l = 0, te = 0;
+    for (int s = 0; s < N; s++) {
+        if (lens[s] < 0 || (lens[s] > 0 && !values[s]))
+            return fail(TN_ERR_INVALID_ARGUMENT, std::string(what) + ": bad values tensor of slot " + std::to_string(s));
+        SlotDesc& d = descs[s];
+        d.values = values[s];
+        d.len = (uint32_t)lens[s];
+        d.lbase = (uint32_t)l;
+        d.tbase = (uint32_t)te;
+        size_t tcap = (size_t)lens[s] + (size_t)lens[s] / 2 + 8;
+        d.tcap = (uint32_t)tcap;
+        lbase[s] = (uint32_t)l;
+        l += (size_t)lens[s];
+        te += tcap + 1;
+        if (l > 0x7FFFFFF0ull || te > 0xFFFFFFF0ull)
+            return fail(TN_ERR_UNSUPPORTED, std::string(what) + ": more than 2^31 lookups in one call");
+    }
+    lbase[N] = (uint32_t)l;
+    L = l;
+    dt_entries = te;
+    return TN_OK;
+}
+
+int upload_slots(SparseTable* t, const OpScratch& w, const std::vector<SlotDesc>& descs,
+                 const std::vector<uint32_t>& lbase, hipStream_t st) {
+    if (t->stage_pending) {
+        TN_HIP(hipEventSynchronize(t->stage_ev));
+        t->stage_pending = false;
+    }
+    const size_t db = descs.size() * sizeof(SlotDesc);
+    const size_t lb = lbase.size() * sizeof(uint32_t);
+    std::memcpy(t->hstage, descs.data(), db);
+    std::memcpy(t->hstage + db, lbase.data(), lb);
+    TN_HIP(hipMemcpyAsync(w.descs, t->hstage, db, hipMemcpyHostToDevice, st));
+    TN_HIP(hipMemcpyAsync(w.lbase, t->hstage + db, lb, hipMemcpyHostToDevice, st));
+    TN_HIP(hipEventRecord(t->stage_ev, st));
+    t->stage_pending = true;
+    return TN_OK;
+}
+
+// Remap steps 1-4 shared by pull and push (k_remap_insert .. k_assign_rank).
+void launch_remap(const OpScratch& w, int N, uint32_t L, DevStatus* dstatus, hipStream_t st) {
+    hipLaunchKernelGGL(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), 0, st,
+                       reinterpret_cast<uint4*>(w.dt), w.dt_entries);
+    hipLaunchKernelGGL(k_remap_insert, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase, N, L,
+                       w.dt, w.tidx);
+    hipLaunchKernelGGL(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), 0, st, w.lbase, N, L, w.dt, w.tidx, w.flag8,
+                       w.tilesum);
+    hipLaunchKernelGGL(k_scan_tiles, dim3(1), dim3(1024), 0, st, w.tilesum, w.tileoff, w.ntiles, w.lbase, w.ubase, N, L,
+                       dstatus);
+    hipLaunchKernelGGL(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), 0, st, w.descs, w.lbase, N, L, w.dt, w.tidx,
+                       w.flag8, w.tileoff, w.ubase, w.uniq_sign, w.uniq_slot, w.ushow, w.uclick);
+}
+
+template <int KIND>
+void launch_apply_kind(int lpg, int blocks_hint, const Store& s, const OptDev& o, const PushSrc& src,
+                       DevStatus* dstatus, const OpScratch& w, int64_t n_upper, hipStream_t st) {
+    (void)blocks_hint;
+#define TN_LAUNCH_VEC(LPG)                                                                                            \
+    hipLaunchKernelGGL((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 2)), dim3(256), 0, st, \
+                       s, o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list)
+    switch (lpg) {
+        case 1: TN_LAUNCH_VEC(1); break;
+        case 2: TN_LAUNCH_VEC(2); break;
+        case 4: TN_LAUNCH_VEC(4); break;
+        case 8: TN_LAUNCH_VEC(8); break;
+        case 16: TN_LAUNCH_VEC(16); break;
+        case 32: TN_LAUNCH_VEC(32); break;
+        default:
+            hipLaunchKernelGGL((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), 0, st, s,
+                               o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list);
+    }
+#undef TN_LAUNCH_VEC
+}
+
+// Group the records by sign, find the rows, apply.  n_upper bounds the number
+// of records; the exact number is n_host (table level) or status->n_unique.
+void launch_push_tail(SparseTable* t, const OpScratch& w, const PushSrc& src, int64_t n_host, int64_t n_upper,
+                      bool vec_ok, hipStream_t st) {
+    const Store& s = t->store;
+    const OptDev o = make_optdev(t);
+    DevStatus* ds = t->dstatus;
+    const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
+    const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
+    hipLaunchKernelGGL(k_fill_groups, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), 0, st, w.gt, ds);
+    hipLaunchKernelGGL(k_group_insert, dim3(gblocks), dim3(256), 0, st, src, n_host, ds, w.gt, w.gidx, w.ord);
+    hipLaunchKernelGGL(k_group_compact, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), 0, st, ds,
+                       w.gt, w.grp_sign, w.grp_off, w.grp_cnt);
+    hipLaunchKernelGGL(k_group_fill, dim3(gblocks), dim3(256), 0, st, n_host, n_dev, w.gt, w.gidx, w.ord, w.list);
+    hipLaunchKernelGGL((k_probe<false>), dim3(gblocks), dim3(256), 0, st, s, w.grp_sign, (int64_t)0, &ds->n_groups,
+                       w.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+    int lpg = 0;
+    if (vec_ok && s.D % 4 == 0) {
+        int q = s.D / 4;
+        if (q >= 1 && q <= 32 && (q & (q - 1)) == 0) lpg = q;
+    }
+    switch (o.kind) {
+        case OPT_ADAGRAD: launch_apply_kind<OPT_ADAGRAD>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
+        case OPT_ADAM: launch_apply_kind<OPT_ADAM>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
+        default: launch_apply_kind<OPT_FTRL>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
+    }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+}  // namespace tn
+
+using namespace tn;
+
+extern "C" {
+
+int tn_sparse_table_create(tn_opt_t opt, const char* name, int dimension, int use_cvm, int shard_num,
+                           int self_shard_id, const char* embedding_group, uint32_t* handle) {
+    if (!handle) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_create: handle is NULL");
+    auto conf = get_opt(opt);
+    if (!conf) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_create: unknown optimizer handle");
+    if (dimension <= 0 || dimension > 4096)
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_create: dimension must be in [1, 4096]");
+    if (shard_num != 1 || self_shard_id != 0)
+        return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_create: one worker only (shard_num 1, self_shard_id 0)");
+    std::string group = embedding_group ? embedding_group : "";
+    std::lock_guard<std::mutex> lk(g_tables_mu);
+    if (!group.empty()) {  // sparse_table.cc:175-180
+        for (SparseTable* t : g_tables)
+            if (t->group == group) {
+                *handle = t->handle;
+                return TN_OK;
+            }
+    }
+    SparseTable* t = new SparseTable();
+    t->opt = conf;
+    t->name = name ? name : "";
+    t->group = group;
+    t->dim = dimension;
+    // only the AdaGrad row maintains the cvm columns (ada_grad_kernel.cc:99-102,123-128)
+    t->use_cvm = (use_cvm && conf->kind == OPT_ADAGRAD) ? 1 : 0;
+    t->shard_num = shard_num;
+    t->self_shard_id = self_shard_id;
+    if (hipGetDevice(&t->device) != hipSuccess) t->device = 0;
+    t->handle = (uint32_t)g_tables.size();
+    g_tables.push_back(t);
+    *handle = t->handle;
+    return TN_OK;
+}
+
+int tn_sparse_table_reserve(uint32_t handle, uint64_t max_keys) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_reserve: bad table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (!t->allocated) {
+        t->reserve_keys = max_keys;
+        return TN_OK;
+    }
+    hipStream_t st = t->last_stream;
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    uint64_t want = (uint64_t)((double)max_keys / MAX_LOAD) + 64;
+    if (want <= t->store.cap) return TN_OK;
+    return grow_to(t, want, st);
+}
+
+int tn_sparse_table_set_seed(uint32_t handle, uint64_t seed) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_set_seed: bad table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->seed = seed;
+    return TN_OK;
+}
+
+int tn_sparse_table_key_count(uint32_t handle, uint64_t* count) {
+    SparseTable* t = get_table(handle);
+    if (!t || !count) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_key_count: bad table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    *count = 0;
+    if (!t->allocated) return TN_OK;
+    if (t->last_stream) TN_HIP(hipStreamSynchronize(t->last_stream));
+    TN_HIP(hipDeviceSynchronize());
+    unsigned long long cnt = 0;
+    TN_HIP(hipMemcpy(&cnt, t->store.count, sizeof(cnt), hipMemcpyDeviceToHost));
+    t->count_upper = cnt;
+    *count = cnt;
+    return TN_OK;
+}
+
+int tn_sparse_table_capacity(uint32_t handle, uint64_t* slots) {
+    SparseTable* t = get_table(handle);
+    if (!t || !slots) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_capacity: bad table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    *slots = t->allocated ? t->store.cap : 0;
+    return TN_OK;
+}
+
+int tn_sparse_table_row_layout(uint32_t handle, int* weight_floats, int* state_floats_out) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_row_layout: bad table handle");
+    if (weight_floats) *weight_floats = t->dim + (t->use_cvm ? 2 : 0);
+    if (state_floats_out) *state_floats_out = state_floats(t);
+    return TN_OK;
+}
+
+int tn_sparse_table_set_async(uint32_t handle, int async_pull) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_set_async: bad table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->async_pull = async_pull ? 1 : 0;
+    return TN_OK;
+}
+
+int tn_sparse_table_sync(uint32_t handle) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_sync: bad table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (!t->allocated) return TN_OK;
+    return sync_table(t, t->last_stream);
+}
+
+int tn_sparse_table_last_unique_counts(uint32_t handle, int N, int64_t* counts) {
+    SparseTable* t = get_table(handle);
+    if (!t || !counts) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_last_unique_counts: bad table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (t->pull_pending || t->push_pending) {
+        TN_HIP(hipStreamSynchronize(t->last_stream));
+        harvest(t);
+    }
+    if ((int)t->last_counts.size() != N)
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_last_unique_counts: last op had " +
+                                                 std::to_string(t->last_counts.size()) + " slots");
+    for (int s = 0; s < N; s++) counts[s] = t->last_counts[s];
+    return TN_OK;
+}
+
+// ------------------------------------------------------------ table level
+int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_pull: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && (!signs || !out))) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_pull: NULL buffer");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    const int wdim = t->dim + (t->use_cvm ? 2 : 0);
+    if (dim != wdim)
+        return fail(TN_ERR_DIM_MISMATCH,
+                    "tn_sparse_table_pull: dim " + std::to_string(dim) + " but table rows hold " + std::to_string(wdim));
+    if (n > 0x7FFFFFF0LL) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_pull: more than 2^31 signs");
+    t->last_stream = st;
+    if (n == 0) return sync_table(t, st);
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    TN_TRY(ensure_room(t, (uint64_t)n, st));
+    TN_TRY(t->ws.ensure(2 * align_up((size_t)n * sizeof(uint32_t), 256)));
+    Carver c{(char*)t->ws.p};
+    uint32_t* rows = c.take<uint32_t>(n);
+    uint32_t* newlist = c.take<uint32_t>(n);
+    const Store& s = t->store;
+    const OptDev o = make_optdev(t);
+    const int blocks = launch_grid(n, 256, GRID_CAP * 2);
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, 0u);
+    hipLaunchKernelGGL((k_probe<true>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
+                       newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    hipLaunchKernelGGL(k_init_rows, dim3(blocks), dim3(256), 0, st, s, o, t->seed, signs, rows, newlist, t->dstatus);
+    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
+    if (wdim % 4 == 0 && s.wstride % 4 == 0 && aligned16(out))
+        hipLaunchKernelGGL((k_gather_rows<4>), dim3(launch_grid(n * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), 0, st, s,
+                           rows, n, out);
+    else
+        hipLaunchKernelGGL((k_gather_rows<1>), dim3(launch_grid(n * wdim, 256, GRID_CAP * 4)), dim3(256), 0, st, s, rows,
+                           n, out);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    t->hpull->ubase[0] = 0;
+    t->pull_pending = true;
+    t->pending_slots = 0;
+    t->pending_rows.clear();
+    return sync_table(t, st);
+}
+
+int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float* grads, int64_t n, int dim,
+                         void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_push: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && (!infos || !grads))) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_push: NULL buffer");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    const int wdim = t->dim + (t->use_cvm ? 2 : 0);
+    if (dim != wdim)
+        return fail(TN_ERR_DIM_MISMATCH,
+                    "tn_sparse_table_push: dim " + std::to_string(dim) + " but table rows hold " + std::to_string(wdim));
+    if (n > 0x7FFFFFF0LL) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_push: more than 2^31 records");
+    t->last_stream = st;
+    if (n == 0) return TN_OK;
+    if (t->push_pending || t->pull_pending) {  // one status block per direction: collect the previous one first
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    OpScratch w{};
+    {
+        Carver probe{nullptr};
+        carve_group(probe, w, (size_t)n);
+        TN_TRY(t->ws.ensure(align_up(probe.off, 256) + 256));
+        Carver c{(char*)t->ws.p};
+        carve_group(c, w, (size_t)n);
+    }
+    PushSrc src{};
+    src.infos = infos;
+    src.grads = grads;
+    src.dim = dim;
+    const uint32_t gcap = (uint32_t)std::max<int64_t>(16, 2 * n);
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, gcap);
+    launch_push_tail(t, w, src, n, n, aligned16(grads) && dim % 4 == 0, st);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    t->push_pending = true;
+    t->pending_slots = 0;
+    return TN_OK;
+}
+
+int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const float* w, const float* state, int64_t n,
+                              void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_load_rows: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && (!signs || !w))) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_load_rows: NULL buffer");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    t->last_stream = st;
+    if (n == 0) return TN_OK;
+    if (n > 0x7FFFFFF0LL) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_load_rows: more than 2^31 rows per call");
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    TN_TRY(ensure_room(t, (uint64_t)n, st));
+    TN_TRY(t->ws.ensure(2 * align_up((size_t)n * sizeof(uint32_t), 256)));
+    Carver c{(char*)t->ws.p};
+    uint32_t* rows = c.take<uint32_t>(n);
+    uint32_t* newlist = c.take<uint32_t>(n);
+    const Store& s = t->store;
+    const int blocks = launch_grid(n, 256, GRID_CAP * 4);
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, 0u);
+    hipLaunchKernelGGL((k_probe<true>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
+                       newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
+    hipLaunchKernelGGL(k_load_rows, dim3(blocks), dim3(256), 0, st, s, make_optdev(t), rows, n, w, state);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    t->pull_pending = true;
+    t->pending_slots = 0;
+    t->pending_rows.clear();
+    return sync_table(t, st);
+}
+
+int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t n, float* w, float* state,
+                                uint8_t* found, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_export_rows: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && !signs)) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_export_rows: NULL buffer");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    t->last_stream = st;
+    if (n == 0) return TN_OK;
+    if (n > 0x7FFFFFF0LL) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_export_rows: more than 2^31 rows per call");
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    TN_TRY(t->ws.ensure(align_up((size_t)n * sizeof(uint32_t), 256)));
+    uint32_t* rows = (uint32_t*)t->ws.p;
+    const Store& s = t->store;
+    const int blocks = launch_grid(n, 256, GRID_CAP * 4);
+    hipLaunchKernelGGL((k_probe<false>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
+                       (uint32_t*)nullptr, t->dstatus, 0u);
+    hipLaunchKernelGGL(k_export_rows, dim3(blocks), dim3(256), 0, st, s, make_optdev(t), rows, n, w, state, found);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipStreamSynchronize(st));
+    return TN_OK;
+}
+
+// --------------------------------------------------------------- op level
+int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                            float* const* vars, const int64_t* var_rows, int var_dim, int64_t* const* mapped_values,
+                            void* stream) {
+    SparseTable* t = get_table(table_handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "SparseTablePull: bad table handle " + std::to_string(table_handle));
+    if (!vars || !var_rows || !mapped_values) return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePull: NULL argument");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    const int wdim = t->dim + (t->use_cvm ? 2 : 0);
+    if (var_dim != wdim)
+        return fail(TN_ERR_DIM_MISMATCH, "SparseTablePull: variable dim " + std::to_string(var_dim) +
+                                             " but table rows hold " + std::to_string(wdim));
+    std::vector<SlotDesc> descs;
+    std::vector<uint32_t> lbase;
+    size_t L = 0, dt_entries = 0;
+    TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePull"));
+    bool vec = (wdim % 4 == 0) && (t->store.wstride % 4 == 0);
+    for (int s = 0; s < N; s++) {
+        if (var_rows[s] < 0 || !vars[s] || (value_lens[s] > 0 && !mapped_values[s]))
+            return fail(TN_ERR_INVALID_ARGUMENT,
+                        "sparse pull variable must Matrix(sign_id_cnt, dim), slot " + std::to_string(s));
+        descs[s].var = vars[s];
+        descs[s].rows = var_rows[s];
+        descs[s].mapped = mapped_values[s];
+        vec = vec && aligned16(vars[s]);
+    }
+    t->last_stream = st;
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    if (L == 0) {
+        t->last_counts.assign(N, 0);
+        return take_latched(t);
+    }
+    TN_TRY(ensure_room(t, (uint64_t)L, st));
+    OpScratch w{};
+    size_t need = carve_op(nullptr, w, N, L, dt_entries, false);
+    TN_TRY(t->ws.ensure(need));
+    carve_op((char*)t->ws.p, w, N, L, dt_entries, false);
+    TN_TRY(upload_slots(t, w, descs, lbase, st));
+
+    const Store& s = t->store;
+    const OptDev o = make_optdev(t);
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
+    launch_remap(w, N, (uint32_t)L, t->dstatus, st);
+    hipLaunchKernelGGL(k_write_mapped, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase,
+                       w.ubase, N, (uint32_t)L, w.dt, w.tidx);
+    const int ublocks = launch_grid(L, 256, GRID_CAP * 2);
+    hipLaunchKernelGGL((k_probe<true>), dim3(ublocks), dim3(256), 0, st, s, w.uniq_sign, (int64_t)0,
+                       &t->dstatus->n_unique, w.rows, w.newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    hipLaunchKernelGGL(k_init_rows, dim3(ublocks), dim3(256), 0, st, s, o, t->seed, w.uniq_sign, w.rows, w.newlist,
+                       t->dstatus);
+    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
+    if (vec)
+        hipLaunchKernelGGL((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), 0,
+                           st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+    else
+        hipLaunchKernelGGL((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), 0, st,
+                           s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(t->hpull->ubase, w.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    t->pull_pending = true;
+    t->pending_slots = N;
+    t->pending_rows.assign(var_rows, var_rows + N);
+    if (t->async_pull) return TN_OK;
+    return sync_table(t, st);
+}
+
+int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                            const float* const* grads, const int64_t* grad_rows, int grad_dim,
+                            const int64_t* const* feature_labels, void* stream) {
+    SparseTable* t = get_table(table_handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "SparseTablePush: bad table handle " + std::to_string(table_handle));
+    if (!grads || !grad_rows || !feature_labels) return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush: NULL argument");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    const int wdim = t->dim + (t->use_cvm ? 2 : 0);
+    if (grad_dim != wdim)
+        return fail(TN_ERR_DIM_MISMATCH, "SparseTablePush: gradient dim " + std::to_string(grad_dim) +
+                                             " but table rows hold " + std::to_string(wdim));
+    std::vector<SlotDesc> descs;
+    std::vector<uint32_t> lbase;
+    size_t L = 0, dt_entries = 0;
+    TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePush"));
+    bool vec = (grad_dim % 4 == 0);
+    for (int s = 0; s < N; s++) {
+        if (grad_rows[s] < 0 || (grad_rows[s] > 0 && !grads[s]) || (value_lens[s] > 0 && !feature_labels[s]))
+            return fail(TN_ERR_INVALID_ARGUMENT,
+                        "sparse push grad must Matrix(sign_id_cnt, dim), slot " + std::to_string(s));
+        descs[s].grads = grads[s];
+        descs[s].rows = grad_rows[s];
+        descs[s].labels = feature_labels[s];
+        vec = vec && aligned16(grads[s]);
+    }
+    t->last_stream = st;
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    if (L == 0) return TN_OK;
+    OpScratch w{};
+    size_t need = carve_op(nullptr, w, N, L, dt_entries, true);
+    TN_TRY(t->ws.ensure(need));
+    carve_op((char*)t->ws.p, w, N, L, dt_entries, true);
+    TN_TRY(upload_slots(t, w, descs, lbase, st));
+
+    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
+    launch_remap(w, N, (uint32_t)L, t->dstatus, st);
+    hipLaunchKernelGGL(k_count_show, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase, N,
+                       (uint32_t)L, w.dt, w.tidx, w.ushow, w.uclick);
+    PushSrc src{};
+    src.uniq_sign = w.uniq_sign;
+    src.uniq_slot = w.uniq_slot;
+    src.ubase = w.ubase;
+    src.ushow = w.ushow;
+    src.uclick = w.uclick;
+    src.descs = w.descs;
+    src.dim = grad_dim;
+    launch_push_tail(t, w, src, 0, (int64_t)L, vec, st);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(t->hpush->ubase, w.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    t->push_pending = true;
+    t->pending_slots = N;
+    return TN_OK;
+}
+
+}  // extern "C"

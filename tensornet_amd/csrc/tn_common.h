@@ -1,0 +1,123 @@
+// Shared declarations of the HIP library behind include/tensornet_amd.h.
+// gfx950 only: 64-wide wavefronts, no portability layers.
+#ifndef TN_COMMON_H_
+#define TN_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "tensornet_amd.h"
+
+namespace tn {
+
+// ------------------------------------------------------------------ errors
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+
+#define TN_HIP(expr)                                                                               \
+    do {                                                                                           \
+        hipError_t _e = (expr);                                                                    \
+        if (_e != hipSuccess) {                                                                    \
+            return ::tn::fail(TN_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(_e));      \
+        }                                                                                          \
+    } while (0)
+
+#define TN_TRY(expr)              \
+    do {                          \
+        int _rc = (expr);         \
+        if (_rc != TN_OK) return _rc; \
+    } while (0)
+
+// -------------------------------------------------------------- optimizers
+enum OptKind { OPT_ADAGRAD = 0, OPT_ADAM = 1, OPT_FTRL = 2 };
+
+// All hyper-parameters are float, as in core/ps/optimizer/optimizer.h:36-144.
+struct OptConf {
+    int kind = OPT_ADAGRAD;
+    float learning_rate = 0.01f;
+    float show_decay_rate = 0.98f;
+    int sparse_zero_init = 0;
+    // AdaGrad
+    float initial_g2sum = 0.f, initial_scale = 1.f, epsilon = 1e-8f;
+    float grad_decay_rate = 1.f, mom_decay_rate = 1.f, show_threshold = 0.f;
+    int no_show_days = 1000, elimination_logic = 0;
+    // Adam
+    float beta1 = 0.9f, beta2 = 0.999f;
+    // Ftrl
+    float beta = 1.f, lambda1 = 0.1f, lambda2 = 1.f;
+};
+
+// Snapshot of the optimizer passed by value to kernels.
+struct OptDev {
+    int kind;
+    int zero_init;
+    int use_cvm;
+    float lr, eps, initial_g2sum, initial_scale;
+    float beta1, beta2;           // Adam
+    float beta, lambda1, lambda2; // Ftrl
+};
+
+std::shared_ptr<OptConf> get_opt(tn_opt_t h);
+
+// ------------------------------------------------------------ device bits
+constexpr uint64_t EMPTY_KEY = 0xFFFFFFFFFFFFFFFFull;
+constexpr uint32_t NO_ROW = 0xFFFFFFFFu;
+
+// status / error flags latched on the device by kernels
+enum : uint32_t {
+    DEV_ERR_VAR_CAPACITY = 1u,
+    DEV_ERR_UNKNOWN_KEY = 2u,
+    DEV_ERR_TABLE_FULL = 4u,
+    DEV_ERR_GRAD_ROWS = 8u,
+};
+
+struct DevStatus {
+    uint32_t err;        // DEV_ERR_* bits
+    uint32_t n_unique;   // U = sum of per-slot distinct signs
+    uint32_t n_groups;   // globally distinct signs of a push
+    uint32_t n_new;      // rows inserted by this call
+    uint32_t gcap;       // slots of the per-call group table
+    uint32_t list_cursor;
+    uint32_t pad[2];
+};
+
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+    x ^= x >> 33;
+    x *= 0xff51afd7ed558ccdull;
+    x ^= x >> 33;
+    x *= 0xc4ceb9fe1a85ec53ull;
+    x ^= x >> 33;
+    return x;
+}
+
+// maps a sign to [0, cap) without a division
+__device__ __forceinline__ uint64_t slot_of(uint64_t sign, uint64_t cap) { return __umul64hi(mix64(sign), cap); }
+
+__device__ __forceinline__ uint64_t ld_relaxed(const uint64_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t ld_relaxed(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// grow-only device buffer
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+    int ensure(size_t need);
+    void release();
+};
+
+int launch_grid(int64_t work_items, int threads, int max_blocks);
+
+}  // namespace tn
+
+#endif  // TN_COMMON_H_

@@ -1,0 +1,93 @@
+"""Shared scaffolding of the GPU parity tests: the same seeded snapshot and the
+same batches are fed to the HIP path (through the C ABI) and to the CPU
+oracle."""
+import numpy as np
+import torch
+
+from tensornet_amd import synth
+
+KINDS = {"AdaGrad": 0, "Adam": 1, "Ftrl": 2}
+
+# tolerance of the post-update comparison (reduction / evaluation order may differ)
+RTOL, ATOL = 1e-5, 1e-7
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+class Pair(object):
+    """One sparse table on the GPU and its CPU oracle twin."""
+
+    def __init__(self, tn, oracle, opt, dim, hyper, use_cvm=False, reserve=200000, zero_init=False, seed=11):
+        self.tn, self.oracle = tn, oracle
+        self.opt, self.dim, self.use_cvm = opt, dim, use_cvm
+        factory = getattr(tn.core, opt)
+        self.gopt = factory(**hyper)
+        if zero_init:
+            tn.core.set_sparse_init_mode(self.gopt, False)
+        self.h = tn.core.create_sparse_table(self.gopt, "", dim, use_cvm, "")
+        tn.core.reserve_sparse_table(self.h, reserve)
+        tn.core.set_sparse_table_seed(self.h, seed)
+        self.o = oracle.Table(KINDS[opt], dim, use_cvm=use_cvm, zero_init=zero_init, buckets=1 << 16, **hyper)
+        self.wf, self.sf = tn.core.sparse_table_row_layout(self.h)
+        assert (self.wf, self.sf) == (self.o.wf, self.o.sf)
+
+    def populate(self, signs_u64, seed=0, state=None):
+        signs_u64 = np.unique(np.asarray(signs_u64, dtype=np.uint64))
+        w = synth.snapshot_rows(signs_u64, self.wf, seed=seed)
+        if self.use_cvm:
+            w[:, self.dim:] = 0
+        self.o.set_rows(signs_u64, w, state)
+        self.tn.ops.table_load_rows(self.h, dev(signs_u64.view(np.int64)), dev(w),
+                                    dev(state) if state is not None else None)
+        return signs_u64
+
+    def pull_op(self, values, var_rows=None):
+        """Runs the op on both sides; returns (gpu mapped, gpu vars, cpu mapped, cpu vars, counts)."""
+        n = len(values)
+        if var_rows is None:
+            var_rows = [len(v) + 1 for v in values]
+        cvars = [np.full((r, self.wf), -7.0, np.float32) for r in var_rows]
+        rc, cmapped, counts = self.o.pull_op(values, cvars)
+        assert rc == 0
+        gvars = [torch.full((r, self.wf), -7.0, dtype=torch.float32, device="cuda") for r in var_rows]
+        gvalues = [dev(v) for v in values]
+        gmapped = self.tn.ops.sparse_table_pull(gvars, gvalues, self.h)
+        gcounts = self.tn.ops.sparse_table_last_unique_counts(self.h, n)
+        assert gcounts == counts.tolist()
+        return gmapped, gvars, cmapped, cvars, counts
+
+    def push_op(self, values, grads, labels):
+        rc, counts = self.o.push_op(values, grads, labels)
+        assert rc == 0
+        self.tn.ops.sparse_table_push([dev(v) for v in values], [dev(g) for g in grads], [dev(l) for l in labels],
+                                      self.h)
+        self.tn.ops.sparse_table_sync(self.h)
+        return counts
+
+    def export(self, signs_u64):
+        signs_u64 = np.asarray(signs_u64, dtype=np.uint64)
+        gw, gs, gf = self.tn.ops.table_export_rows(self.h, dev(signs_u64.view(np.int64)))
+        cw, cs, cf = self.o.get_rows(signs_u64)
+        return (gw.cpu().numpy(), gs.cpu().numpy(), gf.cpu().numpy()), (cw, cs, cf)
+
+    def assert_rows_match(self, signs_u64, exact=False):
+        (gw, gs, gf), (cw, cs, cf) = self.export(signs_u64)
+        assert (gf == cf).all()
+        sel = cf.astype(bool)
+        if exact:
+            assert (gw[sel].view(np.int32) == cw[sel].view(np.int32)).all()
+            assert (gs[sel].view(np.int32) == cs[sel].view(np.int32)).all()
+            return 1.0
+        np.testing.assert_allclose(gw[sel], cw[sel], rtol=RTOL, atol=ATOL)
+        nf = self.sf - 1 if self.opt != "AdaGrad" else 3
+        np.testing.assert_allclose(gs[sel][:, :nf], cs[sel][:, :nf], rtol=RTOL, atol=ATOL)
+        # integer words of the state (no_show_days / delta_show) are exact
+        assert (gs[sel][:, -1].view(np.int32) == cs[sel][:, -1].view(np.int32)).all()
+        same = (gw[sel].view(np.int32) == cw[sel].view(np.int32)).mean() if sel.any() else 1.0
+        return float(same)
+
+
+def all_signs(values):
+    return np.unique(np.concatenate([np.asarray(v, dtype=np.int64) for v in values]).view(np.uint64))

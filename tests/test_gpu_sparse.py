@@ -1,0 +1,372 @@
+"""GPU parity of the sparse pull / push path against the CPU oracle, through
+the C ABI.  Bar: mapped ids and pulled rows bit-exact; post-update weights and
+state within 1e-5 relative / 1e-7 absolute; integer state exact."""
+import numpy as np
+import pytest
+import torch
+
+from tensornet_amd import synth
+
+from helpers import ATOL, RTOL, Pair, all_signs, dev
+
+pytestmark = pytest.mark.gpu
+
+ADAGRAD_HP = dict(learning_rate=0.01, initial_g2sum=0.1, epsilon=1e-8)
+ADAM_HP = dict(learning_rate=1e-3, beta1=0.9, beta2=0.999, epsilon=1e-8)
+FTRL_HP = dict(learning_rate=0.05, beta=1.0, lambda1=1.0, lambda2=1.0)
+
+
+def random_batch(rng, slots, max_len, vocab, ragged=True):
+    pool = synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)).view(np.int64)
+    out = []
+    for _ in range(slots):
+        n = int(rng.integers(0, max_len + 1)) if ragged else max_len
+        out.append(pool[rng.integers(0, vocab, n)])
+    return out
+
+
+def check_pull(pair, values, var_rows=None):
+    gm, gv, cm, cv, counts = pair.pull_op(values, var_rows)
+    for s in range(len(values)):
+        assert (gm[s].cpu().numpy() == cm[s]).all(), "mapped ids of slot %d" % s
+        # bit-exact rows, including the untouched tail of the variable
+        assert (gv[s].cpu().numpy().view(np.int32) == cv[s].view(np.int32)).all(), "var rows of slot %d" % s
+    return counts
+
+
+def test_cfg1_pull_then_push(tn, oracle):
+    """The reference's own CPU-runnable case: 1024 x 8 single-id slots, dim 8 AdaGrad."""
+    cfg = synth.CONFIGS["cfg1"]
+    pair = Pair(tn, oracle, "AdaGrad", cfg["dim"], cfg["hyper"], reserve=1 << 20)
+    values = synth.make_batch(cfg, 0)
+    assert sum(len(v) for v in values) == 8192
+    # resident set: every key of the 1e6 vocabulary that the batch can touch is loaded on both sides
+    resident = synth.splitmix64(np.arange(1, 200001, dtype=np.uint64))
+    pair.populate(np.concatenate([resident, all_signs(values)]))
+    counts = check_pull(pair, values)
+    grads = synth.make_grads(counts, cfg["dim"], cfg["grad_sigma"])
+    labels = [np.zeros(len(v), np.int64) for v in values]
+    pair.push_op(values, grads, labels)
+    same = pair.assert_rows_match(all_signs(values))
+    assert same > 0.99
+    check_pull(pair, values)  # pulling again returns the updated rows
+
+
+@pytest.mark.parametrize("opt,dim,hyper", [
+    ("AdaGrad", 16, ADAGRAD_HP), ("AdaGrad", 64, ADAGRAD_HP), ("AdaGrad", 1, ADAGRAD_HP), ("AdaGrad", 6, ADAGRAD_HP),
+    ("Adam", 16, ADAM_HP), ("Adam", 8, ADAM_HP), ("Adam", 3, ADAM_HP),
+    ("Ftrl", 1, FTRL_HP), ("Ftrl", 16, FTRL_HP),
+])
+def test_multi_batch_parity(tn, oracle, opt, dim, hyper):
+    """Several ragged batches with labels; the same sign occurs in several slots."""
+    rng = np.random.default_rng(dim * 7 + len(opt))
+    pair = Pair(tn, oracle, opt, dim, hyper)
+    vocab = 3000
+    pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)), seed=dim)
+    touched = []
+    sigma = 0.6 if opt == "Ftrl" else 0.01
+    for b in range(4):
+        values = random_batch(rng, 7, 900, vocab)
+        if b == 1:
+            values[3] = values[3][:0]  # an empty slot in the middle
+        counts = check_pull(pair, values)
+        grads = [(rng.standard_normal((int(u), dim)) * sigma).astype(np.float32) for u in counts]
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+        touched.append(all_signs(values))
+        pair.assert_rows_match(np.unique(np.concatenate(touched)))
+    assert tn.core.sparse_table_key_count(pair.h) == pair.o.key_count()
+
+
+def test_cvm_columns(tn, oracle):
+    rng = np.random.default_rng(5)
+    pair = Pair(tn, oracle, "AdaGrad", 8, ADAGRAD_HP, use_cvm=True)
+    assert pair.wf == 10
+    pair.populate(synth.splitmix64(np.arange(1, 501, dtype=np.uint64)))
+    for _ in range(2):
+        values = random_batch(rng, 3, 400, 500)
+        counts = check_pull(pair, values)
+        grads = [(rng.standard_normal((int(u), 10)) * 0.01).astype(np.float32) for u in counts]
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+        pair.assert_rows_match(all_signs(values))
+
+
+def test_extreme_signs_and_single_lookups(tn, oracle):
+    """Signs 0, 2^63 and 2^64-1 (the hash table's own free marker) are ordinary keys."""
+    pair = Pair(tn, oracle, "AdaGrad", 4, ADAGRAD_HP)
+    special = np.asarray([0, 1 << 63, (1 << 64) - 1, 1], dtype=np.uint64)
+    pair.populate(special)
+    values = [special.view(np.int64)[[2, 0, 2, 1, 3, 2]], special.view(np.int64)[[2]], special.view(np.int64)[[0, 0]]]
+    counts = check_pull(pair, values)
+    assert counts.tolist() == [4, 1, 1]
+    grads = [np.full((int(u), 4), 0.5 + i, np.float32) for i, u in enumerate(counts)]
+    labels = [np.ones(len(v), np.int64) for v in values]
+    pair.push_op(values, grads, labels)
+    pair.assert_rows_match(special)
+    (gw, gs, gf), _ = pair.export(special)
+    assert gs[2, 1] == 4.0 and gs[2, 2] == 4.0  # sign 2^64-1: show = 3 + 1, click likewise
+
+
+def test_same_sign_in_many_slots_is_sequential(tn, oracle):
+    """A sign present in k slots gets k Applies, slot 0 first -- not one Apply of the sum."""
+    D, k = 16, 37
+    pair = Pair(tn, oracle, "AdaGrad", D, dict(learning_rate=0.1, initial_g2sum=0.1, epsilon=1e-8))
+    hot = synth.splitmix64(np.asarray([42], dtype=np.uint64))
+    others = synth.splitmix64(np.arange(100, 100 + k, dtype=np.uint64))
+    pair.populate(np.concatenate([hot, others]))
+    values = [np.asarray([others[s], hot[0], others[s], hot[0]], dtype=np.uint64).view(np.int64) for s in range(k)]
+    counts = check_pull(pair, values)
+    rng = np.random.default_rng(0)
+    grads = [(rng.standard_normal((int(u), D)) * 0.3).astype(np.float32) for u in counts]
+    labels = [np.zeros(len(v), np.int64) for v in values]
+    pair.push_op(values, grads, labels)
+    pair.assert_rows_match(np.concatenate([hot, others]))
+    # the summed-gradient shortcut would give a visibly different row
+    ref = oracle.Table(oracle.ADAGRAD, D, buckets=64, learning_rate=0.1, initial_g2sum=0.1, epsilon=1e-8)
+    ref.set_rows(hot, synth.snapshot_rows(hot, D))
+    info = np.zeros(1, dtype=oracle.sign_info_dtype)
+    info["sign"], info["batch_show"] = hot[0], 2 * k
+    ref.push(info, sum(g[1] for g in grads)[None, :])
+    (gw, _, _), _ = pair.export(hot)
+    assert np.abs(gw - ref.get_rows(hot)[0]).max() > 1e-3
+
+
+def test_new_keys_are_inserted_and_initialised(tn, oracle):
+    """Pull of unseen signs inserts rows drawn from N(0, scale/sqrt(D)) (mean / std
+    within 1 %), deterministic in (seed, sign); they then behave like any row."""
+    D, scale = 16, 0.1
+    hp = dict(learning_rate=0.01, initial_g2sum=0.1, initial_scale=scale, epsilon=1e-8)
+    pair = Pair(tn, oracle, "AdaGrad", D, hp, reserve=400000, seed=3)
+    fresh = synth.splitmix64(np.arange(10 ** 6, 10 ** 6 + 60000, dtype=np.uint64))
+    values = [fresh[:40000].view(np.int64), fresh[30000:].view(np.int64)]
+    gvars = [torch.zeros((len(v) + 1, D), device="cuda") for v in values]
+    gm = tn.ops.sparse_table_pull(gvars, [dev(v) for v in values], pair.h)
+    assert tn.core.sparse_table_key_count(pair.h) == 60000
+    assert (gm[0].cpu().numpy() == np.arange(40000)).all()
+    w = torch.cat([gvars[0][:40000], gvars[1][10000:30000]]).cpu().numpy()
+    sigma = scale / np.sqrt(D)
+    assert abs(w.mean()) < 0.01 * sigma
+    assert abs(w.std() / sigma - 1) < 0.01
+    # the same sign pulled through two slots of one call reads one row
+    assert torch.equal(gvars[0][30000:40000], gvars[1][:10000])
+    (gw, gs, gf), _ = pair.export(fresh)
+    assert gf.all() and (gs[:, 0] == np.float32(0.1)).all() and (gs[:, 1:] == 0).all()
+    # deterministic: a second table with the same seed draws the same rows
+    twin = Pair(tn, oracle, "AdaGrad", D, hp, reserve=400000, seed=3)
+    assert torch.equal(tn.ops.table_pull(twin.h, dev(fresh[:1000].view(np.int64)), D), dev(gw[:1000]))
+    # continue on both sides from the GPU's rows
+    pair.o.set_rows(fresh, gw, gs)
+    counts = check_pull(pair, values)
+    grads = synth.make_grads(counts, D, 0.01)
+    pair.push_op(values, grads, [np.zeros(len(v), np.int64) for v in values])
+    pair.assert_rows_match(fresh)
+    # Adam / Ftrl rows start with zero moments
+    for opt, hyper in (("Adam", ADAM_HP), ("Ftrl", FTRL_HP)):
+        p2 = Pair(tn, oracle, opt, 8, dict(hyper, initial_scale=1.0))
+        out = tn.ops.table_pull(p2.h, dev(fresh[:20000].view(np.int64)), 8).cpu().numpy()
+        assert abs(out.std() * np.sqrt(8) - 1) < 0.01 and abs(out.mean()) < 0.01
+        (_, s2, f2), _ = p2.export(fresh[:50])
+        assert f2.all() and (s2 == 0).all()
+    # sparse_zero_init: rows of zeros
+    pz = Pair(tn, oracle, "AdaGrad", 8, ADAGRAD_HP, zero_init=True)
+    assert (tn.ops.table_pull(pz.h, dev(fresh[:100].view(np.int64)), 8) == 0).all()
+
+
+def test_table_level_pull_push_with_repeated_records(tn, oracle):
+    """SparseTable::Pull / Push: request order kept; records applied in array order."""
+    D = 8
+    rng = np.random.default_rng(9)
+    for opt, hyper in (("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP), ("Ftrl", FTRL_HP)):
+        pair = Pair(tn, oracle, opt, D, hyper)
+        base = pair.populate(synth.splitmix64(np.arange(1, 301, dtype=np.uint64)))
+        req = base[rng.integers(0, 300, 1000)]
+        out = tn.ops.table_pull(pair.h, dev(req.view(np.int64)), D).cpu().numpy()
+        assert (out.view(np.int32) == pair.o.pull(req).view(np.int32)).all()
+        infos = np.zeros(1000, dtype=oracle.sign_info_dtype)
+        infos["sign"] = req
+        infos["batch_show"] = rng.integers(1, 5, 1000)
+        infos["batch_click"] = rng.integers(0, 2, 1000)
+        grads = (rng.standard_normal((1000, D)) * (0.5 if opt == "Ftrl" else 0.01)).astype(np.float32)
+        assert pair.o.push(infos, grads) == 0
+        rec = tn.ops.make_sign_infos(dev(req.view(np.int64)), dev(infos["batch_show"].astype(np.int64)),
+                                     dev(infos["batch_click"].astype(np.int64)))
+        tn.ops.table_push(pair.h, rec, dev(grads))
+        tn.ops.sparse_table_sync(pair.h)
+        pair.assert_rows_match(base)
+
+
+def test_errors_come_back_as_codes(tn, oracle):
+    D = 8
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP)
+    signs = pair.populate(synth.splitmix64(np.arange(1, 11, dtype=np.uint64)))
+    v = [dev(signs.view(np.int64))]
+    # U_s must be strictly smaller than the variable's rows (sparse_table_ops.cc:136)
+    with pytest.raises(tn.TensorNetError) as e:
+        tn.ops.sparse_table_pull([torch.zeros((10, D), device="cuda")], v, pair.h)
+    assert e.value.code == 4
+    tn.ops.sparse_table_pull([torch.zeros((11, D), device="cuda")], v, pair.h)
+    # dim mismatch
+    with pytest.raises(tn.TensorNetError) as e:
+        tn.ops.sparse_table_pull([torch.zeros((11, D + 1), device="cuda")], v, pair.h)
+    assert e.value.code == 3
+    # push of a sign that was never pulled (optimizer_kernel.h:315): reported, others applied
+    unknown = np.asarray([123456789], dtype=np.int64)
+    vals = [np.concatenate([signs.view(np.int64)[:3], unknown])]
+    tn.ops.sparse_table_push([dev(vals[0])], [torch.full((4, D), 0.1, device="cuda")],
+                             [torch.zeros(4, dtype=torch.int64, device="cuda")], pair.h)
+    with pytest.raises(tn.TensorNetError) as e:
+        tn.ops.sparse_table_sync(pair.h)
+    assert e.value.code == 5
+    pair.o.push_op([vals[0][:3]], [np.full((3, D), 0.1, np.float32)], [np.zeros(3, np.int64)])
+    pair.assert_rows_match(signs)
+    # bad handle
+    with pytest.raises(tn.TensorNetError) as e:
+        tn.ops.sparse_table_pull([torch.zeros((11, D), device="cuda")], v, 10 ** 6)
+    assert e.value.code == 2
+    # wrong argument kinds are rejected on the host side
+    with pytest.raises(ValueError):
+        tn.ops.sparse_table_pull([torch.zeros((11, D))], v, pair.h)
+    with pytest.raises(ValueError):
+        tn.ops.sparse_table_pull([torch.zeros((11 * D,), device="cuda")], v, pair.h)
+
+
+def test_table_grows_past_its_reservation(tn, oracle):
+    """Load factor 0.75 triggers re-insertion into a larger table (optimizer_kernel.h:266)."""
+    D = 4
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=1000)
+    cap0 = None
+    signs = synth.splitmix64(np.arange(1, 50001, dtype=np.uint64))
+    for lo in range(0, 50000, 5000):
+        pair.populate(signs[lo:lo + 5000], seed=1)
+        cap = tn.core.sparse_table_capacity(pair.h)
+        cap0 = cap0 or cap
+    assert tn.core.sparse_table_capacity(pair.h) > cap0
+    assert tn.core.sparse_table_key_count(pair.h) == 50000
+    assert tn.core.sparse_table_key_count(pair.h) <= 0.75 * tn.core.sparse_table_capacity(pair.h)
+    pair.assert_rows_match(signs, exact=True)
+    # pulls of fresh signs also grow the table
+    fresh = synth.splitmix64(np.arange(10 ** 7, 10 ** 7 + 200000, dtype=np.uint64))
+    tn.ops.table_pull(pair.h, dev(fresh.view(np.int64)), D)
+    assert tn.core.sparse_table_key_count(pair.h) == 250000
+    pair.assert_rows_match(signs, exact=True)
+
+
+def test_cfg2_shape_adam_batches(tn, oracle):
+    """Wide&deep-shaped Adam steps (26 single-hot slots, dim 16), resident set scaled
+    down, some keys new in every batch; state compared after every batch."""
+    cfg = dict(synth.CONFIGS["cfg2"], vocab=2 * 10 ** 5, batch=2048)
+    pair = Pair(tn, oracle, "Adam", 16, cfg["hyper"], reserve=1 << 20)
+    pair.populate(synth.splitmix64(np.arange(1, 10 ** 5 + 1, dtype=np.uint64)))
+    seen = []
+    for b in range(6):
+        values = synth.make_batch(cfg, b)
+        # new keys: let the GPU insert, then mirror its rows into the oracle
+        gv = [torch.zeros((len(v) + 1, 16), device="cuda") for v in values]
+        tn.ops.sparse_table_pull(gv, [dev(v) for v in values], pair.h)
+        signs = all_signs(values)
+        (gw, gs, gf), (_, _, cf) = pair.export(signs)
+        new = ~cf.astype(bool)
+        assert gf.all()
+        if b > 0:
+            assert 0 < new.mean() < 0.2
+        pair.o.set_rows(signs[new], gw[new], gs[new])
+        counts = check_pull(pair, values)
+        grads = synth.make_grads(counts, 16, cfg["grad_sigma"], seed=b)
+        pair.push_op(values, grads, [np.zeros(len(v), np.int64) for v in values])
+        seen.append(signs)
+        pair.assert_rows_match(np.unique(np.concatenate(seen)))
+
+
+def test_cfg4_shape_two_tables_same_signs(tn, oracle):
+    """Insert-heavy mix: dim-1 Ftrl wide weights and dim-64 AdaGrad embeddings share
+    the batch's signs, 20 % of which are fresh."""
+    cfg = dict(synth.CONFIGS["cfg4"], vocab=10 ** 5, batch=1024)
+    wide = Pair(tn, oracle, "Ftrl", 1, dict(learning_rate=0.05, beta=1.0, lambda1=1.0, lambda2=1.0), reserve=1 << 19)
+    deep = Pair(tn, oracle, "AdaGrad", 64, dict(learning_rate=0.01, initial_g2sum=0.1), reserve=1 << 19)
+    resident = synth.splitmix64(np.arange(1, 10 ** 5 + 1, dtype=np.uint64))
+    for pair in (wide, deep):
+        pair.populate(resident)
+    for b in range(2):
+        values = synth.make_batch(cfg, b)
+        signs = all_signs(values)
+        for pair, sigma in ((wide, 0.5), (deep, 1e-2)):
+            gv = [torch.zeros((len(v) + 1, pair.wf), device="cuda") for v in values]
+            tn.ops.sparse_table_pull(gv, [dev(v) for v in values], pair.h)
+            (gw, gs, gf), (_, _, cf) = pair.export(signs)
+            new = ~cf.astype(bool)
+            assert 0.1 < new.mean() < 0.5
+            pair.o.set_rows(signs[new], gw[new], gs[new])
+            counts = check_pull(pair, values)
+            grads = synth.make_grads(counts, pair.wf, sigma, seed=b)
+            pair.push_op(values, grads, [np.zeros(len(v), np.int64) for v in values])
+            pair.assert_rows_match(signs)
+
+
+def test_full_size_batch_properties(tn, oracle):
+    """cfg3's full batch (16384 x 100 slots, ~5 M lookups) cannot go through the CPU
+    oracle in seconds; check size-independent properties instead, on the GPU:
+    ids of equal signs agree, ids are dense and in first-occurrence order, the
+    variable row of every lookup is the row of its sign, pull is idempotent, and a
+    push changes exactly the pulled rows."""
+    cfg = synth.CONFIGS["cfg3"]
+    D = cfg["dim"]
+    opt = tn.core.AdaGrad(**cfg["hyper"])
+    h = tn.core.create_sparse_table(opt, "", D, False, "")
+    tn.core.reserve_sparse_table(h, 6 * 10 ** 6)
+    values = synth.make_batch(cfg, 0)
+    L = sum(len(v) for v in values)
+    assert 4.5e6 < L < 5.5e6
+    gvalues = [dev(v) for v in values]
+    uniq = torch.unique(torch.cat(gvalues))
+    w0 = synth.snapshot_rows_torch(uniq, D)
+    tn.ops.table_load_rows(h, uniq, w0)
+    assert tn.core.sparse_table_key_count(h) == uniq.numel()
+    rows = [len(v) + 1 for v in values]
+    gvars = [torch.full((r, D), 9.0, device="cuda") for r in rows]
+    mapped = tn.ops.sparse_table_pull(gvars, gvalues, h)
+    counts = tn.ops.sparse_table_last_unique_counts(h, len(values))
+    for s in (0, 1, 17, 50, 99):
+        v, m = gvalues[s], mapped[s]
+        u, inv = torch.unique(v, return_inverse=True)
+        assert counts[s] == u.numel() == int(m.max()) + 1
+        # first-occurrence order: position of first occurrence increases with the id
+        first = torch.full((u.numel(),), len(v), dtype=torch.int64, device="cuda")
+        first.scatter_reduce_(0, inv, torch.arange(len(v), device="cuda"), reduce="amin")
+        first_by_id = torch.empty_like(first)
+        first_by_id[m[first]] = first
+        assert bool((first_by_id[1:] > first_by_id[:-1]).all())
+        assert torch.equal(m, m[first][inv])  # equal signs <=> equal ids
+        # the row a lookup maps to is its sign's snapshot row
+        assert torch.equal(gvars[s][m], synth.snapshot_rows_torch(v, D))
+        assert bool((gvars[s][counts[s]:] == 9.0).all())
+    # idempotent
+    gvars2 = [torch.full((r, D), 9.0, device="cuda") for r in rows]
+    mapped2 = tn.ops.sparse_table_pull(gvars2, gvalues, h)
+    assert all(torch.equal(a, b) for a, b in zip(mapped, mapped2))
+    assert all(torch.equal(a, b) for a, b in zip(gvars, gvars2))
+    # push with zero gradients: weights unchanged, show counts add up to L
+    grads = [torch.zeros((c, D), device="cuda") for c in counts]
+    labels = [torch.zeros_like(v) for v in gvalues]
+    tn.ops.sparse_table_push(gvalues, grads, labels, h)
+    tn.ops.sparse_table_sync(h)
+    w1, st1, found = tn.ops.table_export_rows(h, uniq)
+    assert bool(found.all()) and torch.equal(w1, w0)
+    assert float(st1[:, 1].sum()) == float(L) and bool((st1[:, 0] == 0.1).all())
+    # push with a constant gradient g: a key present in k slots gets k sequential Applies,
+    # each adding g^2 to g2sum and moving every weight by -lr*g/sqrt(g2sum)
+    g = 0.5
+    grads = [torch.full((c, D), g, device="cuda") for c in counts]
+    tn.ops.sparse_table_push(gvalues, grads, labels, h)
+    tn.ops.sparse_table_sync(h)
+    w2, st2, _ = tn.ops.table_export_rows(h, uniq)
+    k = torch.zeros(uniq.numel(), device="cuda")
+    for v in gvalues:
+        k[torch.searchsorted(uniq, torch.unique(v))] += 1
+    assert float(k.sum()) == float(sum(counts))
+    np.testing.assert_allclose(st2[:, 0].cpu().numpy(), (0.1 + k * g * g).cpu().numpy(), rtol=1e-5)
+    kmax = int(k.max())
+    steps = torch.arange(1, kmax + 1, device="cuda", dtype=torch.float64)
+    cum = torch.cumsum(0.01 * g / torch.sqrt(0.1 + steps * g * g), 0)
+    expect = w0.double() - cum[(k - 1).long()][:, None]
+    np.testing.assert_allclose(w2.cpu().numpy(), expect.cpu().numpy(), rtol=RTOL, atol=1e-6)
