@@ -1,0 +1,318 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse pull + push hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--resident KEYS] [--config cfg3]
+
+A step is one SparseTablePull followed by one SparseTablePush over one seeded
+synthetic batch whose inputs (signs, labels, gradients) and outputs (mapped
+ids, variables) are already resident in HBM.  The default workload is the one
+the headline metric is quoted on: dim-16 AdaGrad, batch 16384 x 100 slots with
+Poisson(3) id lists (~5 M lookups), Zipf(1.1) signs over a 1e9 vocabulary and
+5e8 resident keys.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def state_bytes(opt, dim):
+    """Optimizer state bytes read+written per applied row (beyond w and the gradient)."""
+    return 28 if opt == "AdaGrad" else 16 * dim + 8
+
+
+def step_algorithmic_bytes(opt, dim, L, U):
+    """Bytes one pull + one push must move, counting each datum once:
+    pull = 8L (signs) + 8L (mapped ids) + U*(8 key + 4D row + 4D var);
+    push = 8L (signs) + 8L (labels) + U*(4D grad + 8 key + 8D w r/w + state)."""
+    return 32 * L + U * (8 + 8 * dim + 4 * dim + 8 + 8 * dim + state_bytes(opt, dim))
+
+
+def kernel_algorithmic_bytes(name, opt, dim, L, U, G):
+    """Algorithmic bytes of one launch of each kernel of the step (L lookups, U
+    per-slot distinct signs, G distinct signs of the whole push)."""
+    row = 4 * dim
+    table = {
+        "k_fill_ff": 0,
+        "k_remap_insert": 8 * L,                      # reads every sign once
+        "k_flag_count": 0,
+        "k_scan_tiles": 0,
+        "k_assign_rank": 8 * U,                       # writes the distinct sign lists
+        "k_write_mapped": 8 * L,                      # writes every mapped id
+        "k_count_show": 8 * L,                        # reads every label
+        "k_probe<true>": 8 * U,                       # one stored-key compare per row
+        "k_probe<false>": 8 * G,
+        "k_init_rows": 0,
+        "k_finish_insert": 0,
+        "k_gather_vars<4>": U * 2 * row,              # row read + variable row write
+        "k_gather_vars<1>": U * 2 * row,
+        "k_fill_groups": 0,
+        "k_group_insert": 8 * U,
+        "k_group_compact": 0,
+        "k_group_fill": 0,
+    }
+    if name.startswith("k_apply"):
+        return U * row + G * (2 * row + state_bytes(opt, dim))
+    return table.get(name, 0)
+
+
+def populate(tn, handle, resident, dim, chunk=1 << 23):
+    """Loads splitmix64(1..resident) with the synthetic snapshot rows, in chunks."""
+    import torch
+
+    from tensornet_amd import synth
+
+    t0 = time.time()
+    for lo in range(1, resident + 1, chunk):
+        hi = min(resident + 1, lo + chunk)
+        ids = torch.arange(lo, hi, dtype=torch.int64, device="cuda")
+        signs = synth.splitmix64_torch(ids)
+        w = synth.snapshot_rows_torch(signs, dim)
+        tn.ops.table_load_rows(handle, signs, w)
+        del ids, signs, w
+    torch.cuda.synchronize()
+    log("populated %d keys in %.1f s" % (resident, time.time() - t0))
+
+
+def cpu_baseline(cfg, values, grads_sigma):
+    """Times the CPU oracle (the reference's data structures, one thread) on one
+    full batch: pull op then push op.  The CPU table only holds the keys the batch
+    touches (the host cannot hold the full resident set)."""
+    import numpy as np
+
+    from oracle import cpu as oracle
+    from tensornet_amd import synth
+
+    kinds = {"AdaGrad": oracle.ADAGRAD, "Adam": oracle.ADAM, "Ftrl": oracle.FTRL}
+    dim = cfg["dim"]
+    t = oracle.Table(kinds[cfg["opt"]], dim, buckets=15485863, **cfg["hyper"])
+    signs = np.unique(np.concatenate(values).view(np.uint64))
+    t.set_rows(signs, synth.snapshot_rows(signs, dim))
+    L = sum(len(v) for v in values)
+    vars_ = [np.zeros((len(v) + 1, dim), np.float32) for v in values]
+    t0 = time.perf_counter()
+    rc, mapped, counts = t.pull_op(values, vars_)
+    t1 = time.perf_counter()
+    assert rc == 0
+    grads = synth.make_grads(counts, dim, grads_sigma)
+    labels = [np.zeros(len(v), np.int64) for v in values]
+    t2 = time.perf_counter()
+    rc, _ = t.push_op(values, grads, labels)
+    t3 = time.perf_counter()
+    assert rc == 0
+    secs = (t1 - t0) + (t3 - t2)
+    log("cpu baseline: pull %.2f s, push %.2f s, %d lookups, %d rows" % (t1 - t0, t3 - t2, L, int(counts.sum())))
+    return {
+        "value": L / secs,
+        "unit": "keys/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "1 full batch (%d lookups, %d per-slot distinct rows), pull op + push op, CPU table "
+                  "pre-populated with only the %d keys the batch touches" % (L, int(counts.sum()), len(signs)),
+        "pull_s": t1 - t0,
+        "push_s": t3 - t2,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg3")
+    ap.add_argument("--resident", type=int, default=None, help="resident keys (default: the config's)")
+    ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated batches cycled through")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
+              "(every box has one GPU, nothing here uses collectives)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import tensornet_amd as tn
+    from tensornet_amd import _lib, synth
+
+    tn.load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    import tensornet_amd.ops  # noqa: F401
+
+    torch.cuda.set_device(0)
+    cfg = synth.CONFIGS[args.config]
+    dim, opt_name = cfg["dim"], cfg["opt"]
+    resident = args.resident if args.resident is not None else cfg["resident"]
+
+    opt = getattr(tn.core, opt_name)(**cfg["hyper"])
+    h = tn.core.create_sparse_table(opt, "bench", dim, False, "")
+    tn.core.reserve_sparse_table(h, int(resident * 1.02) + 16 * 1024 * 1024)
+    populate(tn, h, resident, dim)
+
+    # ---- inputs, resident in HBM -------------------------------------------------
+    nb = max(1, args.batches)
+    host_batches = [synth.make_batch(cfg, b) for b in range(nb)]
+    batches = []
+    rng = torch.Generator(device="cuda")
+    rng.manual_seed(0)
+    for hb in host_batches:
+        values = [torch.from_numpy(v).cuda() for v in hb]
+        labels = [torch.zeros_like(v) for v in values]
+        # gradient matrices have one row per possible distinct sign; the op reads the first U_s
+        grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
+        vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
+        batches.append((values, labels, grads, vars_))
+    L = sum(len(v) for v in host_batches[0])
+    n_slots = len(host_batches[0])
+
+    def step(i):
+        values, labels, grads, vars_ = batches[i % nb]
+        tn.ops.sparse_table_pull(vars_, values, h)
+        tn.ops.sparse_table_push(values, grads, labels, h)
+
+    for i in range(args.warmup):
+        step(i)
+    tn.ops.sparse_table_sync(h)
+    torch.cuda.synchronize()
+    # per-batch sizes (U from the last pull of each batch; G measured once below)
+    Ls, Us = [], []
+    for i in range(nb):
+        values, labels, grads, vars_ = batches[i]
+        tn.ops.sparse_table_pull(vars_, values, h)
+        Us.append(sum(tn.ops.sparse_table_last_unique_counts(h, n_slots)))
+        Ls.append(sum(v.numel() for v in values))
+    G0 = int(torch.unique(torch.cat(batches[0][0])).numel())
+    torch.cuda.synchronize()
+
+    # ---- timed region ------------------------------------------------------------
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(args.steps):
+        step(i)
+    ev1.record()
+    tn.ops.sparse_table_sync(h)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    total_L = sum(Ls[i % nb] for i in range(args.steps))
+    total_U = sum(Us[i % nb] for i in range(args.steps))
+    value = total_L / wall
+    alg = step_algorithmic_bytes(opt_name, dim, total_L, total_U)
+    log("timed %d steps: %.3f ms/step (events %.3f ms/step), %.3e keys/s" %
+        (args.steps, ms_per_step, ev0.elapsed_time(ev1) / args.steps, value))
+
+    # ---- per-kernel durations, HIP events around every launch --------------------
+    lib = tn.load()
+    lib.tn_profile_reset()
+    lib.tn_profile_enable(1)
+    psteps = min(args.steps, 10)
+    for i in range(psteps):
+        step(i)
+    tn.ops.sparse_table_sync(h)
+    torch.cuda.synchronize()
+    lib.tn_profile_enable(0)
+    prof = _lib.profile_summary()
+    lib.tn_profile_reset()
+    per_step = {k: (c / psteps, ms / psteps) for k, (c, ms) in prof.items()}
+    kernel_ms = sum(ms for _, ms in per_step.values())
+    dominant = max(per_step.items(), key=lambda kv: kv[1][1])
+    dname, (dcount, dms) = dominant
+    avg_launch_s = dms / dcount * 1e-3
+    mean_L, mean_U = total_L / args.steps, total_U / args.steps
+    dbytes = kernel_algorithmic_bytes(dname, opt_name, dim, mean_L, mean_U, G0)
+    achieved = dbytes / avg_launch_s
+    for k, (c, ms) in sorted(per_step.items(), key=lambda kv: -kv[1][1]):
+        log("  %-28s %5.1f launches/step %9.3f ms/step" % (k, c, ms))
+    log("  sum of kernel time %.3f ms/step" % kernel_ms)
+
+    out = {
+        "metric": "sparse pull+push keys/sec (dim16 AdaGrad); achieved HBM GB/s vs ~8 TB/s peak",
+        "value": value,
+        "unit": "keys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: batch %d x %d slots, %s id lists, Zipf(%.2f) over %.0e vocab, dim %d %s, %d resident keys"
+                        % (args.config, cfg["batch"], cfg["slots"], cfg["lens"], cfg["zipf_s"], cfg["vocab"], dim,
+                           opt_name, resident),
+            "lookups_per_step": mean_L,
+            "distinct_rows_per_step": mean_U,
+            "globally_distinct_keys_batch0": G0,
+            "distinct_batches": nb,
+        },
+        "rows_per_s": total_U / wall,
+        "step_algorithmic_GBps": alg / wall / 1e9,
+        "step_frac_of_hbm_peak": alg / wall / HBM_PEAK,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dname,
+            "achieved": achieved / 1e9,
+            "peak": HBM_PEAK / 1e9,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK,
+            "traffic": None,
+            "avg_launch_us": avg_launch_s * 1e6,
+            "algorithmic_bytes_per_launch": dbytes,
+        },
+        "kernels_ms_per_step": {k: round(ms, 4) for k, (c, ms) in per_step.items()},
+    }
+
+    # ---- dense Adam side measurement (cfg5's flat array) --------------------------
+    if not args.no_dense:
+        total = synth.CONFIGS["cfg5"]["dense_total"]
+        dh = tn.core.create_dense_table(tn.core.Adam(learning_rate=1e-3, beta1=0.9, beta2=0.999))
+        w = (torch.rand(total, device="cuda") - 0.5) * 0.1
+        g = torch.randn(total, device="cuda") * 1e-4
+        tn.ops.dense_table_init([w], dh)
+        for _ in range(3):
+            tn.ops.dense_table_push_pull([w], [g], 1e-3, dh)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            tn.ops.dense_table_push_pull([w], [g], 1e-3, dh)
+        e1.record()
+        torch.cuda.synchronize()
+        dsec = e0.elapsed_time(e1) / 20 * 1e-3
+        out["dense_adam"] = {
+            "params": total,
+            "ms_per_step": dsec * 1e3,
+            "algorithmic_GBps": 28 * total / dsec / 1e9,  # read g,w,m,v ; write w,m,v
+            "frac_of_hbm_peak": 28 * total / dsec / HBM_PEAK,
+        }
+        del w, g
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(cfg, host_batches[0], cfg["grad_sigma"])
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -269,6 +269,19 @@ int tn_dense_table_set_weight(uint32_t handle, const float* w, void* stream);
 /* Optimizer state read-back for tests: Adam m,v ; AdaGrad d2sum,g2sum,m (device, total floats each; NULL skips). */
 int tn_dense_table_get_state(uint32_t handle, float* s0, float* s1, float* s2, void* stream);
 
+/* --------------------------------------------------------------- profiling */
+/*
+ * Measurement hooks with no counterpart in the reference (which instruments
+ * nothing on this path).  While enabled, every kernel launch of the library is
+ * bracketed by two HIP events on the stream it is launched on.
+ * tn_profile_summary waits for the recorded events and writes one line per
+ * kernel name, "name<TAB>launches<TAB>total_ms", into buf (NUL-terminated).
+ * tn_profile_reset drops the records.
+ */
+int tn_profile_enable(int on);
+int tn_profile_reset(void);
+int tn_profile_summary(char* buf, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -119,6 +119,9 @@ SIGNATURES = {
     "tn_dense_table_get_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_set_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_get_state": (C.c_int, [C.c_uint32, _P, _P, _P, _P]),
+    "tn_profile_enable": (C.c_int, [C.c_int]),
+    "tn_profile_reset": (C.c_int, []),
+    "tn_profile_summary": (C.c_int, [C.c_char_p, C.c_size_t]),
 }
 
 _lib = None
@@ -160,3 +163,14 @@ def i64_array(vals):
     for i, v in enumerate(vals):
         arr[i] = int(v)
     return arr
+
+
+def profile_summary():
+    """{kernel name: (launches, total milliseconds)} of the launches recorded since the last reset."""
+    buf = C.create_string_buffer(1 << 16)
+    check(load().tn_profile_summary(buf, len(buf)))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, ms = line.split("\t")
+        out[name.strip("()")] = (int(count), float(ms))
+    return out

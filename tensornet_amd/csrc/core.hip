@@ -4,6 +4,8 @@
 // (py_wrapper.cc:112).
 #include "tn_common.h"
 
+#include <cstring>
+
 namespace tn {
 
 namespace {
@@ -49,6 +51,41 @@ int DevBuf::ensure(size_t need) {
     return TN_OK;
 }
 
+// ---------------------------------------------------------------- profiling
+bool g_profile_on = false;
+namespace {
+struct ProfRec {
+    const char* name;
+    hipEvent_t a, b;
+};
+std::mutex g_prof_mu;
+std::vector<ProfRec> g_prof_recs;
+std::vector<hipEvent_t> g_prof_pool;
+
+hipEvent_t prof_event() {
+    if (!g_prof_pool.empty()) {
+        hipEvent_t e = g_prof_pool.back();
+        g_prof_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+}  // namespace
+
+void prof_begin(const char* name, hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfRec r{name, prof_event(), prof_event()};
+    (void)hipEventRecord(r.a, st);
+    g_prof_recs.push_back(r);
+}
+
+void prof_end(hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().b, st);
+}
+
 void DevBuf::release() {
     if (p) (void)hipFree(p);
     p = nullptr;
@@ -64,6 +101,57 @@ extern "C" {
 const char* tn_last_error(void) { return t_last_error.c_str(); }
 
 const char* tn_version(void) { return "tensornet_amd 0.1 (gfx950)"; }
+
+int tn_profile_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_profile_on = on != 0;
+    return TN_OK;
+}
+
+int tn_profile_reset(void) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    for (auto& r : g_prof_recs) {
+        (void)hipEventSynchronize(r.b);
+        g_prof_pool.push_back(r.a);
+        g_prof_pool.push_back(r.b);
+    }
+    g_prof_recs.clear();
+    return TN_OK;
+}
+
+int tn_profile_summary(char* buf, size_t cap) {
+    if (!buf || cap == 0) return fail(TN_ERR_INVALID_ARGUMENT, "tn_profile_summary: no buffer");
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    struct Acc {
+        const char* name;
+        long count;
+        double ms;
+    };
+    std::vector<Acc> acc;
+    for (auto& r : g_prof_recs) {
+        TN_HIP(hipEventSynchronize(r.b));
+        float ms = 0.f;
+        TN_HIP(hipEventElapsedTime(&ms, r.a, r.b));
+        bool hit = false;
+        for (auto& a : acc)
+            if (std::string(a.name) == r.name) {
+                a.count++;
+                a.ms += ms;
+                hit = true;
+                break;
+            }
+        if (!hit) acc.push_back(Acc{r.name, 1, ms});
+    }
+    std::string out;
+    for (auto& a : acc) {
+        char line[256];
+        snprintf(line, sizeof(line), "%s\t%ld\t%.6f\n", a.name, a.count, a.ms);
+        out += line;
+    }
+    if (out.size() + 1 > cap) return fail(TN_ERR_INVALID_ARGUMENT, "tn_profile_summary: buffer too small");
+    memcpy(buf, out.c_str(), out.size() + 1);
+    return TN_OK;
+}
 
 void tn_adagrad_params_default(tn_adagrad_params* p) {
     if (!p) return;

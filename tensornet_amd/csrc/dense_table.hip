@@ -166,14 +166,14 @@ static int dense_alloc(DenseTable* t, int64_t total, hipStream_t st) {
     TN_HIP(hipMalloc((void**)&t->s0, bytes));
     TN_HIP(hipMalloc((void**)&t->s1, bytes));
     int blocks = launch_grid(total, 256, 8192);
-    hipLaunchKernelGGL(k_fill_f32, dim3(blocks), dim3(256), 0, st, t->w, total, 0.f);
-    hipLaunchKernelGGL(k_fill_f32, dim3(blocks), dim3(256), 0, st, t->s0, total, 0.f);
+    TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->w, total, 0.f);
+    TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s0, total, 0.f);
     if (t->opt->kind == OPT_ADAGRAD) {
         TN_HIP(hipMalloc((void**)&t->s2, bytes));
-        hipLaunchKernelGGL(k_fill_f32, dim3(blocks), dim3(256), 0, st, t->s1, total, t->opt->initial_g2sum);
-        hipLaunchKernelGGL(k_fill_f32, dim3(blocks), dim3(256), 0, st, t->s2, total, 0.f);
+        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, total, t->opt->initial_g2sum);
+        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s2, total, 0.f);
     } else {
-        hipLaunchKernelGGL(k_fill_f32, dim3(blocks), dim3(256), 0, st, t->s1, total, 0.f);
+        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, total, 0.f);
     }
     TN_HIP(hipGetLastError());
     t->total = total;
@@ -252,20 +252,16 @@ int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const f
             int64_t n4 = vec ? n / 4 : 0;
             if (n4 > 0) {
                 int blocks = launch_grid(n4, 256, 1 << 20);
-                hipLaunchKernelGGL(k_dense_adam_v4, dim3(blocks), dim3(256), 0, st, (const float4*)g,
-                                   (float4*)(t->w + off), (float4*)(t->s0 + off), (float4*)(t->s1 + off),
-                                   (float4*)out, n4, aa);
+                TN_LAUNCH(k_dense_adam_v4, dim3(blocks), dim3(256), st, (const float4*)g, (float4*)(t->w + off), (float4*)(t->s0 + off), (float4*)(t->s1 + off), (float4*)out, n4, aa);
             }
             int64_t done = n4 * 4;
             if (done < n) {
                 int blocks = launch_grid(n - done, 256, 1 << 20);
-                hipLaunchKernelGGL(k_dense_adam_s, dim3(blocks), dim3(256), 0, st, g + done, t->w + off + done,
-                                   t->s0 + off + done, t->s1 + off + done, out ? out + done : nullptr, n - done, aa);
+                TN_LAUNCH(k_dense_adam_s, dim3(blocks), dim3(256), st, g + done, t->w + off + done, t->s0 + off + done, t->s1 + off + done, out ? out + done : nullptr, n - done, aa);
             }
         } else {
             int blocks = launch_grid(n, 256, 1 << 20);
-            hipLaunchKernelGGL(k_dense_adagrad_s, dim3(blocks), dim3(256), 0, st, g, t->w + off, t->s0 + off,
-                               t->s1 + off, t->s2 + off, out, n, ga);
+            TN_LAUNCH(k_dense_adagrad_s, dim3(blocks), dim3(256), st, g, t->w + off, t->s0 + off, t->s1 + off, t->s2 + off, out, n, ga);
         }
         off += n;
     }

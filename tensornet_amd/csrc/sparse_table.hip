@@ -229,9 +229,8 @@ int grow_to(SparseTable* t, uint64_t cap, hipStream_t st) {
         free_store(bigger);
         return rc;
     }
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
-    hipLaunchKernelGGL(k_rehash, dim3(launch_grid((int64_t)s.cap + 1, 256, GRID_CAP * 4)), dim3(256), 0, st, s, bigger,
-                       t->dstatus);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
+    TN_LAUNCH(k_rehash, dim3(launch_grid((int64_t)s.cap + 1, 256, GRID_CAP * 4)), dim3(256), st, s, bigger, t->dstatus);
     TN_HIP(hipMemcpyAsync(bigger.count, s.count, sizeof(unsigned long long), hipMemcpyDeviceToDevice, st));
     TN_HIP(hipStreamSynchronize(st));
     free_store(s);
@@ -398,16 +397,11 @@ int upload_slots(SparseTable* t, const OpScratch& w, const std::vector<SlotDesc>
 
 // Remap steps 1-4 shared by pull and push (k_remap_insert .. k_assign_rank).
 void launch_remap(const OpScratch& w, int N, uint32_t L, DevStatus* dstatus, hipStream_t st) {
-    hipLaunchKernelGGL(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), 0, st,
-                       reinterpret_cast<uint4*>(w.dt), w.dt_entries);
-    hipLaunchKernelGGL(k_remap_insert, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase, N, L,
-                       w.dt, w.tidx);
-    hipLaunchKernelGGL(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), 0, st, w.lbase, N, L, w.dt, w.tidx, w.flag8,
-                       w.tilesum);
-    hipLaunchKernelGGL(k_scan_tiles, dim3(1), dim3(1024), 0, st, w.tilesum, w.tileoff, w.ntiles, w.lbase, w.ubase, N, L,
-                       dstatus);
-    hipLaunchKernelGGL(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), 0, st, w.descs, w.lbase, N, L, w.dt, w.tidx,
-                       w.flag8, w.tileoff, w.ubase, w.uniq_sign, w.uniq_slot, w.ushow, w.uclick);
+    TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st, reinterpret_cast<uint4*>(w.dt), w.dt_entries);
+    TN_LAUNCH(k_remap_insert, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, N, L, w.dt, w.tidx);
+    TN_LAUNCH(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), st, w.lbase, N, L, w.dt, w.tidx, w.flag8, w.tilesum);
+    TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, w.lbase, w.ubase, N, L, dstatus);
+    TN_LAUNCH(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), st, w.descs, w.lbase, N, L, w.dt, w.tidx, w.flag8, w.tileoff, w.ubase, w.uniq_sign, w.uniq_slot, w.ushow, w.uclick);
 }
 
 template <int KIND>
@@ -415,7 +409,7 @@ void launch_apply_kind(int lpg, int blocks_hint, const Store& s, const OptDev& o
                        DevStatus* dstatus, const OpScratch& w, int64_t n_upper, hipStream_t st) {
     (void)blocks_hint;
 #define TN_LAUNCH_VEC(LPG)                                                                                            \
-    hipLaunchKernelGGL((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 2)), dim3(256), 0, st, \
+    TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 2)), dim3(256), st, \
                        s, o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list)
     switch (lpg) {
         case 1: TN_LAUNCH_VEC(1); break;
@@ -425,8 +419,7 @@ void launch_apply_kind(int lpg, int blocks_hint, const Store& s, const OptDev& o
         case 16: TN_LAUNCH_VEC(16); break;
         case 32: TN_LAUNCH_VEC(32); break;
         default:
-            hipLaunchKernelGGL((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), 0, st, s,
-                               o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list);
+            TN_LAUNCH((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, s, o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list);
     }
 #undef TN_LAUNCH_VEC
 }
@@ -440,13 +433,11 @@ void launch_push_tail(SparseTable* t, const OpScratch& w, const PushSrc& src, in
     DevStatus* ds = t->dstatus;
     const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
     const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
-    hipLaunchKernelGGL(k_fill_groups, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), 0, st, w.gt, ds);
-    hipLaunchKernelGGL(k_group_insert, dim3(gblocks), dim3(256), 0, st, src, n_host, ds, w.gt, w.gidx, w.ord);
-    hipLaunchKernelGGL(k_group_compact, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), 0, st, ds,
-                       w.gt, w.grp_sign, w.grp_off, w.grp_cnt);
-    hipLaunchKernelGGL(k_group_fill, dim3(gblocks), dim3(256), 0, st, n_host, n_dev, w.gt, w.gidx, w.ord, w.list);
-    hipLaunchKernelGGL((k_probe<false>), dim3(gblocks), dim3(256), 0, st, s, w.grp_sign, (int64_t)0, &ds->n_groups,
-                       w.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+    TN_LAUNCH(k_fill_groups, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), st, w.gt, ds);
+    TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, w.gt, w.gidx, w.ord);
+    TN_LAUNCH(k_group_compact, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), st, ds, w.gt, w.grp_sign, w.grp_off, w.grp_cnt);
+    TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, w.gidx, w.ord, w.list);
+    TN_LAUNCH((k_probe<false>), dim3(gblocks), dim3(256), st, s, w.grp_sign, (int64_t)0, &ds->n_groups, w.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
     int lpg = 0;
     if (vec_ok && s.D % 4 == 0) {
         int q = s.D / 4;
@@ -617,17 +608,14 @@ int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int 
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     const int blocks = launch_grid(n, 256, GRID_CAP * 2);
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, 0u);
-    hipLaunchKernelGGL((k_probe<true>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
-                       newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
-    hipLaunchKernelGGL(k_init_rows, dim3(blocks), dim3(256), 0, st, s, o, t->seed, signs, rows, newlist, t->dstatus);
-    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH(k_init_rows, dim3(blocks), dim3(256), st, s, o, t->seed, signs, rows, newlist, t->dstatus);
+    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     if (wdim % 4 == 0 && s.wstride % 4 == 0 && aligned16(out))
-        hipLaunchKernelGGL((k_gather_rows<4>), dim3(launch_grid(n * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), 0, st, s,
-                           rows, n, out);
+        TN_LAUNCH((k_gather_rows<4>), dim3(launch_grid(n * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, rows, n, out);
     else
-        hipLaunchKernelGGL((k_gather_rows<1>), dim3(launch_grid(n * wdim, 256, GRID_CAP * 4)), dim3(256), 0, st, s, rows,
-                           n, out);
+        TN_LAUNCH((k_gather_rows<1>), dim3(launch_grid(n * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, rows, n, out);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->hpull->ubase[0] = 0;
@@ -669,7 +657,7 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
     src.grads = grads;
     src.dim = dim;
     const uint32_t gcap = (uint32_t)std::max<int64_t>(16, 2 * n);
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, gcap);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, gcap);
     launch_push_tail(t, w, src, n, n, aligned16(grads) && dim % 4 == 0, st);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
@@ -700,11 +688,10 @@ int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const floa
     uint32_t* newlist = c.take<uint32_t>(n);
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, (uint32_t)n, 0u);
-    hipLaunchKernelGGL((k_probe<true>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
-                       newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
-    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
-    hipLaunchKernelGGL(k_load_rows, dim3(blocks), dim3(256), 0, st, s, make_optdev(t), rows, n, w, state);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
+    TN_LAUNCH(k_load_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->pull_pending = true;
@@ -732,9 +719,8 @@ int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t 
     uint32_t* rows = (uint32_t*)t->ws.p;
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
-    hipLaunchKernelGGL((k_probe<false>), dim3(blocks), dim3(256), 0, st, s, signs, n, (const uint32_t*)nullptr, rows,
-                       (uint32_t*)nullptr, t->dstatus, 0u);
-    hipLaunchKernelGGL(k_export_rows, dim3(blocks), dim3(256), 0, st, s, make_optdev(t), rows, n, w, state, found);
+    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, (uint32_t*)nullptr, t->dstatus, 0u);
+    TN_LAUNCH(k_export_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state, found);
     TN_HIP(hipGetLastError());
     TN_HIP(hipStreamSynchronize(st));
     return TN_OK;
@@ -786,22 +772,17 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
 
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
     launch_remap(w, N, (uint32_t)L, t->dstatus, st);
-    hipLaunchKernelGGL(k_write_mapped, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase,
-                       w.ubase, N, (uint32_t)L, w.dt, w.tidx);
+    TN_LAUNCH(k_write_mapped, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, w.ubase, N, (uint32_t)L, w.dt, w.tidx);
     const int ublocks = launch_grid(L, 256, GRID_CAP * 2);
-    hipLaunchKernelGGL((k_probe<true>), dim3(ublocks), dim3(256), 0, st, s, w.uniq_sign, (int64_t)0,
-                       &t->dstatus->n_unique, w.rows, w.newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
-    hipLaunchKernelGGL(k_init_rows, dim3(ublocks), dim3(256), 0, st, s, o, t->seed, w.uniq_sign, w.rows, w.newlist,
-                       t->dstatus);
-    hipLaunchKernelGGL(k_finish_insert, dim3(1), dim3(64), 0, st, s, t->dstatus);
+    TN_LAUNCH((k_probe<true>), dim3(ublocks), dim3(256), st, s, w.uniq_sign, (int64_t)0, &t->dstatus->n_unique, w.rows, w.newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH(k_init_rows, dim3(ublocks), dim3(256), st, s, o, t->seed, w.uniq_sign, w.rows, w.newlist, t->dstatus);
+    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     if (vec)
-        hipLaunchKernelGGL((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), 0,
-                           st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+        TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
     else
-        hipLaunchKernelGGL((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), 0, st,
-                           s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+        TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     TN_HIP(hipMemcpyAsync(t->hpull->ubase, w.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
@@ -851,10 +832,9 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     carve_op((char*)t->ws.p, w, N, L, dt_entries, true);
     TN_TRY(upload_slots(t, w, descs, lbase, st));
 
-    hipLaunchKernelGGL(k_reset_status, dim3(1), dim3(64), 0, st, t->dstatus, 0u, 0u);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
     launch_remap(w, N, (uint32_t)L, t->dstatus, st);
-    hipLaunchKernelGGL(k_count_show, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), 0, st, w.descs, w.lbase, N,
-                       (uint32_t)L, w.dt, w.tidx, w.ushow, w.uclick);
+    TN_LAUNCH(k_count_show, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, N, (uint32_t)L, w.dt, w.tidx, w.ushow, w.uclick);
     PushSrc src{};
     src.uniq_sign = w.uniq_sign;
     src.uniq_slot = w.uniq_slot;

@@ -118,6 +118,21 @@ struct DevBuf {
 
 int launch_grid(int64_t work_items, int threads, int max_blocks);
 
+// ---------------------------------------------------------------- profiling
+// When enabled (tn_profile_enable) every kernel launch is bracketed by a pair
+// of HIP events on the stream it is launched on; tn_profile_summary adds the
+// elapsed times up per kernel name.
+extern bool g_profile_on;
+void prof_begin(const char* name, hipStream_t st);
+void prof_end(hipStream_t st);
+
+#define TN_LAUNCH(KERNEL, GRID, BLOCK, STREAM, ...)                            \
+    do {                                                                       \
+        if (::tn::g_profile_on) ::tn::prof_begin(#KERNEL, STREAM);             \
+        hipLaunchKernelGGL(KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__);       \
+        if (::tn::g_profile_on) ::tn::prof_end(STREAM);                        \
+    } while (0)
+
 }  // namespace tn
 
 #endif  // TN_COMMON_H_

@@ -25,12 +25,18 @@ def random_batch(rng, slots, max_len, vocab, ragged=True):
     return out
 
 
-def check_pull(pair, values, var_rows=None):
+def check_pull(pair, values, var_rows=None, loose_col=None):
+    """loose_col: a column compared with the update tolerance instead of bit for bit
+    (the cvm log column, whose value depends on the libm in use)."""
     gm, gv, cm, cv, counts = pair.pull_op(values, var_rows)
     for s in range(len(values)):
         assert (gm[s].cpu().numpy() == cm[s]).all(), "mapped ids of slot %d" % s
+        g, c = gv[s].cpu().numpy(), cv[s]
+        if loose_col is not None:
+            np.testing.assert_allclose(g[:, loose_col], c[:, loose_col], rtol=RTOL, atol=ATOL)
+            g, c = np.delete(g, loose_col, 1), np.delete(c, loose_col, 1)
         # bit-exact rows, including the untouched tail of the variable
-        assert (gv[s].cpu().numpy().view(np.int32) == cv[s].view(np.int32)).all(), "var rows of slot %d" % s
+        assert (g.view(np.int32) == c.view(np.int32)).all(), "var rows of slot %d" % s
     return counts
 
 
@@ -85,7 +91,7 @@ def test_cvm_columns(tn, oracle):
     pair.populate(synth.splitmix64(np.arange(1, 501, dtype=np.uint64)))
     for _ in range(2):
         values = random_batch(rng, 3, 400, 500)
-        counts = check_pull(pair, values)
+        counts = check_pull(pair, values, loose_col=9)
         grads = [(rng.standard_normal((int(u), 10)) * 0.01).astype(np.float32) for u in counts]
         labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
         pair.push_op(values, grads, labels)
@@ -295,7 +301,7 @@ def test_cfg4_shape_two_tables_same_signs(tn, oracle):
             tn.ops.sparse_table_pull(gv, [dev(v) for v in values], pair.h)
             (gw, gs, gf), (_, _, cf) = pair.export(signs)
             new = ~cf.astype(bool)
-            assert 0.1 < new.mean() < 0.5
+            assert 0.1 < new.mean() < 0.7  # 20 % of lookups, a larger share of the distinct signs
             pair.o.set_rows(signs[new], gw[new], gs[new])
             counts = check_pull(pair, values)
             grads = synth.make_grads(counts, pair.wf, sigma, seed=b)
