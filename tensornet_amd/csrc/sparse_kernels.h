@@ -12,10 +12,15 @@
 // Per-call scratch (all sized by the number of lookups L of the call):
 //     dedup table   per slot of the op, open addressing over the slot's signs,
 //                   entry {sign, position of first occurrence, rank}
-//     group table   open addressing over the distinct signs of all slots of a
-//                   push, entry {sign, count, list offset}
+//     group table   open addressing over the distinct signs of all slots,
+//                   entry {sign, members - 1, group number}
 // Both are filled with 0xFF bytes before use, which is EMPTY_KEY / "no
 // position yet" / "count -1" at once.
+//
+// What a pull works out about its batch -- the distinct signs of every slot,
+// the groups of equal signs across slots with their table rows -- is kept as
+// the table's "plan"; a push whose signs are verified (on the device) to be
+// the same batch reuses it instead of repeating remap, grouping and probing.
 #ifndef TN_SPARSE_KERNELS_H_
 #define TN_SPARSE_KERNELS_H_
 
@@ -55,14 +60,14 @@ struct DedupEntry {
 
 struct GroupEntry {
     uint64_t key;
-    uint32_t cnt;  // occurrences - 1 (starts at 0xFFFFFFFF)
-    uint32_t off;  // start of the group's member list
+    uint32_t cnt;  // members - 1 (starts at 0xFFFFFFFF)
+    uint32_t g;    // number of the group
 };
 
 constexpr int REMAP_ITEMS = 8;
 constexpr int REMAP_THREADS = 256;
 constexpr int REMAP_TILE = REMAP_ITEMS * REMAP_THREADS;
-constexpr int MAX_SLOTS = 4096;
+constexpr int MAX_SLOTS = 4095;  // lbase[MAX_SLOTS + 1] fills 16 KB of LDS
 
 __device__ __forceinline__ unsigned long long* ull(uint64_t* p) { return reinterpret_cast<unsigned long long*>(p); }
 
@@ -103,6 +108,16 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
         status->n_new = 0;
         status->gcap = gcap;
         status->list_cursor = 0;
+        status->mismatch = 0;
+        status->n_big = 0;
+    }
+}
+
+// start of a push that reuses the plan: keep the counts, clear the flags
+__global__ void k_begin_push(DevStatus* status) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        status->err = 0;
+        status->mismatch = 0;
     }
 }
 
@@ -242,37 +257,6 @@ __global__ __launch_bounds__(256) void k_gather_rows(Store s, const uint32_t* __
     }
 }
 
-// vars[slot][rank, :] = w[rows[u], :] for every distinct sign u of the op
-// (PopulatePulledVariable_, sparse_table_ops.cc:244-265).
-template <int VEC>
-__global__ __launch_bounds__(256) void k_gather_vars(Store s, const uint32_t* __restrict__ rows,
-                                                     const uint32_t* __restrict__ uniq_slot,
-                                                     const uint32_t* __restrict__ ubase,
-                                                     const SlotDesc* __restrict__ descs, DevStatus* status) {
-    const int chunks = s.wdim / VEC;
-    const int64_t total = (int64_t)status->n_unique * chunks;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
-        const int64_t u = t / chunks;
-        const int c = (int)(t - u * chunks);
-        const uint32_t row = rows[u];
-        const uint32_t sl = uniq_slot[u];
-        const int64_t r = (int64_t)u - (int64_t)ubase[sl];
-        const SlotDesc& d = descs[sl];
-        if (r >= d.rows) {
-            if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
-            continue;
-        }
-        if (row == NO_ROW) continue;
-        if (VEC == 4) {
-            float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
-            *reinterpret_cast<float4*>(d.var + r * s.wdim + c * 4) = v;
-        } else {
-            d.var[r * s.wdim + c] = s.w[(uint64_t)row * s.wstride + c];
-        }
-    }
-}
-
 // Snapshot load: table row <- caller row (+ given or fresh state).
 __global__ __launch_bounds__(256) void k_load_rows(Store s, OptDev o, const uint32_t* __restrict__ rows, int64_t n,
                                                    const float* __restrict__ w, const float* __restrict__ state) {
@@ -371,9 +355,13 @@ __device__ __forceinline__ void load_lbase(uint32_t* sh, const uint32_t* lbase, 
 // own in-slot position.  After the kernel, minpos is the position of the
 // sign's first occurrence: exactly the lookup on which the reference's
 // std::map insert succeeds (sparse_table_ops.cc:122-131).
+// Entries only ever change from EMPTY_KEY to a sign and minpos only decreases,
+// so ordinary (possibly stale) loads are safe: a stale value costs one atomic,
+// whose return value is the truth.
 __global__ __launch_bounds__(256) void k_remap_insert(const SlotDesc* __restrict__ descs,
                                                       const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                      DedupEntry* dt, uint32_t* __restrict__ tidx) {
+                                                      DedupEntry* dt, uint32_t* __restrict__ tidx,
+                                                      uint64_t* __restrict__ vals_copy) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -382,6 +370,7 @@ __global__ __launch_bounds__(256) void k_remap_insert(const SlotDesc* __restrict
         const SlotDesc& d = descs[sl];
         const uint32_t li = gi - lb[sl];
         const uint64_t sign = (uint64_t)d.values[li];
+        vals_copy[gi] = sign;
         const uint32_t tbase = d.tbase, tcap = d.tcap;
         uint32_t e;
         if (sign == EMPTY_KEY) {
@@ -390,7 +379,7 @@ __global__ __launch_bounds__(256) void k_remap_insert(const SlotDesc* __restrict
             uint32_t idx = (uint32_t)slot_of(sign, tcap);
             for (;;) {
                 e = tbase + idx;
-                uint64_t k = ld_relaxed(&dt[e].key);
+                uint64_t k = dt[e].key;
                 if (k == sign) break;
                 if (k == EMPTY_KEY) {
                     uint64_t old = atomicCAS(ull(&dt[e].key), EMPTY_KEY, sign);
@@ -400,7 +389,7 @@ __global__ __launch_bounds__(256) void k_remap_insert(const SlotDesc* __restrict
             }
         }
         tidx[gi] = e;
-        if (ld_relaxed(&dt[e].minpos) > li) atomicMin(&dt[e].minpos, li);
+        if (dt[e].minpos > li) atomicMin(&dt[e].minpos, li);
     }
 }
 
@@ -414,18 +403,20 @@ __device__ __forceinline__ uint32_t block_sum_256(uint32_t v, uint32_t* sh /*4*/
     return t;
 }
 
-// exclusive prefix of v over the 256 threads of the block
-__device__ __forceinline__ uint32_t block_excl_scan_256(uint32_t v, uint32_t* sh /*4*/) {
+// exclusive prefix of v over the 256 threads of the block; *total = block sum
+template <typename T>
+__device__ __forceinline__ T block_excl_scan_256(T v, T* sh /*4*/, T* total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint32_t inc = v;
+    T inc = v;
     for (int o = 1; o < 64; o <<= 1) {
-        uint32_t t = __shfl_up(inc, o);
+        T t = __shfl_up(inc, o);
         if (lane >= o) inc += t;
     }
     if (lane == 63) sh[wave] = inc;
     __syncthreads();
-    uint32_t base = 0;
+    T base = 0;
     for (int wv = 0; wv < wave; wv++) base += sh[wv];
+    if (total) *total = sh[0] + sh[1] + sh[2] + sh[3];
     __syncthreads();
     return base + inc - v;
 }
@@ -458,7 +449,7 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_flag_count(const uint32_t* __
 }
 
 // Step 3 (one workgroup): exclusive scan of the tile counts; total distinct
-// count U; size of the push's group table; ubase of trailing empty slots.
+// count U; size of the group table; ubase of trailing empty slots.
 __global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict__ tilesum,
                                                      uint32_t* __restrict__ tileoff, uint32_t ntiles,
                                                      const uint32_t* __restrict__ lbase, uint32_t* __restrict__ ubase,
@@ -488,7 +479,7 @@ __global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict_
     const uint32_t U = carry_sh;
     if (threadIdx.x == 0) {
         status->n_unique = U;
-        uint32_t g = 2 * U;
+        uint32_t g = U + U / 2;
         status->gcap = g < 16 ? 16 : g;
     }
     for (int sl = threadIdx.x; sl <= N; sl += blockDim.x)
@@ -500,15 +491,14 @@ __global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict_
 __global__ __launch_bounds__(REMAP_THREADS) void k_assign_rank(
     const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L, DedupEntry* dt,
     const uint32_t* __restrict__ tidx, const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff,
-    uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign, uint32_t* __restrict__ uniq_slot,
-    int32_t* __restrict__ ushow, int32_t* __restrict__ uclick) {
+    uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign, uint32_t* __restrict__ uniq_slot) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t red[4];
     load_lbase(lb, lbase, N);
     const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
     uint32_t bits = 0;
     if (base < L) bits = flag8[base / REMAP_ITEMS];
-    uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256(__popc(bits), red);
+    uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256<uint32_t>(__popc(bits), red, nullptr);
     if (base >= L) return;
     int sl = find_slot(lb, N, base);
     for (int j = 0; j < REMAP_ITEMS; j++) {
@@ -521,51 +511,120 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_assign_rank(
             for (int e = sl - 1; e >= 0 && lb[e] == gi; e--) ubase[e] = u;
         }
         if (bits & (1u << j)) {
-            const SlotDesc& d = descs[sl];
             dt[tidx[gi]].rank = u;
-            uniq_sign[u] = (uint64_t)d.values[gi - lb[sl]];
+            uniq_sign[u] = (uint64_t)descs[sl].values[gi - lb[sl]];
             uniq_slot[u] = (uint32_t)sl;
-            if (ushow) {
-                ushow[u] = 0;
-                uclick[u] = 0;
-            }
             u++;
         }
     }
 }
 
-// Step 5 (pull): mapped id = rank within the slot (sparse_table_ops.cc:130).
+constexpr uint32_t FIRST_BIT = 0x80000000u;
+
+// Step 5: mapped id = rank within the slot (sparse_table_ops.cc:130).  The
+// index of each lookup's distinct sign is kept for the push (u_of_gi, top bit
+// set on first occurrences).
 __global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict__ descs,
                                                       const uint32_t* __restrict__ lbase,
                                                       const uint32_t* __restrict__ ubase, int N, uint32_t L,
                                                       const DedupEntry* __restrict__ dt,
-                                                      const uint32_t* __restrict__ tidx) {
+                                                      const uint32_t* __restrict__ tidx,
+                                                      const uint8_t* __restrict__ flag8,
+                                                      uint32_t* __restrict__ u_of_gi, int write_ids) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        const int sl = find_slot(lb, N, gi);
         const uint32_t u = dt[tidx[gi]].rank;
-        descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+        const uint32_t first = (flag8[gi >> 3] >> (gi & 7)) & 1u;
+        u_of_gi[gi] = u | (first ? FIRST_BIT : 0u);
+        if (write_ids) {
+            const int sl = find_slot(lb, N, gi);
+            descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+        }
     }
 }
 
-// Step 5 (push): batch_show = occurrences, batch_click = sum of labels
-// (sparse_table_ops.cc:283-296; labels are narrowed to int as there).
-__global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
-                                                    const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                    const DedupEntry* __restrict__ dt,
-                                                    const uint32_t* __restrict__ tidx, int32_t* ushow,
-                                                    int32_t* uclick) {
+// Push: are the signs of this call the ones the plan was built from?
+__global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
+                                                       const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                       const uint64_t* __restrict__ vals_copy, uint32_t* mismatch) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
+    bool bad = false;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
-        const uint32_t u = dt[tidx[gi]].rank;
-        atomicAdd(&ushow[u], 1);
-        const int label = (int)descs[sl].labels[gi - lb[sl]];
-        if (label != 0) atomicAdd(&uclick[u], label);
+        bad |= (uint64_t)descs[sl].values[gi - lb[sl]] != vals_copy[gi];
+    }
+    if (bad) atomicOr(mismatch, 1u);
+}
+
+// Push: batch_show = occurrences, batch_click = sum of labels per distinct sign
+// (sparse_table_ops.cc:283-296; labels are narrowed to int as there).
+// Every distinct sign starts at show 1 / click 0 ...
+__global__ __launch_bounds__(256) void k_reset_counts(int32_t* __restrict__ ushow, int32_t* __restrict__ uclick,
+                                                      const DevStatus* status) {
+    const uint32_t n = status->n_unique;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
+        ushow[u] = 1;
+        uclick[u] = 0;
+    }
+}
+
+constexpr int COUNT_TILE = 2048;
+constexpr int COUNT_SLOTS = 4096;  // LDS table entries per tile (load factor <= 0.5)
+
+// ... and the repeated lookups and the non-zero labels are added.  Repeats
+// are concentrated on few signs, so each tile of 2048 lookups first adds them
+// up in an LDS hash table and issues one global atomic per sign it saw.
+__global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
+                                                    const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                    const uint32_t* __restrict__ u_of_gi, int32_t* ushow,
+                                                    int32_t* uclick, int with_click) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t keys[COUNT_SLOTS];
+    __shared__ int32_t cnts[COUNT_SLOTS];
+    __shared__ int32_t clks[COUNT_SLOTS];
+    if (with_click) load_lbase(lb, lbase, N);
+    const uint32_t ntiles = (L + COUNT_TILE - 1) / COUNT_TILE;
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
+            keys[i] = 0xFFFFFFFFu;
+            cnts[i] = 0;
+            clks[i] = 0;
+        }
+        __syncthreads();
+        for (int j = 0; j < COUNT_TILE / 256; j++) {
+            const uint32_t gi = tile * COUNT_TILE + j * 256 + threadIdx.x;
+            if (gi >= L) break;
+            const uint32_t v = u_of_gi[gi];
+            const uint32_t u = v & ~FIRST_BIT;
+            int label = 0;
+            if (with_click) {
+                const int sl = find_slot(lb, N, gi);
+                label = (int)descs[sl].labels[gi - lb[sl]];
+            }
+            const bool repeat = (v & FIRST_BIT) == 0;
+            if (!repeat && label == 0) continue;
+            uint32_t h = (u * 2654435761u) >> 20;  // 12 bits
+            for (;;) {
+                uint32_t old = atomicCAS(&keys[h], 0xFFFFFFFFu, u);
+                if (old == 0xFFFFFFFFu || old == u) break;
+                h = (h + 1) & (COUNT_SLOTS - 1);
+            }
+            if (repeat) atomicAdd(&cnts[h], 1);
+            if (label != 0) atomicAdd(&clks[h], label);
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
+            const uint32_t u = keys[i];
+            if (u == 0xFFFFFFFFu) continue;
+            if (cnts[i]) atomicAdd(&ushow[u], cnts[i]);
+            if (clks[i]) atomicAdd(&uclick[u], clks[i]);
+        }
+        __syncthreads();
     }
 }
 
@@ -605,7 +664,7 @@ __global__ __launch_bounds__(256) void k_group_insert(PushSrc src, int64_t n_hos
             uint32_t idx = (uint32_t)slot_of(sign, gcap);
             for (;;) {
                 e = idx;
-                uint64_t k = ld_relaxed(&gt[e].key);
+                uint64_t k = gt[e].key;  // a stale EMPTY_KEY only costs a compare-and-swap
                 if (k == sign) break;
                 if (k == EMPTY_KEY) {
                     uint64_t old = atomicCAS(ull(&gt[e].key), EMPTY_KEY, sign);
@@ -619,49 +678,124 @@ __global__ __launch_bounds__(256) void k_group_insert(PushSrc src, int64_t n_hos
     }
 }
 
-// ...every group gets a slice of the member list...
+constexpr int COMPACT_ITEMS = 4;
+
+// ...every group gets a number, a slice of the member list (two atomics per
+// 1024 table entries) and, when it has big_k members or more, a place in the
+// list of big groups...
 __global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupEntry* gt,
                                                        uint64_t* __restrict__ grp_sign,
                                                        uint32_t* __restrict__ grp_off,
-                                                       uint32_t* __restrict__ grp_cnt) {
+                                                       uint32_t* __restrict__ grp_cnt,
+                                                       uint32_t* __restrict__ big_list, uint32_t big_k) {
+    __shared__ unsigned long long sh[4];
+    __shared__ uint32_t bases[2];
     const uint32_t n = status->gcap + 1;
-    const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
-        const uint32_t c = gt[e].cnt;
-        const bool used = c != 0xFFFFFFFFu;
-        const uint32_t g = wave_alloc(used, &status->n_groups);
-        if (!used) continue;
-        const uint32_t k = c + 1;
-        const uint32_t off = atomicAdd(&status->list_cursor, k);
-        gt[e].off = off;
-        grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
-        grp_off[g] = off;
-        grp_cnt[g] = k;
+    const uint32_t span = 256 * COMPACT_ITEMS;
+    for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
+        const uint32_t e0 = base + threadIdx.x * COMPACT_ITEMS;
+        uint32_t ks[COMPACT_ITEMS];
+        unsigned long long mine = 0;  // (groups << 32) | members
+        for (int j = 0; j < COMPACT_ITEMS; j++) {
+            const uint32_t e = e0 + j;
+            const uint32_t c = (e < n) ? gt[e].cnt : 0xFFFFFFFFu;
+            ks[j] = (c != 0xFFFFFFFFu) ? c + 1 : 0;
+            if (ks[j]) mine += (1ull << 32) | ks[j];
+        }
+        unsigned long long total;
+        unsigned long long excl = block_excl_scan_256<unsigned long long>(mine, sh, &total);
+        if (threadIdx.x == 0 && total) {
+            bases[0] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32));
+            bases[1] = atomicAdd(&status->list_cursor, (uint32_t)total);
+        }
+        __syncthreads();
+        uint32_t g = bases[0] + (uint32_t)(excl >> 32);
+        uint32_t off = bases[1] + (uint32_t)excl;
+        for (int j = 0; j < COMPACT_ITEMS; j++) {
+            const uint32_t k = ks[j];
+            const bool big = k >= big_k;
+            const uint32_t b = wave_alloc(big, &status->n_big);
+            if (k == 0) continue;
+            const uint32_t e = e0 + j;
+            gt[e].g = g;
+            grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
+            grp_off[g] = off;
+            grp_cnt[g] = k;
+            if (big) big_list[b] = g;
+            g++;
+            off += k;
+        }
+        __syncthreads();
     }
 }
 
-// ...and the members are written into it (in arrival order; the apply kernel
-// walks them in ascending record order).
+// ...the members are written into it in arrival order...
 __global__ __launch_bounds__(256) void k_group_fill(int64_t n_host, const uint32_t* n_dev, const GroupEntry* gt,
+                                                    const uint32_t* __restrict__ grp_off,
                                                     const uint32_t* __restrict__ gidx,
-                                                    const uint32_t* __restrict__ ord, uint32_t* __restrict__ list) {
+                                                    const uint32_t* __restrict__ ord, uint32_t* __restrict__ arrival) {
     const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride)
-        list[gt[gidx[u]].off + ord[u]] = (uint32_t)u;
+        arrival[grp_off[gt[gidx[u]].g] + ord[u]] = (uint32_t)u;
+}
+
+// ...and finally put in ascending record order: the place of a record is the
+// number of members of its group that precede it.
+__global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32_t* n_dev, const GroupEntry* gt,
+                                                    const uint32_t* __restrict__ grp_off,
+                                                    const uint32_t* __restrict__ gidx,
+                                                    const uint32_t* __restrict__ arrival, uint32_t* __restrict__ list,
+                                                    uint32_t* __restrict__ g_of_u) {
+    const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
+        const GroupEntry en = gt[gidx[u]];
+        const uint32_t k = en.cnt + 1;
+        const uint32_t off = grp_off[en.g];
+        uint32_t pos = 0;
+        if (k > 1) {
+            const uint32_t* mem = arrival + off;
+            for (uint32_t t = 0; t < k; t++) pos += mem[t] < (uint32_t)u;
+        }
+        list[off + pos] = (uint32_t)u;
+        g_of_u[u] = en.g;
+    }
+}
+
+// vars[slot][rank, :] = table row of the sign, for every distinct sign u of
+// every slot (PopulatePulledVariable_, sparse_table_ops.cc:244-265).
+template <int VEC>
+__global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status, const uint32_t* __restrict__ grp_row,
+                                                     const uint32_t* __restrict__ g_of_u,
+                                                     const uint32_t* __restrict__ uniq_slot,
+                                                     const uint32_t* __restrict__ ubase,
+                                                     const SlotDesc* __restrict__ descs) {
+    const int chunks = s.wdim / VEC;
+    const int64_t total = (int64_t)status->n_unique * chunks;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int64_t u = t / chunks;
+        const int c = (int)(t - u * chunks);
+        const uint32_t row = grp_row[g_of_u[u]];
+        const uint32_t sl = uniq_slot[u];
+        const int64_t r = (int64_t)u - (int64_t)ubase[sl];
+        const SlotDesc& d = descs[sl];
+        if (r >= d.rows) {
+            if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
+            continue;
+        }
+        if (row == NO_ROW) continue;
+        if (VEC == 4) {
+            float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
+            *reinterpret_cast<float4*>(d.var + r * s.wdim + c * 4) = v;
+        } else {
+            d.var[r * s.wdim + c] = s.w[(uint64_t)row * s.wstride + c];
+        }
+    }
 }
 
 // -------------------------------------------------------------------- apply
-// smallest member of the group's list that is larger than prev (prev = -1 first)
-__device__ __forceinline__ uint32_t next_member(const uint32_t* list, uint32_t k, int64_t prev) {
-    uint32_t best = 0xFFFFFFFFu;
-    for (uint32_t t = 0; t < k; t++) {
-        uint32_t v = list[t];
-        if ((int64_t)v > prev && v < best) best = v;
-    }
-    return best;
-}
-
 // Resolves record u to its gradient row and counts; false if the op's gradient
 // matrix has no such row.
 __device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, const float*& g, int& show, int& click) {
@@ -681,27 +815,53 @@ __device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, const f
     return true;
 }
 
-// One group of LPG lanes owns one distinct sign: it loads the row once, applies
-// the sign's records in ascending record order (slot 0 first) and stores the
-// row once.  Each lane holds one float4 of every per-element array.
+// The three update rules on one element.
 //   AdaGrad  ada_grad_kernel.cc:105-129     Adam  adam_kernel.cc:112-125
 //   Ftrl     ftrl_kernel.cc:57-80
+__device__ __forceinline__ void adam_elem(const OptDev& o, float c1, float c2, float g, float& w, float& m, float& v) {
+    m = o.beta1 * m + c1 * g;
+    v = o.beta2 * v + c2 * g * g;
+    w -= o.lr * m / (o.eps + sqrtf(v));
+}
+
+__device__ __forceinline__ void ftrl_elem(const OptDev& o, float g, float& w, float& z, float& n) {
+    const float g2 = g * g;
+    z += g - o.lr * (sqrtf(n + g2) - sqrtf(n)) * w;
+    n += g2;
+    if (fabsf(z) <= o.lambda1) {
+        w = 0.f;
+    } else {
+        w = -1 / ((o.beta + sqrtf(n)) * o.lr + o.lambda2);
+        if (z > 0)
+            w *= z - o.lambda1;
+        else
+            w *= z + o.lambda1;
+    }
+}
+
+// One group of LPG lanes owns one distinct sign: it loads the row once, applies
+// the sign's records in ascending record order (slot 0 first; the member list
+// is sorted) and stores the row once.  Each lane holds one float4 of every
+// per-element array; the next record's gradient is fetched while the current
+// one is applied.  Groups with big_k records or more are left to k_apply_big.
 template <int KIND, int LPG>
 __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc src, DevStatus* status,
                                                    const uint32_t* __restrict__ grp_row,
                                                    const uint32_t* __restrict__ grp_off,
                                                    const uint32_t* __restrict__ grp_cnt,
-                                                   const uint32_t* __restrict__ list) {
+                                                   const uint32_t* __restrict__ list, uint32_t big_k) {
     const uint32_t n_groups = status->n_groups;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;                       // my float4 inside the row
     const int lane = (int)__lane_id();
     const int lane0 = lane - sub;                            // first lane of my group in the wavefront
     const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
     for (uint32_t g = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; g < n_groups; g += gstride) {
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
         const uint32_t k = grp_cnt[g];
+        if (k >= big_k) continue;
         const uint32_t* mem = list + grp_off[g];
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
@@ -719,19 +879,25 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
             b = reinterpret_cast<float4*>(sp + D)[sub];
             delta_show = __float_as_int(sp[2 * D + 1]);
         }
-        int64_t prev = -1;
         bool any = false;
+        const float* gp;
+        int nshow = 0, nclick = 0;
+        bool nok = src_record(src, mem[0], gp, nshow, nclick);
+        float4 gnext = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
         for (uint32_t j = 0; j < k; j++) {
-            const uint32_t u = (k == 1) ? mem[0] : next_member(mem, k, prev);
-            prev = u;
-            const float* gp;
-            int bshow, bclick;
-            if (!src_record(src, u, gp, bshow, bclick)) {
+            const float4 gr = gnext;
+            const int bshow = nshow, bclick = nclick;
+            const bool ok = nok;
+            if (j + 1 < k) {
+                nok = src_record(src, mem[j + 1], gp, nshow, nclick);
+                if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
+            }
+            if (!ok) {
                 if (sub == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
                 continue;
             }
             any = true;
-            const float4 gr = reinterpret_cast<const float4*>(gp)[sub];
             if (KIND == OPT_ADAGRAD) {
                 show += (float)bshow;
                 click += (float)bclick;
@@ -754,38 +920,16 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                 w.w -= o.lr * gr.w / den;
             } else if (KIND == OPT_ADAM) {
                 delta_show += bshow;
-                const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
-#define TN_ADAM_E(W, M, V, G)                    \
-    M = o.beta1 * M + c1 * G;                    \
-    V = o.beta2 * V + c2 * G * G;                \
-    W -= o.lr * M / (o.eps + sqrtf(V));
-                TN_ADAM_E(w.x, a.x, b.x, gr.x)
-                TN_ADAM_E(w.y, a.y, b.y, gr.y)
-                TN_ADAM_E(w.z, a.z, b.z, gr.z)
-                TN_ADAM_E(w.w, a.w, b.w, gr.w)
-#undef TN_ADAM_E
+                adam_elem(o, c1, c2, gr.x, w.x, a.x, b.x);
+                adam_elem(o, c1, c2, gr.y, w.y, a.y, b.y);
+                adam_elem(o, c1, c2, gr.z, w.z, a.z, b.z);
+                adam_elem(o, c1, c2, gr.w, w.w, a.w, b.w);
             } else {
                 delta_show += bshow;
-#define TN_FTRL_E(W, Z, NN, G)                                                   \
-    {                                                                            \
-        const float g2 = G * G;                                                  \
-        Z += G - o.lr * (sqrtf(NN + g2) - sqrtf(NN)) * W;                        \
-        NN += g2;                                                                \
-        if (fabsf(Z) <= o.lambda1) {                                             \
-            W = 0.f;                                                             \
-        } else {                                                                 \
-            W = -1 / ((o.beta + sqrtf(NN)) * o.lr + o.lambda2);                  \
-            if (Z > 0)                                                           \
-                W *= Z - o.lambda1;                                              \
-            else                                                                 \
-                W *= Z + o.lambda1;                                              \
-        }                                                                        \
-    }
-                TN_FTRL_E(w.x, a.x, b.x, gr.x)
-                TN_FTRL_E(w.y, a.y, b.y, gr.y)
-                TN_FTRL_E(w.z, a.z, b.z, gr.z)
-                TN_FTRL_E(w.w, a.w, b.w, gr.w)
-#undef TN_FTRL_E
+                ftrl_elem(o, gr.x, w.x, a.x, b.x);
+                ftrl_elem(o, gr.y, w.y, a.y, b.y);
+                ftrl_elem(o, gr.z, w.z, a.z, b.z);
+                ftrl_elem(o, gr.w, w.w, a.w, b.w);
             }
         }
         if (!any) continue;
@@ -806,13 +950,132 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
     }
 }
 
+constexpr int BIG_DIM_MAX = 512;    // largest dim k_apply_big stages in LDS
+constexpr int BIG_GBUF = 2048;      // floats of gradient staging per wavefront
+
+// A sign with many records (it occurs in many slots) would make one lane
+// group chase a long chain of dependent loads.  Here one wavefront owns the
+// sign: the row lives in LDS, the gradients of up to 64 records at a time are
+// fetched by all lanes in parallel and then applied strictly in record order,
+// lanes working on different elements of the row.
+template <int KIND>
+__global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                  const uint32_t* __restrict__ big_list,
+                                                  const uint32_t* __restrict__ grp_row,
+                                                  const uint32_t* __restrict__ grp_off,
+                                                  const uint32_t* __restrict__ grp_cnt,
+                                                  const uint32_t* __restrict__ list) {
+    __shared__ float rw[BIG_DIM_MAX], ra[BIG_DIM_MAX], rb[BIG_DIM_MAX];
+    __shared__ float gbuf[BIG_GBUF];
+    __shared__ const float* gptr[64];
+    __shared__ int gshow[64], gclick[64], gok[64];
+    const int D = s.D;
+    const int lane = threadIdx.x;
+    const uint32_t n_big = status->n_big;
+    const int per_chunk = (BIG_GBUF / D) < 64 ? (BIG_GBUF / D) : 64;
+    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+    for (uint32_t bi = blockIdx.x; bi < n_big; bi += gridDim.x) {
+        const uint32_t g = big_list[bi];
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;
+        const uint32_t k = grp_cnt[g];
+        const uint32_t* mem = list + grp_off[g];
+        float* wp = s.w + (uint64_t)row * s.wstride;
+        float* sp = s.st + (uint64_t)row * s.sstride;
+        for (int i = lane; i < D; i += 64) {
+            rw[i] = wp[i];
+            if (KIND != OPT_ADAGRAD) {
+                ra[i] = sp[i];
+                rb[i] = sp[D + i];
+            }
+        }
+        float g2sum = 0.f, show = 0.f, click = 0.f;
+        int delta_show = 0;
+        if (KIND == OPT_ADAGRAD) {
+            g2sum = sp[0];
+            show = sp[1];
+            click = sp[2];
+        } else {
+            delta_show = __float_as_int(sp[2 * D + 1]);
+        }
+        bool any = false;
+        __syncthreads();
+        for (uint32_t c0 = 0; c0 < k; c0 += per_chunk) {
+            const int cn = (int)((k - c0) < (uint32_t)per_chunk ? (k - c0) : (uint32_t)per_chunk);
+            if (lane < cn) {
+                const float* gp = nullptr;
+                int sh = 0, ck = 0;
+                const bool ok = src_record(src, mem[c0 + lane], gp, sh, ck);
+                gptr[lane] = gp;
+                gshow[lane] = sh;
+                gclick[lane] = ck;
+                gok[lane] = ok ? 1 : 0;
+            }
+            __syncthreads();
+            for (int t = lane; t < cn * D; t += 64) {
+                const int m = t / D, i = t - m * D;
+                gbuf[t] = gok[m] ? gptr[m][i] : 0.f;
+            }
+            __syncthreads();
+            for (int m = 0; m < cn; m++) {
+                if (!gok[m]) {
+                    if (lane == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+                    continue;
+                }
+                any = true;
+                const float* gr = gbuf + m * D;
+                if (KIND == OPT_ADAGRAD) {
+                    show += (float)gshow[m];
+                    click += (float)gclick[m];
+                    double tot = 0.0;  // every lane adds up all D products in element order
+                    for (int i = 0; i < D; i++) tot += (double)(gr[i] * gr[i]);
+                    g2sum = (float)((double)g2sum + tot / (double)D);
+                    const float den = o.eps + sqrtf(g2sum);
+                    for (int i = lane; i < D; i += 64) rw[i] -= o.lr * gr[i] / den;
+                } else if (KIND == OPT_ADAM) {
+                    delta_show += gshow[m];
+                    for (int i = lane; i < D; i += 64) adam_elem(o, c1, c2, gr[i], rw[i], ra[i], rb[i]);
+                } else {
+                    delta_show += gshow[m];
+                    for (int i = lane; i < D; i += 64) ftrl_elem(o, gr[i], rw[i], ra[i], rb[i]);
+                }
+            }
+            __syncthreads();
+        }
+        if (any) {
+            for (int i = lane; i < D; i += 64) {
+                wp[i] = rw[i];
+                if (KIND != OPT_ADAGRAD) {
+                    sp[i] = ra[i];
+                    sp[D + i] = rb[i];
+                }
+            }
+            if (lane == 0) {
+                if (KIND == OPT_ADAGRAD) {
+                    sp[0] = g2sum;
+                    sp[1] = show;
+                    sp[2] = click;
+                    sp[3] = 0.f;  // no_show_days = 0
+                    if (o.use_cvm) {
+                        wp[D] = show;
+                        wp[D + 1] = logf(click + 1) - logf(show + 1);
+                    }
+                } else {
+                    sp[2 * D + 1] = __int_as_float(delta_show);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // Any dim / alignment: one thread per distinct sign, scalar loops.
 template <int KIND>
 __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc src, DevStatus* status,
                                                       const uint32_t* __restrict__ grp_row,
                                                       const uint32_t* __restrict__ grp_off,
                                                       const uint32_t* __restrict__ grp_cnt,
-                                                      const uint32_t* __restrict__ list) {
+                                                      const uint32_t* __restrict__ list, uint32_t big_k) {
     const uint32_t n_groups = status->n_groups;
     const int D = s.D;
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -820,13 +1083,12 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;
         const uint32_t k = grp_cnt[g];
+        if (k >= big_k) continue;
         const uint32_t* mem = list + grp_off[g];
         float* w = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
-        int64_t prev = -1;
         for (uint32_t j = 0; j < k; j++) {
-            const uint32_t u = (k == 1) ? mem[0] : next_member(mem, k, prev);
-            prev = u;
+            const uint32_t u = mem[j];
             const float* gp;
             int bshow, bclick;
             if (!src_record(src, u, gp, bshow, bclick)) {

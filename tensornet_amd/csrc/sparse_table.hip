@@ -34,7 +34,14 @@ struct SparseTable {
     uint64_t booked = 0;       // part of count_upper booked for the inserts of the pending call
 
     DevBuf ws;                      // per-call scratch
-    DevStatus* dstatus = nullptr;   // device
+    DevBuf plan_buf;                // what the last pull op worked out about its batch (see Plan)
+    bool plan_valid = false;
+    int plan_N = 0;
+    std::vector<int64_t> plan_lens;
+    uint64_t epoch = 0;             // bumped whenever rows move (growth)
+    uint64_t plan_epoch = 0;
+    DevStatus* dstatus = nullptr;   // device: status of table-level calls
+    DevStatus* dplan = nullptr;     // device: status / counts of the op-level plan
     HostStatus* hpull = nullptr;    // pinned
     HostStatus* hpush = nullptr;    // pinned
     char* hstage = nullptr;         // pinned staging of slot descriptors
@@ -125,8 +132,9 @@ void free_store(Store& s) {
 
 int ensure_side_buffers(SparseTable* t) {
     if (t->dstatus) return TN_OK;
-    TN_HIP(hipMalloc((void**)&t->dstatus, sizeof(DevStatus)));
-    TN_HIP(hipMemset(t->dstatus, 0, sizeof(DevStatus)));
+    TN_HIP(hipMalloc((void**)&t->dstatus, 2 * sizeof(DevStatus)));
+    TN_HIP(hipMemset(t->dstatus, 0, 2 * sizeof(DevStatus)));
+    t->dplan = t->dstatus + 1;
     TN_HIP(hipHostMalloc((void**)&t->hpull, sizeof(HostStatus), hipHostMallocDefault));
     TN_HIP(hipHostMalloc((void**)&t->hpush, sizeof(HostStatus), hipHostMallocDefault));
     std::memset(t->hpull, 0, sizeof(HostStatus));
@@ -235,6 +243,7 @@ int grow_to(SparseTable* t, uint64_t cap, hipStream_t st) {
     TN_HIP(hipStreamSynchronize(st));
     free_store(s);
     s = bigger;
+    t->epoch++;  // cached row numbers are stale now
     return TN_OK;
 }
 
@@ -278,11 +287,32 @@ struct Carver {
     }
 };
 
-// Scratch of one op call, carved from the table's workspace buffer.
-struct OpScratch {
+// Results of analysing one batch.  For an op-level call they live in the
+// table's plan buffer and survive until the next op-level call, so that a push
+// of the same batch can reuse them; a table-level push carves the group part
+// from the per-call scratch.
+struct Plan {
     SlotDesc* descs;
     uint32_t* lbase;
     uint32_t* ubase;
+    uint64_t* vals_copy;   // signs of every lookup, concatenated
+    uint32_t* u_of_gi;     // lookup -> index of its distinct sign
+    uint64_t* uniq_sign;   // per-slot distinct signs, slot-major, first-occurrence order
+    uint32_t* uniq_slot;
+    int32_t* ushow;
+    int32_t* uclick;
+    uint64_t* grp_sign;    // distinct signs over all slots
+    uint32_t* grp_row;     // their table rows
+    uint32_t* grp_off;
+    uint32_t* grp_cnt;
+    uint32_t* list;        // members (indices into uniq_*) of every group, ascending
+    uint32_t* g_of_u;      // record -> its group
+    uint32_t* big_list;    // groups with BIG_GROUP records or more
+    uint32_t* newlist;     // groups whose row was inserted by the pull
+};
+
+// Per-call scratch of the analysis.
+struct Scratch {
     DedupEntry* dt;
     size_t dt_entries;
     uint32_t* tidx;
@@ -290,40 +320,54 @@ struct OpScratch {
     uint32_t* tilesum;
     uint32_t* tileoff;
     uint32_t ntiles;
-    uint64_t* uniq_sign;
-    uint32_t* uniq_slot;
-    int32_t* ushow;
-    int32_t* uclick;
-    uint32_t* rows;
-    uint32_t* newlist;
-    // push grouping
     GroupEntry* gt;
     uint32_t* gidx;
     uint32_t* ord;
-    uint32_t* list;
-    uint64_t* grp_sign;
-    uint32_t* grp_off;
-    uint32_t* grp_cnt;
-    uint32_t* grp_row;
+    uint32_t* arrival;
 };
 
-void carve_group(Carver& c, OpScratch& w, size_t n) {
-    size_t gcap = std::max<size_t>(16, 2 * n);
-    w.gt = c.take<GroupEntry>(gcap + 1);
-    w.gidx = c.take<uint32_t>(n);
-    w.ord = c.take<uint32_t>(n);
-    w.list = c.take<uint32_t>(n);
-    w.grp_sign = c.take<uint64_t>(n);
-    w.grp_off = c.take<uint32_t>(n);
-    w.grp_cnt = c.take<uint32_t>(n);
-    w.grp_row = c.take<uint32_t>(n);
+size_t group_cap(size_t n) { return std::max<size_t>(16, n + n / 2); }
+
+// Signs with this many records or more are applied by one wavefront each
+// (k_apply_big); rows too wide for its LDS staging stay with the lane groups.
+constexpr uint32_t BIG_GROUP = 16;
+uint32_t big_threshold(const Store& s) { return s.D <= BIG_DIM_MAX ? BIG_GROUP : 0xFFFFFFFFu; }
+
+void carve_groups(Carver& c, Plan& p, size_t n) {
+    p.grp_sign = c.take<uint64_t>(n);
+    p.grp_row = c.take<uint32_t>(n);
+    p.grp_off = c.take<uint32_t>(n);
+    p.grp_cnt = c.take<uint32_t>(n);
+    p.list = c.take<uint32_t>(n);
+    p.g_of_u = c.take<uint32_t>(n);
+    p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
+    p.newlist = c.take<uint32_t>(n);
 }
 
-size_t carve_op(char* base, OpScratch& w, int N, size_t L, size_t dt_entries, bool push) {
+void carve_group_scratch(Carver& c, Scratch& w, size_t n) {
+    w.gt = c.take<GroupEntry>(group_cap(n) + 1);
+    w.gidx = c.take<uint32_t>(n);
+    w.ord = c.take<uint32_t>(n);
+    w.arrival = c.take<uint32_t>(n);
+}
+
+size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     Carver c{base};
-    w.descs = c.take<SlotDesc>(N);
-    w.lbase = c.take<uint32_t>(N + 1);
-    w.ubase = c.take<uint32_t>(N + 1);
+    p.descs = c.take<SlotDesc>(N);
+    p.lbase = c.take<uint32_t>(N + 1);
+    p.ubase = c.take<uint32_t>(N + 1);
+    p.vals_copy = c.take<uint64_t>(L);
+    p.u_of_gi = c.take<uint32_t>(L);
+    p.uniq_sign = c.take<uint64_t>(L);
+    p.uniq_slot = c.take<uint32_t>(L);
+    p.ushow = c.take<int32_t>(L);
+    p.uclick = c.take<int32_t>(L);
+    carve_groups(c, p, L);
+    return align_up(c.off, 256);
+}
+
+size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries) {
+    Carver c{base};
     w.dt = c.take<DedupEntry>(dt_entries);
     w.dt_entries = dt_entries;
     w.tidx = c.take<uint32_t>(L);
@@ -331,23 +375,11 @@ size_t carve_op(char* base, OpScratch& w, int N, size_t L, size_t dt_entries, bo
     w.ntiles = (uint32_t)((L + REMAP_TILE - 1) / REMAP_TILE);
     w.tilesum = c.take<uint32_t>(w.ntiles + 1);
     w.tileoff = c.take<uint32_t>(w.ntiles + 1);
-    w.uniq_sign = c.take<uint64_t>(L);
-    w.uniq_slot = c.take<uint32_t>(L);
-    if (push) {
-        w.ushow = c.take<int32_t>(L);
-        w.uclick = c.take<int32_t>(L);
-        carve_group(c, w, L);
-        w.rows = nullptr;
-        w.newlist = nullptr;
-    } else {
-        w.ushow = w.uclick = nullptr;
-        w.rows = c.take<uint32_t>(L);
-        w.newlist = c.take<uint32_t>(L);
-    }
+    carve_group_scratch(c, w, L);
     return align_up(c.off, 256);
 }
 
-// Validates the slot arrays of an op and stages descriptors; returns L.
+// Validates the slot arrays of an op and fills the descriptors; returns L.
 int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64_t* lens, std::vector<SlotDesc>& descs,
                 std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what) {
     if (N <= 0 || !values || !lens) return fail(TN_ERR_INVALID_ARGUMENT, std::string(what) + ": no slots");
@@ -378,7 +410,7 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
     return TN_OK;
 }
 
-int upload_slots(SparseTable* t, const OpScratch& w, const std::vector<SlotDesc>& descs,
+int upload_slots(SparseTable* t, const Plan& p, const std::vector<SlotDesc>& descs,
                  const std::vector<uint32_t>& lbase, hipStream_t st) {
     if (t->stage_pending) {
         TN_HIP(hipEventSynchronize(t->stage_ev));
@@ -388,29 +420,75 @@ int upload_slots(SparseTable* t, const OpScratch& w, const std::vector<SlotDesc>
     const size_t lb = lbase.size() * sizeof(uint32_t);
     std::memcpy(t->hstage, descs.data(), db);
     std::memcpy(t->hstage + db, lbase.data(), lb);
-    TN_HIP(hipMemcpyAsync(w.descs, t->hstage, db, hipMemcpyHostToDevice, st));
-    TN_HIP(hipMemcpyAsync(w.lbase, t->hstage + db, lb, hipMemcpyHostToDevice, st));
+    TN_HIP(hipMemcpyAsync(p.descs, t->hstage, db, hipMemcpyHostToDevice, st));
+    TN_HIP(hipMemcpyAsync(p.lbase, t->hstage + db, lb, hipMemcpyHostToDevice, st));
     TN_HIP(hipEventRecord(t->stage_ev, st));
     t->stage_pending = true;
     return TN_OK;
 }
 
-// Remap steps 1-4 shared by pull and push (k_remap_insert .. k_assign_rank).
-void launch_remap(const OpScratch& w, int N, uint32_t L, DevStatus* dstatus, hipStream_t st) {
-    TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st, reinterpret_cast<uint4*>(w.dt), w.dt_entries);
-    TN_LAUNCH(k_remap_insert, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, N, L, w.dt, w.tidx);
-    TN_LAUNCH(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), st, w.lbase, N, L, w.dt, w.tidx, w.flag8, w.tilesum);
-    TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, w.lbase, w.ubase, N, L, dstatus);
-    TN_LAUNCH(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), st, w.descs, w.lbase, N, L, w.dt, w.tidx, w.flag8, w.tileoff, w.ubase, w.uniq_sign, w.uniq_slot, w.ushow, w.uclick);
+PushSrc op_source(const Plan& p, int dim) {
+    PushSrc src{};
+    src.uniq_sign = p.uniq_sign;
+    src.uniq_slot = p.uniq_slot;
+    src.ubase = p.ubase;
+    src.ushow = p.ushow;
+    src.uclick = p.uclick;
+    src.descs = p.descs;
+    src.dim = dim;
+    return src;
+}
+
+// Groups n records (n_host of them, or status->n_unique) by sign: group arrays
+// and member lists in ascending record order.
+void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_t n_host, int64_t n_upper,
+                     uint32_t big_k, DevStatus* ds, hipStream_t st) {
+    const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
+    const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
+    const int tblocks = launch_grid((int64_t)group_cap(n_upper) + 1, 256, GRID_CAP * 2);
+    TN_LAUNCH(k_fill_groups, dim3(tblocks), dim3(256), st, w.gt, ds);
+    TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, w.gt, w.gidx, w.ord);
+    TN_LAUNCH(k_group_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
+              dim3(256), st, ds, w.gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
+    TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, p.grp_off, w.gidx, w.ord, w.arrival);
+    TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, p.grp_off, w.gidx, w.arrival, p.list,
+              p.g_of_u);
+}
+
+// Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids
+// (steps of k_remap_insert .. k_write_mapped), groups of equal signs, and the
+// table row of every group (inserting absent signs for a pull).
+void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull,
+                       hipStream_t st) {
+    DevStatus* ds = t->dplan;
+    const Store& s = t->store;
+    const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, 0u, 0u);
+    TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st,
+              reinterpret_cast<uint4*>(w.dt), w.dt_entries);
+    TN_LAUNCH(k_remap_insert, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, L, w.dt, w.tidx, p.vals_copy);
+    TN_LAUNCH(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.lbase, N, L, w.dt, w.tidx, w.flag8, w.tilesum);
+    TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
+    TN_LAUNCH(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.dt, w.tidx, w.flag8,
+              w.tileoff, p.ubase, p.uniq_sign, p.uniq_slot);
+    TN_LAUNCH(k_write_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.dt, w.tidx, w.flag8,
+              p.u_of_gi, for_pull ? 1 : 0);
+    launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ds, st);
+    if (for_pull)
+        TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, &ds->n_groups, p.grp_row,
+                  p.newlist, ds, (uint32_t)DEV_ERR_TABLE_FULL);
+    else
+        TN_LAUNCH((k_probe<false>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, &ds->n_groups, p.grp_row,
+                  (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
 }
 
 template <int KIND>
-void launch_apply_kind(int lpg, int blocks_hint, const Store& s, const OptDev& o, const PushSrc& src,
-                       DevStatus* dstatus, const OpScratch& w, int64_t n_upper, hipStream_t st) {
-    (void)blocks_hint;
-#define TN_LAUNCH_VEC(LPG)                                                                                            \
-    TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 2)), dim3(256), st, \
-                       s, o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list)
+void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds, const Plan& p,
+                       int64_t n_upper, hipStream_t st) {
+    const uint32_t big_k = big_threshold(s);
+#define TN_LAUNCH_VEC(LPG)                                                                                   \
+    TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, o, \
+              src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k)
     switch (lpg) {
         case 1: TN_LAUNCH_VEC(1); break;
         case 2: TN_LAUNCH_VEC(2); break;
@@ -419,34 +497,29 @@ void launch_apply_kind(int lpg, int blocks_hint, const Store& s, const OptDev& o
         case 16: TN_LAUNCH_VEC(16); break;
         case 32: TN_LAUNCH_VEC(32); break;
         default:
-            TN_LAUNCH((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, s, o, src, dstatus, w.grp_row, w.grp_off, w.grp_cnt, w.list);
+            TN_LAUNCH((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, s, o, src, ds,
+                      p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k);
     }
 #undef TN_LAUNCH_VEC
+    if (big_k != 0xFFFFFFFFu)
+        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, GRID_CAP * 2)), dim3(64), st, s, o,
+                  src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list);
 }
 
-// Group the records by sign, find the rows, apply.  n_upper bounds the number
-// of records; the exact number is n_host (table level) or status->n_unique.
-void launch_push_tail(SparseTable* t, const OpScratch& w, const PushSrc& src, int64_t n_host, int64_t n_upper,
-                      bool vec_ok, hipStream_t st) {
+// Applies the grouped records; n_upper bounds the number of records.
+void launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
+                  hipStream_t st) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
-    DevStatus* ds = t->dstatus;
-    const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
-    const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_fill_groups, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), st, w.gt, ds);
-    TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, w.gt, w.gidx, w.ord);
-    TN_LAUNCH(k_group_compact, dim3(launch_grid(2 * n_upper + 17, 256, GRID_CAP * 2)), dim3(256), st, ds, w.gt, w.grp_sign, w.grp_off, w.grp_cnt);
-    TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, w.gidx, w.ord, w.list);
-    TN_LAUNCH((k_probe<false>), dim3(gblocks), dim3(256), st, s, w.grp_sign, (int64_t)0, &ds->n_groups, w.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
     int lpg = 0;
     if (vec_ok && s.D % 4 == 0) {
         int q = s.D / 4;
         if (q >= 1 && q <= 32 && (q & (q - 1)) == 0) lpg = q;
     }
     switch (o.kind) {
-        case OPT_ADAGRAD: launch_apply_kind<OPT_ADAGRAD>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
-        case OPT_ADAM: launch_apply_kind<OPT_ADAM>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
-        default: launch_apply_kind<OPT_FTRL>(lpg, gblocks, s, o, src, ds, w, n_upper, st); break;
+        case OPT_ADAGRAD: launch_apply_kind<OPT_ADAGRAD>(lpg, s, o, src, ds, p, n_upper, st); break;
+        case OPT_ADAM: launch_apply_kind<OPT_ADAM>(lpg, s, o, src, ds, p, n_upper, st); break;
+        default: launch_apply_kind<OPT_FTRL>(lpg, s, o, src, ds, p, n_upper, st); break;
     }
 }
 
@@ -644,21 +717,27 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
         TN_HIP(hipStreamSynchronize(st));
         harvest(t);
     }
-    OpScratch w{};
+    Plan p{};
+    Scratch w{};
     {
         Carver probe{nullptr};
-        carve_group(probe, w, (size_t)n);
+        carve_groups(probe, p, (size_t)n);
+        carve_group_scratch(probe, w, (size_t)n);
         TN_TRY(t->ws.ensure(align_up(probe.off, 256) + 256));
         Carver c{(char*)t->ws.p};
-        carve_group(c, w, (size_t)n);
+        carve_groups(c, p, (size_t)n);
+        carve_group_scratch(c, w, (size_t)n);
     }
     PushSrc src{};
     src.infos = infos;
     src.grads = grads;
     src.dim = dim;
-    const uint32_t gcap = (uint32_t)std::max<int64_t>(16, 2 * n);
-    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, gcap);
-    launch_push_tail(t, w, src, n, n, aligned16(grads) && dim % 4 == 0, st);
+    DevStatus* ds = t->dstatus;
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, (uint32_t)n, (uint32_t)group_cap((size_t)n));
+    launch_grouping(p, w, src, n, n, big_threshold(t->store), ds, st);
+    TN_LAUNCH((k_probe<false>), dim3(launch_grid(n, 256, GRID_CAP * 2)), dim3(256), st, t->store, p.grp_sign,
+              (int64_t)0, &ds->n_groups, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+    launch_apply(t, p, src, ds, n, aligned16(grads) && dim % 4 == 0, st);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->push_pending = true;
@@ -764,31 +843,39 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         return take_latched(t);
     }
     TN_TRY(ensure_room(t, (uint64_t)L, st));
-    OpScratch w{};
-    size_t need = carve_op(nullptr, w, N, L, dt_entries, false);
-    TN_TRY(t->ws.ensure(need));
-    carve_op((char*)t->ws.p, w, N, L, dt_entries, false);
-    TN_TRY(upload_slots(t, w, descs, lbase, st));
+    Plan p{};
+    Scratch w{};
+    TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
+    carve_plan((char*)t->plan_buf.p, p, N, L);
+    TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries)));
+    carve_scratch((char*)t->ws.p, w, L, dt_entries);
+    t->plan_valid = false;
+    TN_TRY(upload_slots(t, p, descs, lbase, st));
 
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
-    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
-    launch_remap(w, N, (uint32_t)L, t->dstatus, st);
-    TN_LAUNCH(k_write_mapped, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, w.ubase, N, (uint32_t)L, w.dt, w.tidx);
-    const int ublocks = launch_grid(L, 256, GRID_CAP * 2);
-    TN_LAUNCH((k_probe<true>), dim3(ublocks), dim3(256), st, s, w.uniq_sign, (int64_t)0, &t->dstatus->n_unique, w.rows, w.newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
-    TN_LAUNCH(k_init_rows, dim3(ublocks), dim3(256), st, s, o, t->seed, w.uniq_sign, w.rows, w.newlist, t->dstatus);
-    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
+    DevStatus* ds = t->dplan;
+    launch_build_plan(t, p, w, N, (uint32_t)L, true, st);
+    const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
+    TN_LAUNCH(k_init_rows, dim3(gblocks), dim3(256), st, s, o, t->seed, p.grp_sign, p.grp_row, p.newlist, ds);
+    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
     if (vec)
-        TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+        TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, ds,
+                  p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
     else
-        TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, w.rows, w.uniq_slot, w.ubase, w.descs, t->dstatus);
+        TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
+                  p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
     TN_HIP(hipGetLastError());
-    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
-    TN_HIP(hipMemcpyAsync(t->hpull->ubase, w.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(t->hpull->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
     t->pull_pending = true;
     t->pending_slots = N;
     t->pending_rows.assign(var_rows, var_rows + N);
+    // a push of the same batch may reuse the analysis
+    t->plan_valid = true;
+    t->plan_N = N;
+    t->plan_lens.assign(value_lens, value_lens + N);
+    t->plan_epoch = t->epoch;
     if (t->async_pull) return TN_OK;
     return sync_table(t, st);
 }
@@ -826,27 +913,41 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         harvest(t);
     }
     if (L == 0) return TN_OK;
-    OpScratch w{};
-    size_t need = carve_op(nullptr, w, N, L, dt_entries, true);
-    TN_TRY(t->ws.ensure(need));
-    carve_op((char*)t->ws.p, w, N, L, dt_entries, true);
-    TN_TRY(upload_slots(t, w, descs, lbase, st));
-
-    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
-    launch_remap(w, N, (uint32_t)L, t->dstatus, st);
-    TN_LAUNCH(k_count_show, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, w.descs, w.lbase, N, (uint32_t)L, w.dt, w.tidx, w.ushow, w.uclick);
-    PushSrc src{};
-    src.uniq_sign = w.uniq_sign;
-    src.uniq_slot = w.uniq_slot;
-    src.ubase = w.ubase;
-    src.ushow = w.ushow;
-    src.uclick = w.uclick;
-    src.descs = w.descs;
-    src.dim = grad_dim;
-    launch_push_tail(t, w, src, 0, (int64_t)L, vec, st);
+    Plan p{};
+    Scratch w{};
+    // Same batch as the last pull?  Necessary conditions on the host, the signs
+    // themselves are compared on the device.
+    bool reuse = t->plan_valid && t->plan_epoch == t->epoch && t->plan_N == N &&
+                 std::equal(value_lens, value_lens + N, t->plan_lens.begin());
+    DevStatus* ds = t->dplan;
+    if (reuse) {
+        carve_plan((char*)t->plan_buf.p, p, N, L);
+        TN_TRY(upload_slots(t, p, descs, lbase, st));
+        TN_LAUNCH(k_begin_push, dim3(1), dim3(64), st, ds);
+        TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
+                  (uint32_t)L, p.vals_copy, &ds->mismatch);
+        TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+        TN_HIP(hipStreamSynchronize(st));
+        reuse = t->hpush->st.mismatch == 0;
+    }
+    if (!reuse) {
+        t->plan_valid = false;
+        TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
+        carve_plan((char*)t->plan_buf.p, p, N, L);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries);
+        TN_TRY(upload_slots(t, p, descs, lbase, st));
+        launch_build_plan(t, p, w, N, (uint32_t)L, false, st);
+    }
+    const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
+    TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ushow, p.uclick, ds);
+    // AdaGrad is the only optimizer that reads batch_click
+    TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256), st,
+              p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ushow, p.uclick, t->opt->kind == OPT_ADAGRAD ? 1 : 0);
+    launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
     TN_HIP(hipGetLastError());
-    TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
-    TN_HIP(hipMemcpyAsync(t->hpush->ubase, w.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipMemcpyAsync(t->hpush->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
     t->push_pending = true;
     t->pending_slots = N;
     return TN_OK;

@@ -84,7 +84,8 @@ struct DevStatus {
     uint32_t n_new;      // rows inserted by this call
     uint32_t gcap;       // slots of the per-call group table
     uint32_t list_cursor;
-    uint32_t pad[2];
+    uint32_t mismatch;   // a push found other signs than the plan was built from
+    uint32_t n_big;      // groups with many records (handled one wavefront each)
 };
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {

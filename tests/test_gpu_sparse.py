@@ -376,3 +376,39 @@ def test_full_size_batch_properties(tn, oracle):
     cum = torch.cumsum(0.01 * g / torch.sqrt(0.1 + steps * g * g), 0)
     expect = w0.double() - cum[(k - 1).long()][:, None]
     np.testing.assert_allclose(w2.cpu().numpy(), expect.cpu().numpy(), rtol=RTOL, atol=1e-6)
+
+
+def test_push_of_another_batch_than_the_last_pull(tn, oracle):
+    """A push reuses what the last pull worked out about its batch only if the
+    signs are the same; same-shaped batches with other signs, pushes after
+    another table call, and pushes with no pull before them all take the full path."""
+    D = 16
+    rng = np.random.default_rng(21)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP)
+    vocab = 2000
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    a = random_batch(rng, 5, 700, vocab, ragged=False)
+    b = random_batch(rng, 5, 700, vocab, ragged=False)  # same lengths, other signs
+
+    def push(values, seed):
+        counts = [len(np.unique(v)) for v in values]
+        grads = synth.make_grads(counts, D, 0.01, seed=seed)
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+
+    push(a, 0)                      # no pull at all before the first push
+    pair.assert_rows_match(base)
+    check_pull(pair, a)
+    push(b, 1)                      # pull(a) then push(b)
+    pair.assert_rows_match(base)
+    check_pull(pair, b)
+    push(b, 2)                      # the matching push
+    push(b, 3)                      # and once more from the same analysis
+    pair.assert_rows_match(base)
+    check_pull(pair, a)
+    tn.ops.table_pull(pair.h, dev(base[:10].view(np.int64)), D)  # a table-level call in between
+    b2 = [v.copy() for v in a]
+    b2[2][5] = b[2][5]              # one sign differs
+    pair.o.pull_op(b2, [np.zeros((len(v) + 1, D), np.float32) for v in b2])
+    push(b2, 4)
+    pair.assert_rows_match(base)
