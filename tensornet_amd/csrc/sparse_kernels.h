@@ -561,16 +561,12 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
 }
 
 // Push: batch_show = occurrences, batch_click = sum of labels per distinct sign
-// (sparse_table_ops.cc:283-296; labels are narrowed to int as there).
-// Every distinct sign starts at show 1 / click 0 ...
-__global__ __launch_bounds__(256) void k_reset_counts(int32_t* __restrict__ ushow, int32_t* __restrict__ uclick,
-                                                      const DevStatus* status) {
+// (sparse_table_ops.cc:283-296; labels are narrowed to int as there), kept as
+// one {show, click} pair per distinct sign.  Every sign starts at show 1 / click 0 ...
+__global__ __launch_bounds__(256) void k_reset_counts(int2* __restrict__ ucnt, const DevStatus* status) {
     const uint32_t n = status->n_unique;
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
-        ushow[u] = 1;
-        uclick[u] = 0;
-    }
+    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) ucnt[u] = make_int2(1, 0);
 }
 
 constexpr int COUNT_TILE = 2048;
@@ -581,8 +577,8 @@ constexpr int COUNT_SLOTS = 4096;  // LDS table entries per tile (load factor <=
 // up in an LDS hash table and issues one global atomic per sign it saw.
 __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                    const uint32_t* __restrict__ u_of_gi, int32_t* ushow,
-                                                    int32_t* uclick, int with_click) {
+                                                    const uint32_t* __restrict__ u_of_gi, int2* ucnt,
+                                                    int with_click) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t keys[COUNT_SLOTS];
     __shared__ int32_t cnts[COUNT_SLOTS];
@@ -621,8 +617,8 @@ __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__
         for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
             const uint32_t u = keys[i];
             if (u == 0xFFFFFFFFu) continue;
-            if (cnts[i]) atomicAdd(&ushow[u], cnts[i]);
-            if (clks[i]) atomicAdd(&uclick[u], clks[i]);
+            if (cnts[i]) atomicAdd(&ucnt[u].x, cnts[i]);
+            if (clks[i]) atomicAdd(&ucnt[u].y, clks[i]);
         }
         __syncthreads();
     }
@@ -637,9 +633,9 @@ struct PushSrc {
     // op-level push: compact distinct lists of the remap + per-slot gradient matrices
     const uint64_t* uniq_sign;
     const uint32_t* uniq_slot;
+    const uint32_t* m_slot;  // slot of every member, in member-list order
     const uint32_t* ubase;
-    const int32_t* ushow;
-    const int32_t* uclick;
+    const int2* ucnt;        // {batch_show, batch_click} per distinct sign
     const SlotDesc* descs;
     int dim;
 };
@@ -680,48 +676,52 @@ __global__ __launch_bounds__(256) void k_group_insert(PushSrc src, int64_t n_hos
 
 constexpr int COMPACT_ITEMS = 4;
 
-// ...every group gets a number, a slice of the member list (two atomics per
-// 1024 table entries) and, when it has big_k members or more, a place in the
-// list of big groups...
+// Signs with big_k records or more are applied by one wavefront each.
+__device__ __forceinline__ bool is_big(uint32_t k, uint32_t big_k) { return k >= big_k; }
+
+// ...every group gets a number, a slice of the member list and, when it has
+// big_k members or more, a place in the list of big groups (three atomics per
+// 1024 table entries)...
 __global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupEntry* gt,
                                                        uint64_t* __restrict__ grp_sign,
                                                        uint32_t* __restrict__ grp_off,
                                                        uint32_t* __restrict__ grp_cnt,
                                                        uint32_t* __restrict__ big_list, uint32_t big_k) {
     __shared__ unsigned long long sh[4];
-    __shared__ uint32_t bases[2];
+    __shared__ uint32_t bases[3];
     const uint32_t n = status->gcap + 1;
     const uint32_t span = 256 * COMPACT_ITEMS;
     for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
         const uint32_t e0 = base + threadIdx.x * COMPACT_ITEMS;
         uint32_t ks[COMPACT_ITEMS];
-        unsigned long long mine = 0;  // (groups << 32) | members
+        unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t e = e0 + j;
             const uint32_t c = (e < n) ? gt[e].cnt : 0xFFFFFFFFu;
             ks[j] = (c != 0xFFFFFFFFu) ? c + 1 : 0;
             if (ks[j]) mine += (1ull << 32) | ks[j];
+            if (is_big(ks[j], big_k)) mine += 1ull << 48;
         }
         unsigned long long total;
         unsigned long long excl = block_excl_scan_256<unsigned long long>(mine, sh, &total);
-        if (threadIdx.x == 0 && total) {
-            bases[0] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32));
-            bases[1] = atomicAdd(&status->list_cursor, (uint32_t)total);
+        if (total) {
+            if (threadIdx.x == 0) bases[0] = atomicAdd(&status->list_cursor, (uint32_t)total);
+            if (threadIdx.x == 64) bases[1] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32) & 0xFFFFu);
+            if (threadIdx.x == 128 && (total >> 48)) bases[2] = atomicAdd(&status->n_big, (uint32_t)(total >> 48));
         }
         __syncthreads();
-        uint32_t g = bases[0] + (uint32_t)(excl >> 32);
-        uint32_t off = bases[1] + (uint32_t)excl;
+        uint32_t off = bases[0] + (uint32_t)excl;
+        uint32_t g = bases[1] + ((uint32_t)(excl >> 32) & 0xFFFFu);
+        uint32_t b = bases[2] + (uint32_t)(excl >> 48);
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t k = ks[j];
-            const bool big = k >= big_k;
-            const uint32_t b = wave_alloc(big, &status->n_big);
             if (k == 0) continue;
             const uint32_t e = e0 + j;
             gt[e].g = g;
             grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
             grp_off[g] = off;
             grp_cnt[g] = k;
-            if (big) big_list[b] = g;
+            if (is_big(k, big_k)) big_list[b++] = g;
             g++;
             off += k;
         }
@@ -745,7 +745,9 @@ __global__ __launch_bounds__(256) void k_group_fill(int64_t n_host, const uint32
 __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32_t* n_dev, const GroupEntry* gt,
                                                     const uint32_t* __restrict__ grp_off,
                                                     const uint32_t* __restrict__ gidx,
-                                                    const uint32_t* __restrict__ arrival, uint32_t* __restrict__ list,
+                                                    const uint32_t* __restrict__ arrival,
+                                                    const uint32_t* __restrict__ uniq_slot,
+                                                    uint32_t* __restrict__ list, uint32_t* __restrict__ m_slot,
                                                     uint32_t* __restrict__ g_of_u) {
     const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -759,7 +761,132 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
             for (uint32_t t = 0; t < k; t++) pos += mem[t] < (uint32_t)u;
         }
         list[off + pos] = (uint32_t)u;
+        if (uniq_slot) m_slot[off + pos] = uniq_slot[u];
         g_of_u[u] = en.g;
+    }
+}
+
+// ------------------------------------------ grouping by slot masks (N <= 128)
+// Within one slot all signs are distinct, so a sign has at most one record per
+// slot and its records in ascending order are its slots in ascending order.
+// With at most 128 slots the set of slots of a sign fits two words: records
+// mark their slot with one atomic (no value returned), and the place of a
+// record in its group's member list is the number of marked slots below its
+// own -- no arrival order, no sorting.  A cleared bit means "slot present"
+// (entries are filled with 0xFF bytes).
+struct MaskEntry {
+    uint64_t key;
+    uint64_t nlo, nhi;  // complemented slot masks
+    uint32_t g;
+    uint32_t pad;
+};
+
+__global__ __launch_bounds__(256) void k_fill_masks(MaskEntry* gt, const DevStatus* status) {
+    size_t n16 = ((size_t)status->gcap + 1) * 2;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4 v = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+    uint4* p = reinterpret_cast<uint4*>(gt);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void k_mask_insert(const uint64_t* __restrict__ uniq_sign,
+                                                     const uint32_t* __restrict__ uniq_slot, DevStatus* status,
+                                                     MaskEntry* gt, uint32_t* __restrict__ gidx) {
+    const uint32_t n = status->n_unique;
+    const uint32_t gcap = status->gcap;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
+        const uint64_t sign = uniq_sign[u];
+        uint32_t e;
+        if (sign == EMPTY_KEY) {
+            e = gcap;
+        } else {
+            uint32_t idx = (uint32_t)slot_of(sign, gcap);
+            for (;;) {
+                e = idx;
+                uint64_t k = gt[e].key;  // a stale EMPTY_KEY only costs a compare-and-swap
+                if (k == sign) break;
+                if (k == EMPTY_KEY) {
+                    uint64_t old = atomicCAS(ull(&gt[e].key), EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                }
+                idx = (idx + 1 == gcap) ? 0 : idx + 1;
+            }
+        }
+        gidx[u] = e;
+        const uint32_t sl = uniq_slot[u];
+        atomicAnd(ull(sl < 64 ? &gt[e].nlo : &gt[e].nhi), ~(1ull << (sl & 63)));
+    }
+}
+
+__global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEntry* gt,
+                                                      uint64_t* __restrict__ grp_sign,
+                                                      uint32_t* __restrict__ grp_off,
+                                                      uint32_t* __restrict__ grp_cnt,
+                                                      uint32_t* __restrict__ big_list, uint32_t big_k) {
+    __shared__ unsigned long long sh[4];
+    __shared__ uint32_t bases[3];
+    const uint32_t n = status->gcap + 1;
+    const uint32_t span = 256 * COMPACT_ITEMS;
+    for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
+        const uint32_t e0 = base + threadIdx.x * COMPACT_ITEMS;
+        uint32_t ks[COMPACT_ITEMS];
+        unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
+        for (int j = 0; j < COMPACT_ITEMS; j++) {
+            const uint32_t e = e0 + j;
+            ks[j] = (e < n) ? (uint32_t)(__popcll(~gt[e].nlo) + __popcll(~gt[e].nhi)) : 0;
+            if (ks[j]) mine += (1ull << 32) | ks[j];
+            if (ks[j] && is_big(ks[j], big_k)) mine += 1ull << 48;
+        }
+        unsigned long long total;
+        unsigned long long excl = block_excl_scan_256<unsigned long long>(mine, sh, &total);
+        if (total) {
+            if (threadIdx.x == 0) bases[0] = atomicAdd(&status->list_cursor, (uint32_t)total);
+            if (threadIdx.x == 64) bases[1] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32) & 0xFFFFu);
+            if (threadIdx.x == 128 && (total >> 48)) bases[2] = atomicAdd(&status->n_big, (uint32_t)(total >> 48));
+        }
+        __syncthreads();
+        uint32_t off = bases[0] + (uint32_t)excl;
+        uint32_t g = bases[1] + ((uint32_t)(excl >> 32) & 0xFFFFu);
+        uint32_t b = bases[2] + (uint32_t)(excl >> 48);
+        for (int j = 0; j < COMPACT_ITEMS; j++) {
+            const uint32_t k = ks[j];
+            if (k == 0) continue;
+            const uint32_t e = e0 + j;
+            gt[e].g = g;
+            grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
+            grp_off[g] = off;
+            grp_cnt[g] = k;
+            if (is_big(k, big_k)) big_list[b++] = g;
+            g++;
+            off += k;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, const MaskEntry* gt,
+                                                   const uint32_t* __restrict__ grp_off,
+                                                   const uint32_t* __restrict__ gidx,
+                                                   const uint32_t* __restrict__ uniq_slot,
+                                                   uint32_t* __restrict__ list, uint32_t* __restrict__ m_slot,
+                                                   uint32_t* __restrict__ g_of_u) {
+    const uint32_t n = status->n_unique;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
+        const MaskEntry& en = gt[gidx[u]];
+        const uint32_t sl = uniq_slot[u];
+        const uint64_t lo = ~en.nlo, hi = ~en.nhi;
+        uint32_t pos;
+        if (sl < 64)
+            pos = (uint32_t)__popcll(lo & ((1ull << sl) - 1ull));
+        else
+            pos = (uint32_t)__popcll(lo) + (uint32_t)__popcll(hi & ((1ull << (sl - 64)) - 1ull));
+        const uint32_t g = en.g;
+        const uint32_t at = grp_off[g] + pos;
+        list[at] = u;
+        m_slot[at] = sl;
+        g_of_u[u] = g;
     }
 }
 
@@ -796,22 +923,24 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
 }
 
 // -------------------------------------------------------------------- apply
-// Resolves record u to its gradient row and counts; false if the op's gradient
-// matrix has no such row.
-__device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, const float*& g, int& show, int& click) {
+// Resolves record u, found at place `at` of the member list, to its gradient
+// row and counts; false if the op's gradient matrix has no such row.
+__device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, uint32_t at, const float*& g, int& show,
+                                           int& click) {
     if (p.infos) {
         g = p.grads + (uint64_t)u * p.dim;
         show = p.infos[u].batch_show;
         click = p.infos[u].batch_click;
         return true;
     }
-    const uint32_t sl = p.uniq_slot[u];
+    const uint32_t sl = p.m_slot[at];
     const int64_t r = (int64_t)u - (int64_t)p.ubase[sl];
     const SlotDesc& d = p.descs[sl];
     if (r >= d.rows) return false;
     g = d.grads + (uint64_t)r * p.dim;
-    show = p.ushow[u];
-    click = p.uclick[u];
+    const int2 c = p.ucnt[u];
+    show = c.x;
+    click = c.y;
     return true;
 }
 
@@ -861,8 +990,9 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
         const uint32_t k = grp_cnt[g];
-        if (k >= big_k) continue;
-        const uint32_t* mem = list + grp_off[g];
+        if (is_big(k, big_k)) continue;
+        const uint32_t off = grp_off[g];
+        const uint32_t* mem = list + off;
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         float4 w = reinterpret_cast<float4*>(wp)[sub];
@@ -882,7 +1012,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         bool any = false;
         const float* gp;
         int nshow = 0, nclick = 0;
-        bool nok = src_record(src, mem[0], gp, nshow, nclick);
+        bool nok = src_record(src, mem[0], off, gp, nshow, nclick);
         float4 gnext = make_float4(0.f, 0.f, 0.f, 0.f);
         if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
         for (uint32_t j = 0; j < k; j++) {
@@ -890,7 +1020,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
             const int bshow = nshow, bclick = nclick;
             const bool ok = nok;
             if (j + 1 < k) {
-                nok = src_record(src, mem[j + 1], gp, nshow, nclick);
+                nok = src_record(src, mem[j + 1], off + j + 1, gp, nshow, nclick);
                 if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
             }
             if (!ok) {
@@ -950,14 +1080,16 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
     }
 }
 
-constexpr int BIG_DIM_MAX = 512;    // largest dim k_apply_big stages in LDS
-constexpr int BIG_GBUF = 2048;      // floats of gradient staging per wavefront
+constexpr int BIG_DIM_MAX = 128;    // largest dim k_apply_big stages in LDS
+constexpr int BIG_GBUF = 2176;      // floats of gradient staging per wavefront
 
 // A sign with many records (it occurs in many slots) would make one lane
 // group chase a long chain of dependent loads.  Here one wavefront owns the
-// sign: the row lives in LDS, the gradients of up to 64 records at a time are
-// fetched by all lanes in parallel and then applied strictly in record order,
-// lanes working on different elements of the row.
+// sign: the row lives in LDS and the (already ordered) records are taken up
+// to 64 at a time: all lanes resolve and fetch the gradients in parallel,
+// then the records are applied strictly in order -- for AdaGrad the g2sum
+// chain by one lane, the square roots by one lane per record, the element
+// updates by one lane per element.
 template <int KIND>
 __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src, DevStatus* status,
                                                   const uint32_t* __restrict__ big_list,
@@ -969,17 +1101,22 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
     __shared__ float gbuf[BIG_GBUF];
     __shared__ const float* gptr[64];
     __shared__ int gshow[64], gclick[64], gok[64];
+    __shared__ double msq[64];
+    __shared__ float den[64];
     const int D = s.D;
+    const int Dp = D + 1;  // padded staging row: lanes walking down a column hit different banks
     const int lane = threadIdx.x;
     const uint32_t n_big = status->n_big;
-    const int per_chunk = (BIG_GBUF / D) < 64 ? (BIG_GBUF / D) : 64;
+    const int per_chunk = (BIG_GBUF / Dp) < 64 ? (BIG_GBUF / Dp) : 64;
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+    const bool pow2 = (D & (D - 1)) == 0;
+    const double inv_d = 1.0 / (double)D;  // exact when D is a power of two
     for (uint32_t bi = blockIdx.x; bi < n_big; bi += gridDim.x) {
         const uint32_t g = big_list[bi];
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;
         const uint32_t k = grp_cnt[g];
-        const uint32_t* mem = list + grp_off[g];
+        const uint32_t off = grp_off[g];
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         for (int i = lane; i < D; i += 64) {
@@ -989,6 +1126,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                 rb[i] = sp[D + i];
             }
         }
+        // lane 0 carries the scalars of the row
         float g2sum = 0.f, show = 0.f, click = 0.f;
         int delta_show = 0;
         if (KIND == OPT_ADAGRAD) {
@@ -1005,7 +1143,8 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             if (lane < cn) {
                 const float* gp = nullptr;
                 int sh = 0, ck = 0;
-                const bool ok = src_record(src, mem[c0 + lane], gp, sh, ck);
+                const uint32_t at = off + c0 + lane;
+                const bool ok = src_record(src, list[at], at, gp, sh, ck);
                 gptr[lane] = gp;
                 gshow[lane] = sh;
                 gclick[lane] = ck;
@@ -1014,31 +1153,58 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             __syncthreads();
             for (int t = lane; t < cn * D; t += 64) {
                 const int m = t / D, i = t - m * D;
-                gbuf[t] = gok[m] ? gptr[m][i] : 0.f;
+                gbuf[m * Dp + i] = gok[m] ? gptr[m][i] : 0.f;
             }
             __syncthreads();
-            for (int m = 0; m < cn; m++) {
-                if (!gok[m]) {
-                    if (lane == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-                    continue;
-                }
-                any = true;
-                const float* gr = gbuf + m * D;
-                if (KIND == OPT_ADAGRAD) {
-                    show += (float)gshow[m];
-                    click += (float)gclick[m];
-                    double tot = 0.0;  // every lane adds up all D products in element order
+            if (KIND == OPT_ADAGRAD) {
+                if (lane < cn) {  // add_g2sum / dim of record `lane`: double sum of float products, element order
+                    const float* gr = gbuf + lane * Dp;
+                    double tot = 0.0;
                     for (int i = 0; i < D; i++) tot += (double)(gr[i] * gr[i]);
-                    g2sum = (float)((double)g2sum + tot / (double)D);
-                    const float den = o.eps + sqrtf(g2sum);
-                    for (int i = lane; i < D; i += 64) rw[i] -= o.lr * gr[i] / den;
-                } else if (KIND == OPT_ADAM) {
-                    delta_show += gshow[m];
-                    for (int i = lane; i < D; i += 64) adam_elem(o, c1, c2, gr[i], rw[i], ra[i], rb[i]);
-                } else {
-                    delta_show += gshow[m];
-                    for (int i = lane; i < D; i += 64) ftrl_elem(o, gr[i], rw[i], ra[i], rb[i]);
+                    msq[lane] = pow2 ? tot * inv_d : tot / (double)D;
                 }
+                __syncthreads();
+                if (lane == 0) {  // g2sum after every record (float += double, rounded each time)
+                    for (int m = 0; m < cn; m++) {
+                        if (!gok[m]) continue;
+                        show += (float)gshow[m];
+                        click += (float)gclick[m];
+                        g2sum = (float)((double)g2sum + msq[m]);
+                        den[m] = g2sum;
+                    }
+                }
+                __syncthreads();
+                if (lane < cn) den[lane] = o.eps + sqrtf(den[lane]);
+                __syncthreads();
+                for (int i = lane; i < D; i += 64) {
+                    float w = rw[i];
+                    for (int m = 0; m < cn; m++)
+                        if (gok[m]) w -= o.lr * gbuf[m * Dp + i] / den[m];
+                    rw[i] = w;
+                }
+            } else {
+                if (lane == 0)
+                    for (int m = 0; m < cn; m++)
+                        if (gok[m]) delta_show += gshow[m];
+                for (int i = lane; i < D; i += 64) {
+                    float w = rw[i], a = ra[i], b = rb[i];
+                    for (int m = 0; m < cn; m++) {
+                        if (!gok[m]) continue;
+                        if (KIND == OPT_ADAM)
+                            adam_elem(o, c1, c2, gbuf[m * Dp + i], w, a, b);
+                        else
+                            ftrl_elem(o, gbuf[m * Dp + i], w, a, b);
+                    }
+                    rw[i] = w;
+                    ra[i] = a;
+                    rb[i] = b;
+                }
+            }
+            for (int m = 0; m < cn; m++) {
+                if (gok[m])
+                    any = true;
+                else if (lane == 0)
+                    atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
             }
             __syncthreads();
         }
@@ -1083,15 +1249,16 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;
         const uint32_t k = grp_cnt[g];
-        if (k >= big_k) continue;
-        const uint32_t* mem = list + grp_off[g];
+        if (is_big(k, big_k)) continue;
+        const uint32_t off = grp_off[g];
+        const uint32_t* mem = list + off;
         float* w = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         for (uint32_t j = 0; j < k; j++) {
             const uint32_t u = mem[j];
             const float* gp;
             int bshow, bclick;
-            if (!src_record(src, u, gp, bshow, bclick)) {
+            if (!src_record(src, u, off + j, gp, bshow, bclick)) {
                 atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
                 continue;
             }

@@ -299,13 +299,13 @@ struct Plan {
     uint32_t* u_of_gi;     // lookup -> index of its distinct sign
     uint64_t* uniq_sign;   // per-slot distinct signs, slot-major, first-occurrence order
     uint32_t* uniq_slot;
-    int32_t* ushow;
-    int32_t* uclick;
+    int2* ucnt;            // {batch_show, batch_click} per distinct sign (push)
     uint64_t* grp_sign;    // distinct signs over all slots
     uint32_t* grp_row;     // their table rows
     uint32_t* grp_off;
     uint32_t* grp_cnt;
     uint32_t* list;        // members (indices into uniq_*) of every group, ascending
+    uint32_t* m_slot;      // slot of every member, same order
     uint32_t* g_of_u;      // record -> its group
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     uint32_t* newlist;     // groups whose row was inserted by the pull
@@ -320,7 +320,7 @@ struct Scratch {
     uint32_t* tilesum;
     uint32_t* tileoff;
     uint32_t ntiles;
-    GroupEntry* gt;
+    void* gt;  // GroupEntry[] or MaskEntry[]
     uint32_t* gidx;
     uint32_t* ord;
     uint32_t* arrival;
@@ -339,13 +339,14 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_off = c.take<uint32_t>(n);
     p.grp_cnt = c.take<uint32_t>(n);
     p.list = c.take<uint32_t>(n);
+    p.m_slot = c.take<uint32_t>(n);
     p.g_of_u = c.take<uint32_t>(n);
     p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
     p.newlist = c.take<uint32_t>(n);
 }
 
 void carve_group_scratch(Carver& c, Scratch& w, size_t n) {
-    w.gt = c.take<GroupEntry>(group_cap(n) + 1);
+    w.gt = c.take<MaskEntry>(group_cap(n) + 1);  // the larger of the two entry types
     w.gidx = c.take<uint32_t>(n);
     w.ord = c.take<uint32_t>(n);
     w.arrival = c.take<uint32_t>(n);
@@ -360,8 +361,7 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     p.u_of_gi = c.take<uint32_t>(L);
     p.uniq_sign = c.take<uint64_t>(L);
     p.uniq_slot = c.take<uint32_t>(L);
-    p.ushow = c.take<int32_t>(L);
-    p.uclick = c.take<int32_t>(L);
+    p.ucnt = c.take<int2>(L);
     carve_groups(c, p, L);
     return align_up(c.off, 256);
 }
@@ -432,26 +432,44 @@ PushSrc op_source(const Plan& p, int dim) {
     src.uniq_sign = p.uniq_sign;
     src.uniq_slot = p.uniq_slot;
     src.ubase = p.ubase;
-    src.ushow = p.ushow;
-    src.uclick = p.uclick;
+    src.m_slot = p.m_slot;
+    src.ucnt = p.ucnt;
     src.descs = p.descs;
     src.dim = dim;
     return src;
 }
 
 // Groups n records (n_host of them, or status->n_unique) by sign: group arrays
-// and member lists in ascending record order.
+// and member lists in ascending record order.  Works for any records: arrival
+// order by atomics, then every record finds its place among its group's members.
 void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_t n_host, int64_t n_upper,
                      uint32_t big_k, DevStatus* ds, hipStream_t st) {
     const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
+    GroupEntry* gt = static_cast<GroupEntry*>(w.gt);
     const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
     const int tblocks = launch_grid((int64_t)group_cap(n_upper) + 1, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_fill_groups, dim3(tblocks), dim3(256), st, w.gt, ds);
-    TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, w.gt, w.gidx, w.ord);
+    TN_LAUNCH(k_fill_groups, dim3(tblocks), dim3(256), st, gt, ds);
+    TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, gt, w.gidx, w.ord);
     TN_LAUNCH(k_group_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
-              dim3(256), st, ds, w.gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
-    TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, p.grp_off, w.gidx, w.ord, w.arrival);
-    TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, w.gt, p.grp_off, w.gidx, w.arrival, p.list,
+              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
+    TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.ord, w.arrival);
+    TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.arrival,
+              src.uniq_slot, p.list, p.m_slot, p.g_of_u);
+}
+
+constexpr int MASK_SLOTS = 128;
+
+// The same result for the distinct signs of an op with at most 128 slots, from slot masks.
+void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint32_t big_k, DevStatus* ds,
+                          hipStream_t st) {
+    MaskEntry* gt = static_cast<MaskEntry*>(w.gt);
+    const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
+    const int tblocks = launch_grid(2 * (int64_t)group_cap(n_upper) + 2, 256, GRID_CAP * 2);
+    TN_LAUNCH(k_fill_masks, dim3(tblocks), dim3(256), st, gt, ds);
+    TN_LAUNCH(k_mask_insert, dim3(gblocks), dim3(256), st, p.uniq_sign, p.uniq_slot, ds, gt, w.gidx);
+    TN_LAUNCH(k_mask_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
+              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
+    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, p.grp_off, w.gidx, p.uniq_slot, p.list, p.m_slot,
               p.g_of_u);
 }
 
@@ -473,7 +491,10 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
               w.tileoff, p.ubase, p.uniq_sign, p.uniq_slot);
     TN_LAUNCH(k_write_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.dt, w.tidx, w.flag8,
               p.u_of_gi, for_pull ? 1 : 0);
-    launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ds, st);
+    if (N <= MASK_SLOTS)
+        launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ds, st);
+    else
+        launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ds, st);
     if (for_pull)
         TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, &ds->n_groups, p.grp_row,
                   p.newlist, ds, (uint32_t)DEV_ERR_TABLE_FULL);
@@ -940,10 +961,10 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         launch_build_plan(t, p, w, N, (uint32_t)L, false, st);
     }
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ushow, p.uclick, ds);
+    TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ucnt, ds);
     // AdaGrad is the only optimizer that reads batch_click
     TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256), st,
-              p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ushow, p.uclick, t->opt->kind == OPT_ADAGRAD ? 1 : 0);
+              p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt, t->opt->kind == OPT_ADAGRAD ? 1 : 0);
     launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));

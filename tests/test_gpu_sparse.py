@@ -412,3 +412,51 @@ def test_push_of_another_batch_than_the_last_pull(tn, oracle):
     pair.o.pull_op(b2, [np.zeros((len(v) + 1, D), np.float32) for v in b2])
     push(b2, 4)
     pair.assert_rows_match(base)
+
+
+@pytest.mark.parametrize("opt,hyper", [("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP)])
+def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper):
+    """SparseTable::Push applies records in array order however often a sign repeats:
+    a few records, a few hundred (one wavefront per sign) and more than fit in LDS."""
+    D = 8
+    rng = np.random.default_rng(13)
+    pair = Pair(tn, oracle, opt, D, hyper)
+    base = pair.populate(synth.splitmix64(np.arange(1, 41, dtype=np.uint64)))
+    req = np.concatenate([np.full(5000, base[0]), np.full(300, base[1]), np.full(17, base[2]), np.full(15, base[3]),
+                          base[rng.integers(4, 40, 700)]])
+    req = req[rng.permutation(len(req))]
+    n = len(req)
+    infos = np.zeros(n, dtype=oracle.sign_info_dtype)
+    infos["sign"] = req
+    infos["batch_show"] = rng.integers(1, 4, n)
+    infos["batch_click"] = rng.integers(0, 2, n)
+    grads = (rng.standard_normal((n, D)) * 0.01).astype(np.float32)
+    assert pair.o.push(infos, grads) == 0
+    rec = tn.ops.make_sign_infos(dev(req.view(np.int64)), dev(infos["batch_show"].astype(np.int64)),
+                                 dev(infos["batch_click"].astype(np.int64)))
+    tn.ops.table_push(pair.h, rec, dev(grads))
+    tn.ops.sparse_table_sync(pair.h)
+    pair.assert_rows_match(base)
+
+
+@pytest.mark.parametrize("slots", [70, 128, 129, 300])
+def test_many_slots(tn, oracle, slots):
+    """Slot counts on both sides of the 64- and 128-slot boundaries of the
+    grouping by slot masks; a handful of signs occur in (nearly) every slot."""
+    D = 16
+    rng = np.random.default_rng(slots)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP)
+    vocab = 400
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    hot = base[:5].view(np.int64)
+    for b in range(2):
+        values = []
+        for s_ in range(slots):
+            n = int(rng.integers(0, 40))
+            v = base.view(np.int64)[rng.integers(0, vocab, n)]
+            values.append(np.concatenate([v, hot[: int(rng.integers(0, 6))]]))
+        counts = check_pull(pair, values)
+        grads = [(rng.standard_normal((int(u), D)) * 0.05).astype(np.float32) for u in counts]
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+        pair.assert_rows_match(base)
