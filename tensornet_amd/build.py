@@ -32,6 +32,10 @@ FLAGS = [
 ]
 
 
+HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "host_mirror_test.cc")
+HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "host_mirror_test")
+
+
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc] + FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", CSRC]
@@ -42,6 +46,18 @@ def build(verbose=True):
     return LIB
 
 
+def build_host_test(verbose=True):
+    """Builds the C++ program that drives the library through include/tensornet_amd.hpp."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "-std=c++17", "-O1", "-I", os.path.join(ROOT, "include"), HOST_TEST_SRC, "-L", HERE,
+           "-ltensornet_amd", "-Wl,-rpath,$ORIGIN/../../tensornet_amd", "-o", HOST_TEST_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     build()
+    build_host_test()
     sys.exit(0)

@@ -633,7 +633,6 @@ struct PushSrc {
     // op-level push: compact distinct lists of the remap + per-slot gradient matrices
     const uint64_t* uniq_sign;
     const uint32_t* uniq_slot;
-    const uint32_t* m_slot;  // slot of every member, in member-list order
     const uint32_t* ubase;
     const int2* ucnt;        // {batch_show, batch_click} per distinct sign
     const SlotDesc* descs;
@@ -674,7 +673,7 @@ __global__ __launch_bounds__(256) void k_group_insert(PushSrc src, int64_t n_hos
     }
 }
 
-constexpr int COMPACT_ITEMS = 4;
+constexpr int COMPACT_ITEMS = 16;
 
 // Signs with big_k records or more are applied by one wavefront each.
 __device__ __forceinline__ bool is_big(uint32_t k, uint32_t big_k) { return k >= big_k; }
@@ -692,11 +691,10 @@ __global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupE
     const uint32_t n = status->gcap + 1;
     const uint32_t span = 256 * COMPACT_ITEMS;
     for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
-        const uint32_t e0 = base + threadIdx.x * COMPACT_ITEMS;
         uint32_t ks[COMPACT_ITEMS];
         unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
         for (int j = 0; j < COMPACT_ITEMS; j++) {
-            const uint32_t e = e0 + j;
+            const uint32_t e = base + j * 256 + threadIdx.x;  // neighbouring lanes read neighbouring entries
             const uint32_t c = (e < n) ? gt[e].cnt : 0xFFFFFFFFu;
             ks[j] = (c != 0xFFFFFFFFu) ? c + 1 : 0;
             if (ks[j]) mine += (1ull << 32) | ks[j];
@@ -716,7 +714,7 @@ __global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupE
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t k = ks[j];
             if (k == 0) continue;
-            const uint32_t e = e0 + j;
+            const uint32_t e = base + j * 256 + threadIdx.x;
             gt[e].g = g;
             grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
             grp_off[g] = off;
@@ -747,8 +745,7 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
                                                     const uint32_t* __restrict__ gidx,
                                                     const uint32_t* __restrict__ arrival,
                                                     const uint32_t* __restrict__ uniq_slot,
-                                                    uint32_t* __restrict__ list, uint32_t* __restrict__ m_slot,
-                                                    uint32_t* __restrict__ g_of_u) {
+                                                    uint2* __restrict__ list, uint32_t* __restrict__ g_of_u) {
     const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
@@ -760,8 +757,7 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
             const uint32_t* mem = arrival + off;
             for (uint32_t t = 0; t < k; t++) pos += mem[t] < (uint32_t)u;
         }
-        list[off + pos] = (uint32_t)u;
-        if (uniq_slot) m_slot[off + pos] = uniq_slot[u];
+        list[off + pos] = make_uint2((uint32_t)u, uniq_slot ? uniq_slot[u] : 0u);
         g_of_u[u] = en.g;
     }
 }
@@ -776,9 +772,9 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
 // (entries are filled with 0xFF bytes).
 struct MaskEntry {
     uint64_t key;
-    uint64_t nlo, nhi;  // complemented slot masks
-    uint32_t g;
-    uint32_t pad;
+    uint32_t g;         // number of the group
+    uint32_t off;       // start of its member list
+    uint64_t nlo, nhi;  // complemented slot masks (16-byte aligned)
 };
 
 __global__ __launch_bounds__(256) void k_fill_masks(MaskEntry* gt, const DevStatus* status) {
@@ -829,12 +825,15 @@ __global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEnt
     const uint32_t n = status->gcap + 1;
     const uint32_t span = 256 * COMPACT_ITEMS;
     for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
-        const uint32_t e0 = base + threadIdx.x * COMPACT_ITEMS;
         uint32_t ks[COMPACT_ITEMS];
         unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
         for (int j = 0; j < COMPACT_ITEMS; j++) {
-            const uint32_t e = e0 + j;
-            ks[j] = (e < n) ? (uint32_t)(__popcll(~gt[e].nlo) + __popcll(~gt[e].nhi)) : 0;
+            const uint32_t e = base + j * 256 + threadIdx.x;  // neighbouring lanes read neighbouring entries
+            ks[j] = 0;
+            if (e < n) {
+                const ulonglong2 m = *reinterpret_cast<const ulonglong2*>(&gt[e].nlo);
+                ks[j] = (uint32_t)(__popcll(~m.x) + __popcll(~m.y));
+            }
             if (ks[j]) mine += (1ull << 32) | ks[j];
             if (ks[j] && is_big(ks[j], big_k)) mine += 1ull << 48;
         }
@@ -852,8 +851,8 @@ __global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEnt
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t k = ks[j];
             if (k == 0) continue;
-            const uint32_t e = e0 + j;
-            gt[e].g = g;
+            const uint32_t e = base + j * 256 + threadIdx.x;
+            *reinterpret_cast<uint2*>(&gt[e].g) = make_uint2(g, off);
             grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
             grp_off[g] = off;
             grp_cnt[g] = k;
@@ -866,27 +865,24 @@ __global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEnt
 }
 
 __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, const MaskEntry* gt,
-                                                   const uint32_t* __restrict__ grp_off,
                                                    const uint32_t* __restrict__ gidx,
                                                    const uint32_t* __restrict__ uniq_slot,
-                                                   uint32_t* __restrict__ list, uint32_t* __restrict__ m_slot,
-                                                   uint32_t* __restrict__ g_of_u) {
+                                                   uint2* __restrict__ list, uint32_t* __restrict__ g_of_u) {
     const uint32_t n = status->n_unique;
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
-        const MaskEntry& en = gt[gidx[u]];
+        const MaskEntry* en = &gt[gidx[u]];
+        const ulonglong2 m = *reinterpret_cast<const ulonglong2*>(&en->nlo);
+        const uint2 go = *reinterpret_cast<const uint2*>(&en->g);
         const uint32_t sl = uniq_slot[u];
-        const uint64_t lo = ~en.nlo, hi = ~en.nhi;
+        const uint64_t lo = ~m.x, hi = ~m.y;
         uint32_t pos;
         if (sl < 64)
             pos = (uint32_t)__popcll(lo & ((1ull << sl) - 1ull));
         else
             pos = (uint32_t)__popcll(lo) + (uint32_t)__popcll(hi & ((1ull << (sl - 64)) - 1ull));
-        const uint32_t g = en.g;
-        const uint32_t at = grp_off[g] + pos;
-        list[at] = u;
-        m_slot[at] = sl;
-        g_of_u[u] = g;
+        list[go.y + pos] = make_uint2(u, sl);
+        g_of_u[u] = go.x;
     }
 }
 
@@ -923,17 +919,17 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
 }
 
 // -------------------------------------------------------------------- apply
-// Resolves record u, found at place `at` of the member list, to its gradient
-// row and counts; false if the op's gradient matrix has no such row.
-__device__ __forceinline__ bool src_record(const PushSrc& p, uint32_t u, uint32_t at, const float*& g, int& show,
-                                           int& click) {
+// Resolves a member {record u, slot} to its gradient row and counts; false if
+// the op's gradient matrix has no such row.
+__device__ __forceinline__ bool src_record(const PushSrc& p, uint2 member, const float*& g, int& show, int& click) {
+    const uint32_t u = member.x;
     if (p.infos) {
         g = p.grads + (uint64_t)u * p.dim;
         show = p.infos[u].batch_show;
         click = p.infos[u].batch_click;
         return true;
     }
-    const uint32_t sl = p.m_slot[at];
+    const uint32_t sl = member.y;
     const int64_t r = (int64_t)u - (int64_t)p.ubase[sl];
     const SlotDesc& d = p.descs[sl];
     if (r >= d.rows) return false;
@@ -978,7 +974,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                                                    const uint32_t* __restrict__ grp_row,
                                                    const uint32_t* __restrict__ grp_off,
                                                    const uint32_t* __restrict__ grp_cnt,
-                                                   const uint32_t* __restrict__ list, uint32_t big_k) {
+                                                   const uint2* __restrict__ list, uint32_t big_k) {
     const uint32_t n_groups = status->n_groups;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;                       // my float4 inside the row
@@ -991,8 +987,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
-        const uint32_t off = grp_off[g];
-        const uint32_t* mem = list + off;
+        const uint2* mem = list + grp_off[g];
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         float4 w = reinterpret_cast<float4*>(wp)[sub];
@@ -1012,7 +1007,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         bool any = false;
         const float* gp;
         int nshow = 0, nclick = 0;
-        bool nok = src_record(src, mem[0], off, gp, nshow, nclick);
+        bool nok = src_record(src, mem[0], gp, nshow, nclick);
         float4 gnext = make_float4(0.f, 0.f, 0.f, 0.f);
         if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
         for (uint32_t j = 0; j < k; j++) {
@@ -1020,7 +1015,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
             const int bshow = nshow, bclick = nclick;
             const bool ok = nok;
             if (j + 1 < k) {
-                nok = src_record(src, mem[j + 1], off + j + 1, gp, nshow, nclick);
+                nok = src_record(src, mem[j + 1], gp, nshow, nclick);
                 if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
             }
             if (!ok) {
@@ -1096,7 +1091,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                                                   const uint32_t* __restrict__ grp_row,
                                                   const uint32_t* __restrict__ grp_off,
                                                   const uint32_t* __restrict__ grp_cnt,
-                                                  const uint32_t* __restrict__ list) {
+                                                  const uint2* __restrict__ list) {
     __shared__ float rw[BIG_DIM_MAX], ra[BIG_DIM_MAX], rb[BIG_DIM_MAX];
     __shared__ float gbuf[BIG_GBUF];
     __shared__ const float* gptr[64];
@@ -1143,8 +1138,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             if (lane < cn) {
                 const float* gp = nullptr;
                 int sh = 0, ck = 0;
-                const uint32_t at = off + c0 + lane;
-                const bool ok = src_record(src, list[at], at, gp, sh, ck);
+                const bool ok = src_record(src, list[off + c0 + lane], gp, sh, ck);
                 gptr[lane] = gp;
                 gshow[lane] = sh;
                 gclick[lane] = ck;
@@ -1241,7 +1235,7 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
                                                       const uint32_t* __restrict__ grp_row,
                                                       const uint32_t* __restrict__ grp_off,
                                                       const uint32_t* __restrict__ grp_cnt,
-                                                      const uint32_t* __restrict__ list, uint32_t big_k) {
+                                                      const uint2* __restrict__ list, uint32_t big_k) {
     const uint32_t n_groups = status->n_groups;
     const int D = s.D;
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -1250,15 +1244,13 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
         if (row == NO_ROW) continue;
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
-        const uint32_t off = grp_off[g];
-        const uint32_t* mem = list + off;
+        const uint2* mem = list + grp_off[g];
         float* w = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         for (uint32_t j = 0; j < k; j++) {
-            const uint32_t u = mem[j];
             const float* gp;
             int bshow, bclick;
-            if (!src_record(src, u, off + j, gp, bshow, bclick)) {
+            if (!src_record(src, mem[j], gp, bshow, bclick)) {
                 atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
                 continue;
             }

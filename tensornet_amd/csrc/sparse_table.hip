@@ -304,8 +304,7 @@ struct Plan {
     uint32_t* grp_row;     // their table rows
     uint32_t* grp_off;
     uint32_t* grp_cnt;
-    uint32_t* list;        // members (indices into uniq_*) of every group, ascending
-    uint32_t* m_slot;      // slot of every member, same order
+    uint2* list;           // members {index into uniq_*, slot} of every group, ascending
     uint32_t* g_of_u;      // record -> its group
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     uint32_t* newlist;     // groups whose row was inserted by the pull
@@ -338,8 +337,7 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_row = c.take<uint32_t>(n);
     p.grp_off = c.take<uint32_t>(n);
     p.grp_cnt = c.take<uint32_t>(n);
-    p.list = c.take<uint32_t>(n);
-    p.m_slot = c.take<uint32_t>(n);
+    p.list = c.take<uint2>(n);
     p.g_of_u = c.take<uint32_t>(n);
     p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
     p.newlist = c.take<uint32_t>(n);
@@ -432,7 +430,6 @@ PushSrc op_source(const Plan& p, int dim) {
     src.uniq_sign = p.uniq_sign;
     src.uniq_slot = p.uniq_slot;
     src.ubase = p.ubase;
-    src.m_slot = p.m_slot;
     src.ucnt = p.ucnt;
     src.descs = p.descs;
     src.dim = dim;
@@ -454,7 +451,7 @@ void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_
               dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
     TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.ord, w.arrival);
     TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.arrival,
-              src.uniq_slot, p.list, p.m_slot, p.g_of_u);
+              src.uniq_slot, p.list, p.g_of_u);
 }
 
 constexpr int MASK_SLOTS = 128;
@@ -469,8 +466,7 @@ void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint
     TN_LAUNCH(k_mask_insert, dim3(gblocks), dim3(256), st, p.uniq_sign, p.uniq_slot, ds, gt, w.gidx);
     TN_LAUNCH(k_mask_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
               dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
-    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, p.grp_off, w.gidx, p.uniq_slot, p.list, p.m_slot,
-              p.g_of_u);
+    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, p.list, p.g_of_u);
 }
 
 // Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids
