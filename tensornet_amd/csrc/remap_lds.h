@@ -1,0 +1,313 @@
+// Key remap through LDS: the fast path of the per-slot first-occurrence remap
+// (core/kernels/sparse_table_ops.cc:119-131) for large batches.
+//
+// A global hash table costs one or two random 64-byte granules and up to two
+// device atomics per lookup.  Here the lookups of every slot are first
+// partitioned by a hash of the sign into buckets of ~1536 lookups (an LDS
+// histogram and an LDS cursor per 4096-lookup tile: the only global atomics
+// are one per tile and bucket); then one workgroup per bucket builds the
+// bucket's hash table in LDS -- sign, smallest position, number of
+// occurrences -- and writes for every lookup the position of its sign's first
+// occurrence.  All lookups of one (slot, sign) land in one bucket, a bucket
+// belongs to one slot, and the positions it writes to lie inside that slot's
+// window of the concatenated lookup order, so the scatter back stays local.
+//
+//   k_lds_hist     bucket sizes (+ copy of the signs for the plan)
+//   k_lds_offsets  exclusive scan of the bucket sizes (one workgroup)
+//   k_lds_scatter  {sign, position} records grouped by bucket
+//   k_lds_dedup    per bucket: LDS hash table -> first_of[position], occurrence counts
+//   k_lds_flags    first-occurrence flags per tile (coalesced: first_of[gi] == gi)
+//   k_scan_tiles   (shared with the global-table path)
+//   k_lds_assign   ranks, distinct lists, show counts
+//   k_lds_mapped   mapped ids and the per-lookup distinct index
+//
+// If an LDS table ever overflows (more distinct signs in a bucket than it has
+// room for) DEV_ERR_REMAP_OVERFLOW is raised; every index written stays in
+// bounds and the host repeats the call on the global-table path.
+#ifndef TN_REMAP_LDS_H_
+#define TN_REMAP_LDS_H_
+
+#include "sparse_kernels.h"
+
+namespace tn {
+
+constexpr int LDS_TILE = 4096;          // lookups per tile of the partition kernels
+constexpr int LDS_TILE_ITEMS = LDS_TILE / 256;
+constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
+constexpr int LDS_BUCKET_TARGET = 1536; // average lookups per bucket
+constexpr int LDS_MAX_SUB = 2048;       // buckets per slot at most
+constexpr int LDS_TABLE = 4096;         // entries of a bucket's LDS hash table
+
+// In this mode SlotDesc::tbase is the slot's first bucket and SlotDesc::tcap its number of buckets.
+__device__ __forceinline__ uint32_t bucket_of(const SlotDesc& d, uint64_t sign) {
+    return d.tbase + (uint32_t)__umul64hi(mix64(sign), (uint64_t)d.tcap);
+}
+
+// One pass over a tile: calls f(gi, slot, sign) for each of its lookups.
+template <typename F>
+__device__ __forceinline__ void for_tile(uint32_t tile, const SlotDesc* descs, const uint32_t* lb, int N, uint32_t L,
+                                         F f) {
+#pragma unroll 4
+    for (int j = 0; j < LDS_TILE_ITEMS; j++) {
+        const uint32_t gi = tile * LDS_TILE + j * 256 + threadIdx.x;
+        if (gi >= L) break;
+        const int sl = find_slot(lb, N, gi);
+        f(gi, sl, (uint64_t)descs[sl].values[gi - lb[sl]]);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
+}
+
+// Also presets first_of / cnt_at to "every lookup is its own first occurrence",
+// which is what a lookup keeps if an overflow leaves it unprocessed.
+__global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
+                                                  int N, uint32_t L, uint32_t* bcount,
+                                                  uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ first_of,
+                                                  uint32_t* __restrict__ cnt_at, DevStatus* status) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t hist[LDS_SPAN];
+    load_lbase(lb, lbase, N);
+    const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
+        __syncthreads();
+        const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;  // lowest bucket the tile can touch
+        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, uint64_t sign) {
+            vals_copy[gi] = sign;
+            first_of[gi] = gi;
+            cnt_at[gi] = 1;
+            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+            if (local < LDS_SPAN)
+                atomicAdd(&hist[local], 1u);
+            else
+                atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+        });
+        __syncthreads();
+        for (int i = threadIdx.x; i < LDS_SPAN; i += 256)
+            if (hist[i]) atomicAdd(&bcount[b0 + i], hist[i]);
+        __syncthreads();
+    }
+}
+
+// bstart[b] = number of lookups in buckets before b; bcursor starts as a copy.
+__global__ __launch_bounds__(1024) void k_lds_offsets(const uint32_t* __restrict__ bcount, uint32_t* __restrict__ bstart,
+                                                      uint32_t* __restrict__ bcursor, uint32_t nbuckets) {
+    __shared__ uint32_t wsum[16];
+    __shared__ uint32_t carry_sh;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) carry_sh = 0;
+    __syncthreads();
+    for (uint32_t start = 0; start < nbuckets; start += 1024) {
+        const uint32_t i = start + threadIdx.x;
+        const uint32_t v = (i < nbuckets) ? bcount[i] : 0;
+        uint32_t inc = v;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t t = __shfl_up(inc, o);
+            if (lane >= o) inc += t;
+        }
+        if (lane == 63) wsum[wave] = inc;
+        __syncthreads();
+        uint32_t base = carry_sh;
+        for (int wv = 0; wv < wave; wv++) base += wsum[wv];
+        if (i < nbuckets) {
+            bstart[i] = base + inc - v;
+            bcursor[i] = base + inc - v;
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) carry_sh = base + inc;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) bstart[nbuckets] = carry_sh;
+}
+
+__global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict__ descs,
+                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                     uint32_t* bcursor, uint64_t* __restrict__ pkey,
+                                                     uint32_t* __restrict__ pgi) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t hist[LDS_SPAN];  // first the tile's count per bucket, then its write cursor
+    load_lbase(lb, lbase, N);
+    const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
+        __syncthreads();
+        const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;
+        for_tile(tile, descs, lb, N, L, [&](uint32_t, int sl, uint64_t sign) {
+            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+            if (local < LDS_SPAN) atomicAdd(&hist[local], 1u);
+        });
+        __syncthreads();
+        for (int i = threadIdx.x; i < LDS_SPAN; i += 256)
+            if (hist[i]) hist[i] = atomicAdd(&bcursor[b0 + i], hist[i]);  // the tile's slice of the bucket
+        __syncthreads();
+        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, uint64_t sign) {
+            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+            if (local < LDS_SPAN) {
+                const uint32_t at = atomicAdd(&hist[local], 1u);
+                pkey[at] = sign;
+                pgi[at] = gi;
+            }
+        });
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ uint32_t lds_slot(uint64_t sign) { return (uint32_t)(mix64(sign) >> 7) & (LDS_TABLE - 1); }
+
+// One workgroup per bucket.  first_of[gi] = position of the first occurrence
+// of gi's sign in its slot; cnt_at[first position] = occurrences of the sign.
+__global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
+                                                   const uint64_t* __restrict__ pkey, const uint32_t* __restrict__ pgi,
+                                                   uint32_t* __restrict__ first_of, uint32_t* __restrict__ cnt_at,
+                                                   DevStatus* status) {
+    __shared__ unsigned long long keys[LDS_TABLE + 1];  // entry LDS_TABLE: the sign EMPTY_KEY itself
+    __shared__ uint32_t minpos[LDS_TABLE + 1];
+    __shared__ uint32_t cnts[LDS_TABLE + 1];
+    for (uint32_t b = blockIdx.x; b < nbuckets; b += gridDim.x) {
+        const uint32_t lo = bstart[b], hi = bstart[b + 1];
+        if (lo == hi) continue;
+        for (int i = threadIdx.x; i <= LDS_TABLE; i += 256) {
+            keys[i] = EMPTY_KEY;
+            minpos[i] = 0xFFFFFFFFu;
+            cnts[i] = 0;
+        }
+        __syncthreads();
+        for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+            const uint64_t sign = pkey[i];
+            const uint32_t gi = pgi[i];
+            uint32_t h = LDS_TABLE;
+            if (sign != EMPTY_KEY) {
+                h = lds_slot(sign);
+                int tries = 0;
+                for (; tries < LDS_TABLE; tries++) {
+                    unsigned long long old = keys[h];
+                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                    h = (h + 1) & (LDS_TABLE - 1);
+                }
+                if (tries == LDS_TABLE) {  // table full: keep indices in bounds, let the host fall back
+                    atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+                    continue;
+                }
+            }
+            atomicMin(&minpos[h], gi);
+            atomicAdd(&cnts[h], 1u);
+        }
+        __syncthreads();
+        for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+            const uint64_t sign = pkey[i];
+            const uint32_t gi = pgi[i];
+            uint32_t h = LDS_TABLE;
+            bool found = true;
+            if (sign != EMPTY_KEY) {
+                h = lds_slot(sign);
+                int tries = 0;
+                for (; tries < LDS_TABLE && keys[h] != sign; tries++) h = (h + 1) & (LDS_TABLE - 1);
+                found = tries < LDS_TABLE;
+            }
+            const uint32_t f = found ? minpos[h] : gi;
+            first_of[gi] = f;
+            if (f == gi) cnt_at[gi] = found ? cnts[h] : 1u;
+        }
+        __syncthreads();
+    }
+}
+
+// Tile counts of first occurrences; a lookup is one iff first_of[gi] == gi.
+__global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const uint32_t* __restrict__ first_of,
+                                                             uint8_t* __restrict__ flag8,
+                                                             uint32_t* __restrict__ tilesum) {
+    __shared__ uint32_t red[4];
+    const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
+    uint32_t bits = 0;
+    if (base < L) {
+        for (int j = 0; j < REMAP_ITEMS; j++) {
+            const uint32_t gi = base + j;
+            if (gi >= L) break;
+            if (first_of[gi] == gi) bits |= 1u << j;
+        }
+        flag8[base / REMAP_ITEMS] = (uint8_t)bits;
+    }
+    uint32_t total = block_sum_256(__popc(bits), red);
+    if (threadIdx.x == 0) tilesum[blockIdx.x] = total;
+}
+
+// Ranks of the first occurrences (rank_at[gi]), distinct lists, show counts.
+__global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
+    const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L,
+    const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff, const uint32_t* __restrict__ cnt_at,
+    uint32_t* __restrict__ rank_at, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
+    uint32_t* __restrict__ uniq_slot, int2* __restrict__ ucnt) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t red[4];
+    load_lbase(lb, lbase, N);
+    const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
+    uint32_t bits = 0;
+    if (base < L) bits = flag8[base / REMAP_ITEMS];
+    uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256<uint32_t>(__popc(bits), red, nullptr);
+    if (base >= L) return;
+    int sl = find_slot(lb, N, base);
+    for (int j = 0; j < REMAP_ITEMS; j++) {
+        const uint32_t gi = base + j;
+        if (gi >= L) break;
+        while (gi >= lb[sl + 1]) sl++;
+        if (gi == lb[sl]) {
+            ubase[sl] = u;
+            for (int e = sl - 1; e >= 0 && lb[e] == gi; e--) ubase[e] = u;
+        }
+        if (bits & (1u << j)) {
+            rank_at[gi] = u;
+            uniq_sign[u] = (uint64_t)descs[sl].values[gi - lb[sl]];
+            uniq_slot[u] = (uint32_t)sl;
+            ucnt[u] = make_int2((int)cnt_at[gi], 0);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            u++;
+        }
+    }
+}
+
+// mapped id = rank of the sign's first occurrence, relative to the slot.
+__global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__ descs,
+                                                    const uint32_t* __restrict__ lbase,
+                                                    const uint32_t* __restrict__ ubase, int N, uint32_t L,
+                                                    const uint32_t* __restrict__ first_of,
+                                                    const uint32_t* __restrict__ rank_at,
+                                                    uint32_t* __restrict__ u_of_gi) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        const uint32_t f = first_of[gi];
+        const uint32_t u = rank_at[f];
+        u_of_gi[gi] = u | (f == gi ? FIRST_BIT : 0u);
+        const int sl = find_slot(lb, N, gi);
+        descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+    }
+}
+
+// Push on a plan whose show counts are already known: clear the click sums ...
+__global__ __launch_bounds__(256) void k_reset_clicks(int2* __restrict__ ucnt, const DevStatus* status) {
+    const uint32_t n = status->n_unique;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) ucnt[u].y = 0;
+}
+
+// ... and add the non-zero labels (sparse_table_ops.cc:283-296).
+__global__ __launch_bounds__(256) void k_count_click(const SlotDesc* __restrict__ descs,
+                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                     const uint32_t* __restrict__ u_of_gi, int2* ucnt) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        const int sl = find_slot(lb, N, gi);
+        const int label = (int)descs[sl].labels[gi - lb[sl]];
+        if (label != 0) atomicAdd(&ucnt[u_of_gi[gi] & ~FIRST_BIT].y, label);
+    }
+}
+
+}  // namespace tn
+
+#endif  // TN_REMAP_LDS_H_

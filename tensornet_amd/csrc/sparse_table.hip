@@ -1,7 +1,7 @@
 // SparseTable host side: registry, HBM storage management and the launch
 // sequences of pull / push at table level (core/ps/table/sparse_table.cc:52-83)
 // and at operator level (core/kernels/sparse_table_ops.cc:170-265,317-368).
-#include "sparse_kernels.h"
+#include "remap_lds.h"
 
 #include <algorithm>
 #include <cstring>
@@ -14,6 +14,7 @@ constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:26
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
+constexpr size_t LDS_MIN_LOOKUPS = 32768;  // smaller batches are launch-bound: the shorter global-table path wins
 
 struct HostStatus {
     DevStatus st;
@@ -36,6 +37,7 @@ struct SparseTable {
     DevBuf ws;                      // per-call scratch
     DevBuf plan_buf;                // what the last pull op worked out about its batch (see Plan)
     bool plan_valid = false;
+    bool plan_has_show = false;     // the plan already holds batch_show of every distinct sign
     int plan_N = 0;
     std::vector<int64_t> plan_lens;
     uint64_t epoch = 0;             // bumped whenever rows move (growth)
@@ -319,6 +321,16 @@ struct Scratch {
     uint32_t* tilesum;
     uint32_t* tileoff;
     uint32_t ntiles;
+    // LDS remap
+    uint32_t nbuckets;
+    uint32_t* bcount;
+    uint32_t* bstart;
+    uint32_t* bcursor;
+    uint64_t* pkey;
+    uint32_t* pgi;
+    uint32_t* first_of;
+    uint32_t* cnt_at;
+    uint32_t* rank_at;
     void* gt;  // GroupEntry[] or MaskEntry[]
     uint32_t* gidx;
     uint32_t* ord;
@@ -364,11 +376,27 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     return align_up(c.off, 256);
 }
 
-size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries) {
+// dt_entries: entries of the global dedup table, or (use_lds) the number of buckets.
+size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds) {
     Carver c{base};
-    w.dt = c.take<DedupEntry>(dt_entries);
-    w.dt_entries = dt_entries;
-    w.tidx = c.take<uint32_t>(L);
+    if (use_lds) {
+        w.nbuckets = (uint32_t)dt_entries;
+        w.bcount = c.take<uint32_t>(dt_entries + 1);
+        w.bstart = c.take<uint32_t>(dt_entries + 1);
+        w.bcursor = c.take<uint32_t>(dt_entries + 1);
+        w.pkey = c.take<uint64_t>(L);
+        w.pgi = c.take<uint32_t>(L);
+        w.first_of = c.take<uint32_t>(L);
+        w.cnt_at = c.take<uint32_t>(L);
+        w.rank_at = c.take<uint32_t>(L);
+        w.dt = nullptr;
+        w.dt_entries = 0;
+        w.tidx = nullptr;
+    } else {
+        w.dt = c.take<DedupEntry>(dt_entries);
+        w.dt_entries = dt_entries;
+        w.tidx = c.take<uint32_t>(L);
+    }
     w.flag8 = c.take<uint8_t>(L / REMAP_ITEMS + REMAP_THREADS);
     w.ntiles = (uint32_t)((L + REMAP_TILE - 1) / REMAP_TILE);
     w.tilesum = c.take<uint32_t>(w.ntiles + 1);
@@ -378,8 +406,12 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries) {
 }
 
 // Validates the slot arrays of an op and fills the descriptors; returns L.
+// With *use_lds set on entry the slots are laid out for the LDS remap if the batch
+// qualifies (tbase/tcap = first bucket / number of buckets of the slot, dt_entries =
+// number of buckets); otherwise *use_lds comes back false and tbase/tcap describe the
+// slot's region of the global dedup table.
 int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64_t* lens, std::vector<SlotDesc>& descs,
-                std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what) {
+                std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what, bool* use_lds) {
     if (N <= 0 || !values || !lens) return fail(TN_ERR_INVALID_ARGUMENT, std::string(what) + ": no slots");
     if (N > MAX_SLOTS)
         return fail(TN_ERR_UNSUPPORTED, std::string(what) + ": more than " + std::to_string(MAX_SLOTS) + " slots");
@@ -405,6 +437,21 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
     lbase[N] = (uint32_t)l;
     L = l;
     dt_entries = te;
+    if (use_lds && *use_lds) {
+        bool ok = l >= LDS_MIN_LOOKUPS;
+        for (int s = 0; s < N && ok; s++) ok = (size_t)lens[s] <= (size_t)LDS_MAX_SUB * LDS_BUCKET_TARGET;
+        *use_lds = ok;
+        if (ok) {
+            size_t nb = 0;
+            for (int s = 0; s < N; s++) {
+                size_t sub = std::max<size_t>(1, ((size_t)lens[s] + LDS_BUCKET_TARGET - 1) / LDS_BUCKET_TARGET);
+                descs[s].tbase = (uint32_t)nb;
+                descs[s].tcap = (uint32_t)sub;
+                nb += sub;
+            }
+            dt_entries = nb;
+        }
+    }
     return TN_OK;
 }
 
@@ -456,6 +503,7 @@ void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_
 
 constexpr int MASK_SLOTS = 128;
 
+
 // The same result for the distinct signs of an op with at most 128 slots, from slot masks.
 void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint32_t big_k, DevStatus* ds,
                           hipStream_t st) {
@@ -469,24 +517,42 @@ void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint
     TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, p.list, p.g_of_u);
 }
 
-// Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids
-// (steps of k_remap_insert .. k_write_mapped), groups of equal signs, and the
-// table row of every group (inserting absent signs for a pull).
-void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull,
+// Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids,
+// groups of equal signs, and the table row of every group (inserting absent
+// signs for a pull).  use_lds picks the remap through LDS (pull only).
+void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull, bool use_lds,
                        hipStream_t st) {
     DevStatus* ds = t->dplan;
     const Store& s = t->store;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, 0u, 0u);
-    TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st,
-              reinterpret_cast<uint4*>(w.dt), w.dt_entries);
-    TN_LAUNCH(k_remap_insert, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, L, w.dt, w.tidx, p.vals_copy);
-    TN_LAUNCH(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.lbase, N, L, w.dt, w.tidx, w.flag8, w.tilesum);
-    TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
-    TN_LAUNCH(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.dt, w.tidx, w.flag8,
-              w.tileoff, p.ubase, p.uniq_sign, p.uniq_slot);
-    TN_LAUNCH(k_write_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.dt, w.tidx, w.flag8,
-              p.u_of_gi, for_pull ? 1 : 0);
+    if (use_lds) {
+        const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
+        TN_LAUNCH(k_zero_u32, dim3(launch_grid(w.nbuckets + 1, 256, 64)), dim3(256), st, w.bcount, w.nbuckets + 1);
+        TN_LAUNCH(k_lds_hist, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy, w.first_of,
+                  w.cnt_at, ds);
+        TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
+        TN_LAUNCH(k_lds_scatter, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcursor, w.pkey, w.pgi);
+        TN_LAUNCH(k_lds_dedup, dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart, w.nbuckets,
+                  w.pkey, w.pgi, w.first_of, w.cnt_at, ds);
+        TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
+        TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
+        TN_LAUNCH(k_lds_assign, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8, w.tileoff,
+                  w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ucnt);
+        TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.rank_at,
+                  p.u_of_gi);
+    } else {
+        TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st,
+                  reinterpret_cast<uint4*>(w.dt), w.dt_entries);
+        TN_LAUNCH(k_remap_insert, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, L, w.dt, w.tidx, p.vals_copy);
+        TN_LAUNCH(k_flag_count, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.lbase, N, L, w.dt, w.tidx, w.flag8,
+                  w.tilesum);
+        TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
+        TN_LAUNCH(k_assign_rank, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.dt, w.tidx, w.flag8,
+                  w.tileoff, p.ubase, p.uniq_sign, p.uniq_slot);
+        TN_LAUNCH(k_write_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.dt, w.tidx, w.flag8,
+                  p.u_of_gi, for_pull ? 1 : 0);
+    }
     if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ds, st);
     else
@@ -836,65 +902,82 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     if (var_dim != wdim)
         return fail(TN_ERR_DIM_MISMATCH, "SparseTablePull: variable dim " + std::to_string(var_dim) +
                                              " but table rows hold " + std::to_string(wdim));
-    std::vector<SlotDesc> descs;
-    std::vector<uint32_t> lbase;
-    size_t L = 0, dt_entries = 0;
-    TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePull"));
-    bool vec = (wdim % 4 == 0) && (t->store.wstride % 4 == 0);
-    for (int s = 0; s < N; s++) {
-        if (var_rows[s] < 0 || !vars[s] || (value_lens[s] > 0 && !mapped_values[s]))
-            return fail(TN_ERR_INVALID_ARGUMENT,
-                        "sparse pull variable must Matrix(sign_id_cnt, dim), slot " + std::to_string(s));
-        descs[s].var = vars[s];
-        descs[s].rows = var_rows[s];
-        descs[s].mapped = mapped_values[s];
-        vec = vec && aligned16(vars[s]);
-    }
     t->last_stream = st;
     if (t->push_pending || t->pull_pending) {
         TN_HIP(hipStreamSynchronize(st));
         harvest(t);
     }
-    if (L == 0) {
-        t->last_counts.assign(N, 0);
-        return take_latched(t);
-    }
-    TN_TRY(ensure_room(t, (uint64_t)L, st));
-    Plan p{};
-    Scratch w{};
-    TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
-    carve_plan((char*)t->plan_buf.p, p, N, L);
-    TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries)));
-    carve_scratch((char*)t->ws.p, w, L, dt_entries);
-    t->plan_valid = false;
-    TN_TRY(upload_slots(t, p, descs, lbase, st));
+    // The remap through LDS needs the call's status on the host to fall back if a
+    // bucket overflowed, so it is only used when the pull waits for its stream anyway.
+    bool use_lds = !t->async_pull;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        std::vector<SlotDesc> descs;
+        std::vector<uint32_t> lbase;
+        size_t L = 0, dt_entries = 0;
+        TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePull", &use_lds));
+        bool vec = (wdim % 4 == 0) && (t->store.wstride % 4 == 0);
+        for (int s = 0; s < N; s++) {
+            if (var_rows[s] < 0 || !vars[s] || (value_lens[s] > 0 && !mapped_values[s]))
+                return fail(TN_ERR_INVALID_ARGUMENT,
+                            "sparse pull variable must Matrix(sign_id_cnt, dim), slot " + std::to_string(s));
+            descs[s].var = vars[s];
+            descs[s].rows = var_rows[s];
+            descs[s].mapped = mapped_values[s];
+            vec = vec && aligned16(vars[s]);
+        }
+        if (L == 0) {
+            t->last_counts.assign(N, 0);
+            return take_latched(t);
+        }
+        TN_TRY(ensure_room(t, (uint64_t)L, st));
+        Plan p{};
+        Scratch w{};
+        TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
+        carve_plan((char*)t->plan_buf.p, p, N, L);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds);
+        t->plan_valid = false;
+        TN_TRY(upload_slots(t, p, descs, lbase, st));
 
-    const Store& s = t->store;
-    const OptDev o = make_optdev(t);
-    DevStatus* ds = t->dplan;
-    launch_build_plan(t, p, w, N, (uint32_t)L, true, st);
-    const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_init_rows, dim3(gblocks), dim3(256), st, s, o, t->seed, p.grp_sign, p.grp_row, p.newlist, ds);
-    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
-    if (vec)
-        TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, ds,
-                  p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
-    else
-        TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
-                  p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
-    TN_HIP(hipGetLastError());
-    TN_HIP(hipMemcpyAsync(&t->hpull->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
-    TN_HIP(hipMemcpyAsync(t->hpull->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
-    t->pull_pending = true;
-    t->pending_slots = N;
-    t->pending_rows.assign(var_rows, var_rows + N);
-    // a push of the same batch may reuse the analysis
-    t->plan_valid = true;
-    t->plan_N = N;
-    t->plan_lens.assign(value_lens, value_lens + N);
-    t->plan_epoch = t->epoch;
-    if (t->async_pull) return TN_OK;
-    return sync_table(t, st);
+        const Store& s = t->store;
+        const OptDev o = make_optdev(t);
+        DevStatus* ds = t->dplan;
+        launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st);
+        const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
+        TN_LAUNCH(k_init_rows, dim3(gblocks), dim3(256), st, s, o, t->seed, p.grp_sign, p.grp_row, p.newlist, ds);
+        TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
+        if (vec)
+            TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
+                      ds, p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
+        else
+            TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
+                      p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
+        TN_HIP(hipGetLastError());
+        TN_HIP(hipMemcpyAsync(&t->hpull->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+        TN_HIP(hipMemcpyAsync(t->hpull->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+        t->pull_pending = true;
+        t->pending_slots = N;
+        t->pending_rows.assign(var_rows, var_rows + N);
+        // a push of the same batch may reuse the analysis
+        t->plan_valid = true;
+        t->plan_has_show = use_lds;
+        t->plan_N = N;
+        t->plan_lens.assign(value_lens, value_lens + N);
+        t->plan_epoch = t->epoch;
+        if (t->async_pull) return TN_OK;
+        TN_HIP(hipStreamSynchronize(st));
+        if (use_lds && (t->hpull->st.err & DEV_ERR_REMAP_OVERFLOW)) {
+            // rows the failed attempt inserted belong to signs of this batch; keep them counted
+            t->hpull->st.err &= ~DEV_ERR_REMAP_OVERFLOW;
+            harvest(t);
+            t->latched = TN_OK;
+            t->latched_msg.clear();
+            use_lds = false;
+            continue;
+        }
+        return sync_table(t, st);
+    }
+    return fail(TN_ERR_HIP, "SparseTablePull: remap fell back twice");
 }
 
 int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
@@ -913,7 +996,7 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     std::vector<SlotDesc> descs;
     std::vector<uint32_t> lbase;
     size_t L = 0, dt_entries = 0;
-    TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePush"));
+    TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePush", nullptr));
     bool vec = (grad_dim % 4 == 0);
     for (int s = 0; s < N; s++) {
         if (grad_rows[s] < 0 || (grad_rows[s] > 0 && !grads[s]) || (value_lens[s] > 0 && !feature_labels[s]))
@@ -947,20 +1030,30 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_HIP(hipStreamSynchronize(st));
         reuse = t->hpush->st.mismatch == 0;
     }
+    bool has_show = reuse && t->plan_has_show;
     if (!reuse) {
+        // another batch than the last pull's: analyse it here, on the global-table path
+        // (its status cannot be waited for, a push only enqueues)
         t->plan_valid = false;
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
         carve_plan((char*)t->plan_buf.p, p, N, L);
-        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries)));
-        carve_scratch((char*)t->ws.p, w, L, dt_entries);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, false)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
         TN_TRY(upload_slots(t, p, descs, lbase, st));
-        launch_build_plan(t, p, w, N, (uint32_t)L, false, st);
+        launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
     }
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ucnt, ds);
-    // AdaGrad is the only optimizer that reads batch_click
-    TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256), st,
-              p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt, t->opt->kind == OPT_ADAGRAD ? 1 : 0);
+    const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
+    if (has_show) {
+        if (with_click) {
+            TN_LAUNCH(k_reset_clicks, dim3(lblocks), dim3(256), st, p.ucnt, ds);
+            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt);
+        }
+    } else {
+        TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ucnt, ds);
+        TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256),
+                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt, with_click ? 1 : 0);
+    }
     launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));

@@ -75,6 +75,7 @@ enum : uint32_t {
     DEV_ERR_UNKNOWN_KEY = 2u,
     DEV_ERR_TABLE_FULL = 4u,
     DEV_ERR_GRAD_ROWS = 8u,
+    DEV_ERR_REMAP_OVERFLOW = 16u,  // the LDS remap met a bucket it cannot hold: repeat on the global-table path
 };
 
 struct DevStatus {

@@ -460,3 +460,35 @@ def test_many_slots(tn, oracle, slots):
         labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
         pair.push_op(values, grads, labels)
         pair.assert_rows_match(base)
+
+
+def test_remap_falls_back_when_a_bucket_overflows(tn, oracle):
+    """Large batches are remapped through per-bucket hash tables in LDS; a slot whose
+    signs are crafted to fall into one bucket (more distinct signs than the LDS table
+    holds) must still give the reference's ids and rows (the call is redone on the
+    global-table path)."""
+    D = 8
+    rng = np.random.default_rng(77)
+    n_slot = 40000
+    nb = (n_slot + 1535) // 1536  # buckets of the slot
+    cand = rng.integers(0, 1 << 63, 400000, dtype=np.uint64)
+    x = cand.copy()
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xFF51AFD7ED558CCD)
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xC4CEB9FE1A85EC53)
+    x ^= x >> np.uint64(33)
+    bucket = ((x >> np.uint64(32)) * np.uint64(nb)) >> np.uint64(32)  # ~ umulhi(mix64(sign), nb)
+    crowd = cand[bucket == 0][:6000]
+    assert len(crowd) == 6000
+    filler = cand[bucket != 0][: n_slot - 6000]
+    slot0 = rng.permutation(np.concatenate([crowd, filler])).view(np.int64)
+    slot1 = rng.permutation(np.concatenate([crowd[:3000], filler[:5000]])).view(np.int64)
+    values = [slot0, slot1]
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=200000)
+    pair.populate(all_signs(values))
+    counts = check_pull(pair, values)
+    assert counts.tolist() == [len(np.unique(slot0)), len(np.unique(slot1))]
+    grads = synth.make_grads(counts, D, 0.01)
+    pair.push_op(values, grads, [np.ones(len(v), np.int64) for v in values])
+    pair.assert_rows_match(all_signs(values))
