@@ -61,12 +61,13 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
 }
 
-// Also presets first_of / cnt_at to "every lookup is its own first occurrence",
-// which is what a lookup keeps if an overflow leaves it unprocessed.
+// Also presets first_of to "every lookup is its own first occurrence", which is
+// what a lookup keeps if an overflow leaves it unprocessed (its count is then
+// meaningless, but every index stays in bounds until the host repeats the call).
 __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
                                                   int N, uint32_t L, uint32_t* bcount,
                                                   uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ first_of,
-                                                  uint32_t* __restrict__ cnt_at, DevStatus* status) {
+                                                  DevStatus* status) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t hist[LDS_SPAN];
     load_lbase(lb, lbase, N);
@@ -78,7 +79,6 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
         for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, uint64_t sign) {
             vals_copy[gi] = sign;
             first_of[gi] = gi;
-            cnt_at[gi] = 1;
             const uint32_t local = bucket_of(descs[sl], sign) - b0;
             if (local < LDS_SPAN)
                 atomicAdd(&hist[local], 1u);
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L,
     const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff, const uint32_t* __restrict__ cnt_at,
     uint32_t* __restrict__ rank_at, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
-    uint32_t* __restrict__ uniq_slot, int2* __restrict__ ucnt) {
+    uint32_t* __restrict__ uniq_slot, uint32_t* __restrict__ ushow) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t red[4];
     load_lbase(lb, lbase, N);
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
             rank_at[gi] = u;
             uniq_sign[u] = (uint64_t)descs[sl].values[gi - lb[sl]];
             uniq_slot[u] = (uint32_t)sl;
-            ucnt[u] = make_int2((int)cnt_at[gi], 0);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            ushow[u] = cnt_at[gi];  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             u++;
         }
     }
@@ -287,24 +287,20 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
     }
 }
 
-// Push on a plan whose show counts are already known: clear the click sums ...
-__global__ __launch_bounds__(256) void k_reset_clicks(int2* __restrict__ ucnt, const DevStatus* status) {
-    const uint32_t n = status->n_unique;
-    const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) ucnt[u].y = 0;
-}
-
-// ... and add the non-zero labels (sparse_table_ops.cc:283-296).
+// Push on a plan whose member lists already hold the show counts: the click
+// sums are cleared (k_reset_counts) and the non-zero labels added
+// (sparse_table_ops.cc:283-296).
 __global__ __launch_bounds__(256) void k_count_click(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     const uint32_t* __restrict__ u_of_gi, int2* ucnt) {
+                                                     const uint32_t* __restrict__ u_of_gi,
+                                                     const uint32_t* __restrict__ pos_of_u, Member* list) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
         const int label = (int)descs[sl].labels[gi - lb[sl]];
-        if (label != 0) atomicAdd(&ucnt[u_of_gi[gi] & ~FIRST_BIT].y, label);
+        if (label != 0) atomicAdd(&list[pos_of_u[u_of_gi[gi] & ~FIRST_BIT]].click, label);
     }
 }
 

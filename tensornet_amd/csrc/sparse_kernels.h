@@ -64,6 +64,15 @@ struct GroupEntry {
     uint32_t g;    // number of the group
 };
 
+// One record of a push in its group's member list: which distinct sign of which
+// slot, and its batch_show / batch_click (SparsePushSignInfo's counts).
+struct __attribute__((aligned(16))) Member {
+    uint32_t u;
+    uint32_t slot;
+    int32_t show;
+    int32_t click;
+};
+
 constexpr int REMAP_ITEMS = 8;
 constexpr int REMAP_THREADS = 256;
 constexpr int REMAP_TILE = REMAP_ITEMS * REMAP_THREADS;
@@ -104,10 +113,11 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         status->err = 0;
         status->n_unique = n_unique;
-        status->n_groups = 0;
+        status->n_single = 0;
+        status->n_multi = 0;
         status->n_new = 0;
         status->gcap = gcap;
-        status->list_cursor = 0;
+        status->n_members = 0;
         status->mismatch = 0;
         status->n_big = 0;
     }
@@ -121,6 +131,29 @@ __global__ void k_begin_push(DevStatus* status) {
     }
 }
 
+// Small host<->device transfers done by kernels on the stream (pinned host
+// memory is device-accessible): cheaper than a copy command each.
+__global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ host_src, uint32_t* __restrict__ dst_a,
+                                                  uint32_t words_a, uint32_t* __restrict__ dst_b, uint32_t words_b) {
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < words_a + words_b; i += stride) {
+        if (i < words_a)
+            dst_a[i] = host_src[i];
+        else
+            dst_b[i - words_a] = host_src[i];
+    }
+}
+
+// host_dst: a DevStatus followed by n_ubase words
+__global__ __launch_bounds__(256) void k_publish(const DevStatus* __restrict__ status,
+                                                 const uint32_t* __restrict__ ubase, uint32_t n_ubase,
+                                                 uint32_t* __restrict__ host_dst) {
+    const uint32_t sw = sizeof(DevStatus) / 4;
+    const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
+    for (uint32_t i = threadIdx.x; i < sw + n_ubase; i += blockDim.x)
+        host_dst[i] = i < sw ? sp[i] : ubase[i - sw];
+}
+
 __global__ void k_finish_insert(Store s, const DevStatus* status) {
     if (threadIdx.x == 0 && blockIdx.x == 0) *s.count += status->n_new;
 }
@@ -130,13 +163,23 @@ __global__ void k_finish_insert(Store s, const DevStatus* status) {
 // With INSERT an absent sign claims the first free slot of its probe sequence
 // (SparseKernelBlock::GetWeight's insert, optimizer_kernel.h:299-308) and the
 // index i of every claim is appended to newlist.
+// Groups with one record are numbered upwards from 0, groups with several
+// downwards from ids_cap - 1: the i-th group in enumeration order.
+__device__ __forceinline__ uint32_t group_id(uint32_t i, uint32_t n_single, uint32_t n_multi, uint32_t ids_cap) {
+    return i < n_single ? i : ids_cap - n_multi + (i - n_single);
+}
+
+// With groups_of != nullptr the signs are those of its groups (ids_cap = size of the id space).
 template <bool INSERT>
 __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restrict__ signs, int64_t n_host,
-                                               const uint32_t* n_dev, uint32_t* __restrict__ rows,
-                                               uint32_t* __restrict__ newlist, DevStatus* status, uint32_t miss_err) {
-    const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
+                                               const DevStatus* groups_of, uint32_t ids_cap,
+                                               uint32_t* __restrict__ rows, uint32_t* __restrict__ newlist,
+                                               DevStatus* status, uint32_t miss_err) {
+    const uint32_t n_single = groups_of ? groups_of->n_single : 0, n_multi = groups_of ? groups_of->n_multi : 0;
+    const int64_t n = groups_of ? (int64_t)n_single + n_multi : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride) {
+        const int64_t i = groups_of ? (int64_t)group_id((uint32_t)t, n_single, n_multi, ids_cap) : t;
         const uint64_t sign = signs[i];
         uint32_t row = NO_ROW;
         bool is_new = false;
@@ -561,12 +604,17 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
 }
 
 // Push: batch_show = occurrences, batch_click = sum of labels per distinct sign
-// (sparse_table_ops.cc:283-296; labels are narrowed to int as there), kept as
-// one {show, click} pair per distinct sign.  Every sign starts at show 1 / click 0 ...
-__global__ __launch_bounds__(256) void k_reset_counts(int2* __restrict__ ucnt, const DevStatus* status) {
-    const uint32_t n = status->n_unique;
+// (sparse_table_ops.cc:283-296; labels are narrowed to int as there), kept in
+// the member lists.  Every sign starts at show 1 / click 0 ...
+__global__ __launch_bounds__(256) void k_reset_counts(Member* __restrict__ list, const DevStatus* status,
+                                                      uint32_t ids_cap, int keep_show) {
+    const uint32_t n_single = status->n_single, n_members = status->n_members;
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) ucnt[u] = make_int2(1, 0);
+    for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < n_single + n_members; t += stride) {
+        const uint32_t i = group_id(t, n_single, n_members, ids_cap);  // the member array is laid out like the ids
+        if (!keep_show) list[i].show = 1;
+        list[i].click = 0;
+    }
 }
 
 constexpr int COUNT_TILE = 2048;
@@ -577,7 +625,8 @@ constexpr int COUNT_SLOTS = 4096;  // LDS table entries per tile (load factor <=
 // up in an LDS hash table and issues one global atomic per sign it saw.
 __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                    const uint32_t* __restrict__ u_of_gi, int2* ucnt,
+                                                    const uint32_t* __restrict__ u_of_gi,
+                                                    const uint32_t* __restrict__ pos_of_u, Member* list,
                                                     int with_click) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t keys[COUNT_SLOTS];
@@ -617,8 +666,9 @@ __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__
         for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
             const uint32_t u = keys[i];
             if (u == 0xFFFFFFFFu) continue;
-            if (cnts[i]) atomicAdd(&ucnt[u].x, cnts[i]);
-            if (clks[i]) atomicAdd(&ucnt[u].y, clks[i]);
+            Member* m = &list[pos_of_u[u]];
+            if (cnts[i]) atomicAdd(&m->show, cnts[i]);
+            if (clks[i]) atomicAdd(&m->click, clks[i]);
         }
         __syncthreads();
     }
@@ -634,7 +684,6 @@ struct PushSrc {
     const uint64_t* uniq_sign;
     const uint32_t* uniq_slot;
     const uint32_t* ubase;
-    const int2* ucnt;        // {batch_show, batch_click} per distinct sign
     const SlotDesc* descs;
     int dim;
 };
@@ -678,52 +727,80 @@ constexpr int COMPACT_ITEMS = 16;
 // Signs with big_k records or more are applied by one wavefront each.
 __device__ __forceinline__ bool is_big(uint32_t k, uint32_t big_k) { return k >= big_k; }
 
-// ...every group gets a number, a slice of the member list and, when it has
-// big_k members or more, a place in the list of big groups (three atomics per
-// 1024 table entries)...
+// Numbers the groups found in one span of 256 x COMPACT_ITEMS table entries
+// (ks[j] = records of the thread's j-th entry, 0 = unused) and gives each a
+// slice of the member array.  Groups with one record get ids and member places
+// counted up from 0 (place == id); groups with several get ids counted down
+// from ids_cap - 1 and slices carved from the top of the member array; groups
+// with big_k records or more are also listed in big_list.  Four atomics per span.
+// write(j, g, off) stores the result for the thread's j-th entry.
+template <typename W>
+__device__ __forceinline__ void compact_span(DevStatus* status, const uint32_t (&ks)[COMPACT_ITEMS], uint32_t ids_cap,
+                                             uint32_t big_k, uint32_t* __restrict__ big_list, W write) {
+    __shared__ unsigned long long sh[4];
+    __shared__ uint32_t bases[4];
+    unsigned long long cnt = 0;  // bits 0-31 single groups, 32-63 multi groups
+    unsigned long long mem = 0;  // bits 0-39 records of multi groups, 40-63 big groups
+    for (int j = 0; j < COMPACT_ITEMS; j++) {
+        if (ks[j] == 1) cnt += 1ull;
+        if (ks[j] > 1) {
+            cnt += 1ull << 32;
+            mem += ks[j];
+            if (is_big(ks[j], big_k)) mem += 1ull << 40;
+        }
+    }
+    unsigned long long tcnt, tmem;
+    const unsigned long long ecnt = block_excl_scan_256<unsigned long long>(cnt, sh, &tcnt);
+    const unsigned long long emem = block_excl_scan_256<unsigned long long>(mem, sh, &tmem);
+    if (threadIdx.x == 0 && (uint32_t)tcnt) bases[0] = atomicAdd(&status->n_single, (uint32_t)tcnt);
+    if (threadIdx.x == 64 && (tcnt >> 32)) bases[1] = atomicAdd(&status->n_multi, (uint32_t)(tcnt >> 32));
+    if (threadIdx.x == 128 && tmem) bases[2] = atomicAdd(&status->n_members, (uint32_t)(tmem & 0xFFFFFFFFFFull));
+    if (threadIdx.x == 192 && (tmem >> 40)) bases[3] = atomicAdd(&status->n_big, (uint32_t)(tmem >> 40));
+    __syncthreads();
+    uint32_t gs = bases[0] + (uint32_t)ecnt;                              // next single id
+    uint32_t gm = bases[1] + (uint32_t)(ecnt >> 32);                      // multi groups before mine
+    uint32_t mm = bases[2] + (uint32_t)(emem & 0xFFFFFFFFFFull);          // multi records before mine
+    uint32_t bb = bases[3] + (uint32_t)(emem >> 40);
+    for (int j = 0; j < COMPACT_ITEMS; j++) {
+        const uint32_t k = ks[j];
+        if (k == 0) continue;
+        if (k == 1) {
+            write(j, gs, gs);
+            gs++;
+        } else {
+            const uint32_t g = ids_cap - 1 - gm;
+            mm += k;
+            write(j, g, ids_cap - mm);
+            if (is_big(k, big_k)) big_list[bb++] = g;
+            gm++;
+        }
+    }
+    __syncthreads();
+}
+
+// ...every group gets a number and a slice of the member array...
 __global__ __launch_bounds__(256) void k_group_compact(DevStatus* status, GroupEntry* gt,
                                                        uint64_t* __restrict__ grp_sign,
                                                        uint32_t* __restrict__ grp_off,
                                                        uint32_t* __restrict__ grp_cnt,
-                                                       uint32_t* __restrict__ big_list, uint32_t big_k) {
-    __shared__ unsigned long long sh[4];
-    __shared__ uint32_t bases[3];
+                                                       uint32_t* __restrict__ big_list, uint32_t big_k,
+                                                       uint32_t ids_cap) {
     const uint32_t n = status->gcap + 1;
     const uint32_t span = 256 * COMPACT_ITEMS;
     for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
         uint32_t ks[COMPACT_ITEMS];
-        unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t e = base + j * 256 + threadIdx.x;  // neighbouring lanes read neighbouring entries
             const uint32_t c = (e < n) ? gt[e].cnt : 0xFFFFFFFFu;
             ks[j] = (c != 0xFFFFFFFFu) ? c + 1 : 0;
-            if (ks[j]) mine += (1ull << 32) | ks[j];
-            if (is_big(ks[j], big_k)) mine += 1ull << 48;
         }
-        unsigned long long total;
-        unsigned long long excl = block_excl_scan_256<unsigned long long>(mine, sh, &total);
-        if (total) {
-            if (threadIdx.x == 0) bases[0] = atomicAdd(&status->list_cursor, (uint32_t)total);
-            if (threadIdx.x == 64) bases[1] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32) & 0xFFFFu);
-            if (threadIdx.x == 128 && (total >> 48)) bases[2] = atomicAdd(&status->n_big, (uint32_t)(total >> 48));
-        }
-        __syncthreads();
-        uint32_t off = bases[0] + (uint32_t)excl;
-        uint32_t g = bases[1] + ((uint32_t)(excl >> 32) & 0xFFFFu);
-        uint32_t b = bases[2] + (uint32_t)(excl >> 48);
-        for (int j = 0; j < COMPACT_ITEMS; j++) {
-            const uint32_t k = ks[j];
-            if (k == 0) continue;
+        compact_span(status, ks, ids_cap, big_k, big_list, [&](int j, uint32_t g, uint32_t off) {
             const uint32_t e = base + j * 256 + threadIdx.x;
             gt[e].g = g;
             grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
             grp_off[g] = off;
-            grp_cnt[g] = k;
-            if (is_big(k, big_k)) big_list[b++] = g;
-            g++;
-            off += k;
-        }
-        __syncthreads();
+            grp_cnt[g] = ks[j];
+        });
     }
 }
 
@@ -745,7 +822,8 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
                                                     const uint32_t* __restrict__ gidx,
                                                     const uint32_t* __restrict__ arrival,
                                                     const uint32_t* __restrict__ uniq_slot,
-                                                    uint2* __restrict__ list, uint32_t* __restrict__ g_of_u) {
+                                                    const uint32_t* __restrict__ ushow, Member* __restrict__ list,
+                                                    uint32_t* __restrict__ g_of_u, uint32_t* __restrict__ pos_of_u) {
     const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
@@ -757,8 +835,14 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
             const uint32_t* mem = arrival + off;
             for (uint32_t t = 0; t < k; t++) pos += mem[t] < (uint32_t)u;
         }
-        list[off + pos] = make_uint2((uint32_t)u, uniq_slot ? uniq_slot[u] : 0u);
+        Member m;
+        m.u = (uint32_t)u;
+        m.slot = uniq_slot ? uniq_slot[u] : 0u;
+        m.show = ushow ? (int32_t)ushow[u] : 1;
+        m.click = 0;
+        list[off + pos] = m;
         g_of_u[u] = en.g;
+        pos_of_u[u] = off + pos;
     }
 }
 
@@ -819,14 +903,12 @@ __global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEnt
                                                       uint64_t* __restrict__ grp_sign,
                                                       uint32_t* __restrict__ grp_off,
                                                       uint32_t* __restrict__ grp_cnt,
-                                                      uint32_t* __restrict__ big_list, uint32_t big_k) {
-    __shared__ unsigned long long sh[4];
-    __shared__ uint32_t bases[3];
+                                                      uint32_t* __restrict__ big_list, uint32_t big_k,
+                                                      uint32_t ids_cap) {
     const uint32_t n = status->gcap + 1;
     const uint32_t span = 256 * COMPACT_ITEMS;
     for (uint32_t base = blockIdx.x * span; base < n; base += gridDim.x * span) {
         uint32_t ks[COMPACT_ITEMS];
-        unsigned long long mine = 0;  // bits 0-31 members, 32-47 groups, 48-63 big groups
         for (int j = 0; j < COMPACT_ITEMS; j++) {
             const uint32_t e = base + j * 256 + threadIdx.x;  // neighbouring lanes read neighbouring entries
             ks[j] = 0;
@@ -834,55 +916,43 @@ __global__ __launch_bounds__(256) void k_mask_compact(DevStatus* status, MaskEnt
                 const ulonglong2 m = *reinterpret_cast<const ulonglong2*>(&gt[e].nlo);
                 ks[j] = (uint32_t)(__popcll(~m.x) + __popcll(~m.y));
             }
-            if (ks[j]) mine += (1ull << 32) | ks[j];
-            if (ks[j] && is_big(ks[j], big_k)) mine += 1ull << 48;
         }
-        unsigned long long total;
-        unsigned long long excl = block_excl_scan_256<unsigned long long>(mine, sh, &total);
-        if (total) {
-            if (threadIdx.x == 0) bases[0] = atomicAdd(&status->list_cursor, (uint32_t)total);
-            if (threadIdx.x == 64) bases[1] = atomicAdd(&status->n_groups, (uint32_t)(total >> 32) & 0xFFFFu);
-            if (threadIdx.x == 128 && (total >> 48)) bases[2] = atomicAdd(&status->n_big, (uint32_t)(total >> 48));
-        }
-        __syncthreads();
-        uint32_t off = bases[0] + (uint32_t)excl;
-        uint32_t g = bases[1] + ((uint32_t)(excl >> 32) & 0xFFFFu);
-        uint32_t b = bases[2] + (uint32_t)(excl >> 48);
-        for (int j = 0; j < COMPACT_ITEMS; j++) {
-            const uint32_t k = ks[j];
-            if (k == 0) continue;
+        compact_span(status, ks, ids_cap, big_k, big_list, [&](int j, uint32_t g, uint32_t off) {
             const uint32_t e = base + j * 256 + threadIdx.x;
             *reinterpret_cast<uint2*>(&gt[e].g) = make_uint2(g, off);
             grp_sign[g] = (e == n - 1) ? EMPTY_KEY : gt[e].key;
             grp_off[g] = off;
-            grp_cnt[g] = k;
-            if (is_big(k, big_k)) big_list[b++] = g;
-            g++;
-            off += k;
-        }
-        __syncthreads();
+            grp_cnt[g] = ks[j];
+        });
     }
 }
 
 __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, const MaskEntry* gt,
                                                    const uint32_t* __restrict__ gidx,
                                                    const uint32_t* __restrict__ uniq_slot,
-                                                   uint2* __restrict__ list, uint32_t* __restrict__ g_of_u) {
+                                                   const uint32_t* __restrict__ ushow, Member* __restrict__ list,
+                                                   uint32_t* __restrict__ g_of_u, uint32_t* __restrict__ pos_of_u) {
     const uint32_t n = status->n_unique;
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
         const MaskEntry* en = &gt[gidx[u]];
-        const ulonglong2 m = *reinterpret_cast<const ulonglong2*>(&en->nlo);
+        const ulonglong2 masks = *reinterpret_cast<const ulonglong2*>(&en->nlo);
         const uint2 go = *reinterpret_cast<const uint2*>(&en->g);
         const uint32_t sl = uniq_slot[u];
-        const uint64_t lo = ~m.x, hi = ~m.y;
+        const uint64_t lo = ~masks.x, hi = ~masks.y;
         uint32_t pos;
         if (sl < 64)
             pos = (uint32_t)__popcll(lo & ((1ull << sl) - 1ull));
         else
             pos = (uint32_t)__popcll(lo) + (uint32_t)__popcll(hi & ((1ull << (sl - 64)) - 1ull));
-        list[go.y + pos] = make_uint2(u, sl);
+        Member m;
+        m.u = u;
+        m.slot = sl;
+        m.show = ushow ? (int32_t)ushow[u] : 1;
+        m.click = 0;
+        list[go.y + pos] = m;
         g_of_u[u] = go.x;
+        pos_of_u[u] = go.y + pos;
     }
 }
 
@@ -919,24 +989,23 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
 }
 
 // -------------------------------------------------------------------- apply
-// Resolves a member {record u, slot} to its gradient row and counts; false if
-// the op's gradient matrix has no such row.
-__device__ __forceinline__ bool src_record(const PushSrc& p, uint2 member, const float*& g, int& show, int& click) {
-    const uint32_t u = member.x;
+// Resolves a member to its gradient row and counts; false if the op's gradient
+// matrix has no such row.
+__device__ __forceinline__ bool src_record(const PushSrc& p, Member member, const float*& g, int& show, int& click) {
+    const uint32_t u = member.u;
     if (p.infos) {
         g = p.grads + (uint64_t)u * p.dim;
         show = p.infos[u].batch_show;
         click = p.infos[u].batch_click;
         return true;
     }
-    const uint32_t sl = member.y;
+    const uint32_t sl = member.slot;
     const int64_t r = (int64_t)u - (int64_t)p.ubase[sl];
     const SlotDesc& d = p.descs[sl];
     if (r >= d.rows) return false;
     g = d.grads + (uint64_t)r * p.dim;
-    const int2 c = p.ucnt[u];
-    show = c.x;
-    click = c.y;
+    show = member.show;
+    click = member.click;
     return true;
 }
 
@@ -964,6 +1033,81 @@ __device__ __forceinline__ void ftrl_elem(const OptDev& o, float g, float& w, fl
     }
 }
 
+// Most signs occur in one slot only: one record, no ordering problem, no
+// loop.  LPG lanes update the row of one such sign; its member entry sits at
+// the place of its group number.
+template <int KIND, int LPG>
+__global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                      const uint32_t* __restrict__ grp_row,
+                                                      const Member* __restrict__ list) {
+    const uint32_t n_single = status->n_single;
+    const int D = s.D;
+    const int sub = threadIdx.x % LPG;
+    const int lane0 = (int)__lane_id() - sub;
+    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+    for (uint32_t g = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; g < n_single; g += gstride) {
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
+        const float* gp;
+        int bshow, bclick;
+        if (!src_record(src, list[g], gp, bshow, bclick)) {
+            if (sub == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+            continue;
+        }
+        float* wp = s.w + (uint64_t)row * s.wstride;
+        float* sp = s.st + (uint64_t)row * s.sstride;
+        const float4 gr = reinterpret_cast<const float4*>(gp)[sub];
+        float4 w = reinterpret_cast<float4*>(wp)[sub];
+        if (KIND == OPT_ADAGRAD) {
+            const float4 h = *reinterpret_cast<const float4*>(sp);
+            const float p0 = gr.x * gr.x, p1 = gr.y * gr.y, p2 = gr.z * gr.z, p3 = gr.w * gr.w;
+            double tot = 0.0;  // add_g2sum: double accumulator over the float products, element order 0..D-1
+            for (int l = 0; l < LPG; l++) {
+                double cand = tot;
+                cand += (double)p0;
+                cand += (double)p1;
+                cand += (double)p2;
+                cand += (double)p3;
+                tot = __shfl(cand, lane0 + l);
+            }
+            const float g2sum = (float)((double)h.x + tot / (double)D);
+            const float den = o.eps + sqrtf(g2sum);
+            w.x -= o.lr * gr.x / den;
+            w.y -= o.lr * gr.y / den;
+            w.z -= o.lr * gr.z / den;
+            w.w -= o.lr * gr.w / den;
+            reinterpret_cast<float4*>(wp)[sub] = w;
+            if (sub == 0) {
+                const float show = h.y + (float)bshow, click = h.z + (float)bclick;
+                *reinterpret_cast<float4*>(sp) = make_float4(g2sum, show, click, 0.f);  // no_show_days = 0
+                if (o.use_cvm) {
+                    wp[D] = show;
+                    wp[D + 1] = logf(click + 1) - logf(show + 1);
+                }
+            }
+        } else {
+            float4 a = reinterpret_cast<float4*>(sp)[sub];
+            float4 b = reinterpret_cast<float4*>(sp + D)[sub];
+            if (KIND == OPT_ADAM) {
+                adam_elem(o, c1, c2, gr.x, w.x, a.x, b.x);
+                adam_elem(o, c1, c2, gr.y, w.y, a.y, b.y);
+                adam_elem(o, c1, c2, gr.z, w.z, a.z, b.z);
+                adam_elem(o, c1, c2, gr.w, w.w, a.w, b.w);
+            } else {
+                ftrl_elem(o, gr.x, w.x, a.x, b.x);
+                ftrl_elem(o, gr.y, w.y, a.y, b.y);
+                ftrl_elem(o, gr.z, w.z, a.z, b.z);
+                ftrl_elem(o, gr.w, w.w, a.w, b.w);
+            }
+            reinterpret_cast<float4*>(wp)[sub] = w;
+            reinterpret_cast<float4*>(sp)[sub] = a;
+            reinterpret_cast<float4*>(sp + D)[sub] = b;
+            if (sub == 0) sp[2 * D + 1] = __int_as_float(__float_as_int(sp[2 * D + 1]) + bshow);
+        }
+    }
+}
+
 // One group of LPG lanes owns one distinct sign: it loads the row once, applies
 // the sign's records in ascending record order (slot 0 first; the member list
 // is sorted) and stores the row once.  Each lane holds one float4 of every
@@ -974,20 +1118,22 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                                                    const uint32_t* __restrict__ grp_row,
                                                    const uint32_t* __restrict__ grp_off,
                                                    const uint32_t* __restrict__ grp_cnt,
-                                                   const uint2* __restrict__ list, uint32_t big_k) {
-    const uint32_t n_groups = status->n_groups;
+                                                   const Member* __restrict__ list, uint32_t big_k,
+                                                   uint32_t ids_cap) {
+    const uint32_t n_multi = status->n_multi;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;                       // my float4 inside the row
     const int lane = (int)__lane_id();
     const int lane0 = lane - sub;                            // first lane of my group in the wavefront
     const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
-    for (uint32_t g = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; g < n_groups; g += gstride) {
+    for (uint32_t gi = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; gi < n_multi; gi += gstride) {
+        const uint32_t g = ids_cap - n_multi + gi;  // groups with several records sit at the top of the id space
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
-        const uint2* mem = list + grp_off[g];
+        const Member* mem = list + grp_off[g];
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         float4 w = reinterpret_cast<float4*>(wp)[sub];
@@ -1091,7 +1237,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                                                   const uint32_t* __restrict__ grp_row,
                                                   const uint32_t* __restrict__ grp_off,
                                                   const uint32_t* __restrict__ grp_cnt,
-                                                  const uint2* __restrict__ list) {
+                                                  const Member* __restrict__ list) {
     __shared__ float rw[BIG_DIM_MAX], ra[BIG_DIM_MAX], rb[BIG_DIM_MAX];
     __shared__ float gbuf[BIG_GBUF];
     __shared__ const float* gptr[64];
@@ -1235,16 +1381,18 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
                                                       const uint32_t* __restrict__ grp_row,
                                                       const uint32_t* __restrict__ grp_off,
                                                       const uint32_t* __restrict__ grp_cnt,
-                                                      const uint2* __restrict__ list, uint32_t big_k) {
-    const uint32_t n_groups = status->n_groups;
+                                                      const Member* __restrict__ list, uint32_t big_k,
+                                                      uint32_t ids_cap) {
+    const uint32_t n_single = status->n_single, n_multi = status->n_multi;
     const int D = s.D;
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < n_groups; g += stride) {
+    for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < n_single + n_multi; t += stride) {
+        const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
-        const uint2* mem = list + grp_off[g];
+        const Member* mem = list + grp_off[g];
         float* w = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         for (uint32_t j = 0; j < k; j++) {

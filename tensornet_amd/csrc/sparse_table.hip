@@ -301,12 +301,13 @@ struct Plan {
     uint32_t* u_of_gi;     // lookup -> index of its distinct sign
     uint64_t* uniq_sign;   // per-slot distinct signs, slot-major, first-occurrence order
     uint32_t* uniq_slot;
-    int2* ucnt;            // {batch_show, batch_click} per distinct sign (push)
+    uint32_t* ushow;       // batch_show per distinct sign, when the remap already knows it
     uint64_t* grp_sign;    // distinct signs over all slots
     uint32_t* grp_row;     // their table rows
     uint32_t* grp_off;
     uint32_t* grp_cnt;
-    uint2* list;           // members {index into uniq_*, slot} of every group, ascending
+    Member* list;          // members of every group, ascending (with their show / click counts)
+    uint32_t* pos_of_u;    // record -> its place in `list`
     uint32_t* g_of_u;      // record -> its group
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     uint32_t* newlist;     // groups whose row was inserted by the pull
@@ -349,7 +350,8 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_row = c.take<uint32_t>(n);
     p.grp_off = c.take<uint32_t>(n);
     p.grp_cnt = c.take<uint32_t>(n);
-    p.list = c.take<uint2>(n);
+    p.list = c.take<Member>(n);
+    p.pos_of_u = c.take<uint32_t>(n);
     p.g_of_u = c.take<uint32_t>(n);
     p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
     p.newlist = c.take<uint32_t>(n);
@@ -371,7 +373,7 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     p.u_of_gi = c.take<uint32_t>(L);
     p.uniq_sign = c.take<uint64_t>(L);
     p.uniq_slot = c.take<uint32_t>(L);
-    p.ucnt = c.take<int2>(L);
+    p.ushow = c.take<uint32_t>(L);
     carve_groups(c, p, L);
     return align_up(c.off, 256);
 }
@@ -465,8 +467,9 @@ int upload_slots(SparseTable* t, const Plan& p, const std::vector<SlotDesc>& des
     const size_t lb = lbase.size() * sizeof(uint32_t);
     std::memcpy(t->hstage, descs.data(), db);
     std::memcpy(t->hstage + db, lbase.data(), lb);
-    TN_HIP(hipMemcpyAsync(p.descs, t->hstage, db, hipMemcpyHostToDevice, st));
-    TN_HIP(hipMemcpyAsync(p.lbase, t->hstage + db, lb, hipMemcpyHostToDevice, st));
+    TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)(db + lb) / 4, 256, 64)), dim3(256), st,
+              reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(p.descs), (uint32_t)(db / 4),
+              p.lbase, (uint32_t)(lb / 4));
     TN_HIP(hipEventRecord(t->stage_ev, st));
     t->stage_pending = true;
     return TN_OK;
@@ -477,7 +480,6 @@ PushSrc op_source(const Plan& p, int dim) {
     src.uniq_sign = p.uniq_sign;
     src.uniq_slot = p.uniq_slot;
     src.ubase = p.ubase;
-    src.ucnt = p.ucnt;
     src.descs = p.descs;
     src.dim = dim;
     return src;
@@ -487,7 +489,7 @@ PushSrc op_source(const Plan& p, int dim) {
 // and member lists in ascending record order.  Works for any records: arrival
 // order by atomics, then every record finds its place among its group's members.
 void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_t n_host, int64_t n_upper,
-                     uint32_t big_k, DevStatus* ds, hipStream_t st) {
+                     uint32_t big_k, const uint32_t* ushow, DevStatus* ds, hipStream_t st) {
     const uint32_t* n_dev = src.infos ? nullptr : &ds->n_unique;
     GroupEntry* gt = static_cast<GroupEntry*>(w.gt);
     const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
@@ -495,26 +497,27 @@ void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_
     TN_LAUNCH(k_fill_groups, dim3(tblocks), dim3(256), st, gt, ds);
     TN_LAUNCH(k_group_insert, dim3(gblocks), dim3(256), st, src, n_host, ds, gt, w.gidx, w.ord);
     TN_LAUNCH(k_group_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
-              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
+              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k, (uint32_t)n_upper);
     TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.ord, w.arrival);
     TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.arrival,
-              src.uniq_slot, p.list, p.g_of_u);
+              src.uniq_slot, ushow, p.list, p.g_of_u, p.pos_of_u);
 }
 
 constexpr int MASK_SLOTS = 128;
 
 
 // The same result for the distinct signs of an op with at most 128 slots, from slot masks.
-void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint32_t big_k, DevStatus* ds,
-                          hipStream_t st) {
+void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint32_t big_k, const uint32_t* ushow,
+                          DevStatus* ds, hipStream_t st) {
     MaskEntry* gt = static_cast<MaskEntry*>(w.gt);
     const int gblocks = launch_grid(n_upper, 256, GRID_CAP * 2);
     const int tblocks = launch_grid(2 * (int64_t)group_cap(n_upper) + 2, 256, GRID_CAP * 2);
     TN_LAUNCH(k_fill_masks, dim3(tblocks), dim3(256), st, gt, ds);
     TN_LAUNCH(k_mask_insert, dim3(gblocks), dim3(256), st, p.uniq_sign, p.uniq_slot, ds, gt, w.gidx);
     TN_LAUNCH(k_mask_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
-              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k);
-    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, p.list, p.g_of_u);
+              dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k, (uint32_t)n_upper);
+    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, ushow, p.list, p.g_of_u,
+              p.pos_of_u);
 }
 
 // Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids,
@@ -530,7 +533,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
         TN_LAUNCH(k_zero_u32, dim3(launch_grid(w.nbuckets + 1, 256, 64)), dim3(256), st, w.bcount, w.nbuckets + 1);
         TN_LAUNCH(k_lds_hist, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy, w.first_of,
-                  w.cnt_at, ds);
+                  ds);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
         TN_LAUNCH(k_lds_scatter, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcursor, w.pkey, w.pgi);
         TN_LAUNCH(k_lds_dedup, dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart, w.nbuckets,
@@ -538,7 +541,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
         TN_LAUNCH(k_lds_assign, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8, w.tileoff,
-                  w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ucnt);
+                  w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
         TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.rank_at,
                   p.u_of_gi);
     } else {
@@ -553,15 +556,16 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
         TN_LAUNCH(k_write_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.dt, w.tidx, w.flag8,
                   p.u_of_gi, for_pull ? 1 : 0);
     }
+    const uint32_t* ushow = use_lds ? p.ushow : nullptr;
     if (N <= MASK_SLOTS)
-        launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ds, st);
+        launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
     else
-        launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ds, st);
+        launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ushow, ds, st);
     if (for_pull)
-        TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, &ds->n_groups, p.grp_row,
-                  p.newlist, ds, (uint32_t)DEV_ERR_TABLE_FULL);
+        TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row, p.newlist,
+                  ds, (uint32_t)DEV_ERR_TABLE_FULL);
     else
-        TN_LAUNCH((k_probe<false>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, &ds->n_groups, p.grp_row,
+        TN_LAUNCH((k_probe<false>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row,
                   (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
 }
 
@@ -569,9 +573,14 @@ template <int KIND>
 void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds, const Plan& p,
                        int64_t n_upper, hipStream_t st) {
     const uint32_t big_k = big_threshold(s);
-#define TN_LAUNCH_VEC(LPG)                                                                                   \
-    TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, o, \
-              src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k)
+    const uint32_t ids_cap = (uint32_t)n_upper;
+#define TN_LAUNCH_VEC(LPG)                                                                                        \
+    do {                                                                                                          \
+        TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
+                  o, src, ds, p.grp_row, p.list);                                                                 \
+        TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256), st, s, \
+                  o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);                           \
+    } while (0)
     switch (lpg) {
         case 1: TN_LAUNCH_VEC(1); break;
         case 2: TN_LAUNCH_VEC(2); break;
@@ -581,7 +590,7 @@ void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& 
         case 32: TN_LAUNCH_VEC(32); break;
         default:
             TN_LAUNCH((k_apply_scalar<KIND>), dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, s, o, src, ds,
-                      p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k);
+                      p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);
     }
 #undef TN_LAUNCH_VEC
     if (big_k != 0xFFFFFFFFu)
@@ -765,7 +774,7 @@ int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int 
     const OptDev o = make_optdev(t);
     const int blocks = launch_grid(n, 256, GRID_CAP * 2);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
-    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
     TN_LAUNCH(k_init_rows, dim3(blocks), dim3(256), st, s, o, t->seed, signs, rows, newlist, t->dstatus);
     TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     if (wdim % 4 == 0 && s.wstride % 4 == 0 && aligned16(out))
@@ -817,9 +826,9 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
     src.dim = dim;
     DevStatus* ds = t->dstatus;
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, (uint32_t)n, (uint32_t)group_cap((size_t)n));
-    launch_grouping(p, w, src, n, n, big_threshold(t->store), ds, st);
+    launch_grouping(p, w, src, n, n, big_threshold(t->store), nullptr, ds, st);
     TN_LAUNCH((k_probe<false>), dim3(launch_grid(n, 256, GRID_CAP * 2)), dim3(256), st, t->store, p.grp_sign,
-              (int64_t)0, &ds->n_groups, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+              (int64_t)0, ds, (uint32_t)n, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
     launch_apply(t, p, src, ds, n, aligned16(grads) && dim % 4 == 0, st);
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
@@ -851,7 +860,7 @@ int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const floa
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
-    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
     TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     TN_LAUNCH(k_load_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state);
     TN_HIP(hipGetLastError());
@@ -881,7 +890,7 @@ int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t 
     uint32_t* rows = (uint32_t*)t->ws.p;
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
-    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const uint32_t*)nullptr, rows, (uint32_t*)nullptr, t->dstatus, 0u);
+    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, (uint32_t*)nullptr, t->dstatus, 0u);
     TN_LAUNCH(k_export_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state, found);
     TN_HIP(hipGetLastError());
     TN_HIP(hipStreamSynchronize(st));
@@ -953,8 +962,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
                       p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
         TN_HIP(hipGetLastError());
-        TN_HIP(hipMemcpyAsync(&t->hpull->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
-        TN_HIP(hipMemcpyAsync(t->hpull->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+        TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
+                  reinterpret_cast<uint32_t*>(t->hpull));
         t->pull_pending = true;
         t->pending_slots = N;
         t->pending_rows.assign(var_rows, var_rows + N);
@@ -1026,7 +1035,7 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_begin_push, dim3(1), dim3(64), st, ds);
         TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
                   (uint32_t)L, p.vals_copy, &ds->mismatch);
-        TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+        TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush));
         TN_HIP(hipStreamSynchronize(st));
         reuse = t->hpush->st.mismatch == 0;
     }
@@ -1046,18 +1055,18 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
     if (has_show) {
         if (with_click) {
-            TN_LAUNCH(k_reset_clicks, dim3(lblocks), dim3(256), st, p.ucnt, ds);
-            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt);
+            TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
+            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
+                      p.pos_of_u, p.list);
         }
     } else {
-        TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.ucnt, ds);
+        TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
         TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256),
-                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.ucnt, with_click ? 1 : 0);
+                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.pos_of_u, p.list, with_click ? 1 : 0);
     }
     launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
     TN_HIP(hipGetLastError());
-    TN_HIP(hipMemcpyAsync(&t->hpush->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
-    TN_HIP(hipMemcpyAsync(t->hpush->ubase, p.ubase, (N + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush));
     t->push_pending = true;
     t->pending_slots = N;
     return TN_OK;

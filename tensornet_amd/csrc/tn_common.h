@@ -81,12 +81,14 @@ enum : uint32_t {
 struct DevStatus {
     uint32_t err;        // DEV_ERR_* bits
     uint32_t n_unique;   // U = sum of per-slot distinct signs
-    uint32_t n_groups;   // globally distinct signs of a push
+    uint32_t n_single;   // distinct signs (groups) with one record: numbered 0 .. n_single-1
+    uint32_t n_multi;    // groups with several records: numbered downwards from the top of the id space
     uint32_t n_new;      // rows inserted by this call
     uint32_t gcap;       // slots of the per-call group table
-    uint32_t list_cursor;
+    uint32_t n_members;  // records in groups with several records (their lists fill the member array from the top)
     uint32_t mismatch;   // a push found other signs than the plan was built from
     uint32_t n_big;      // groups with many records (handled one wavefront each)
+    uint32_t pad[3];
 };
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
