@@ -21,6 +21,14 @@
 //   k_lds_assign   ranks, distinct lists, show counts
 //   k_lds_mapped   mapped ids and the per-lookup distinct index
 //
+// With at most 128 slots the groups of equal signs over all slots come out of
+// LDS too: k_lds_dedup hands every distinct (slot, sign) record -- sign, first
+// position, occurrences -- to a second level of buckets chosen by the sign's
+// hash alone (fixed room per bucket, one global atomic per touched bucket), and
+// one workgroup per such bucket (k_group_lds) finds the signs shared between
+// slots with an LDS table of slot masks, numbers the groups and writes their
+// member lists.
+//
 // If an LDS table ever overflows (more distinct signs in a bucket than it has
 // room for) DEV_ERR_REMAP_OVERFLOW is raised; every index written stays in
 // bounds and the host repeats the call on the global-table path.
@@ -37,6 +45,23 @@ constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
 constexpr int LDS_BUCKET_TARGET = 1536; // average lookups per bucket
 constexpr int LDS_MAX_SUB = 2048;       // buckets per slot at most
 constexpr int LDS_TABLE = 4096;         // entries of a bucket's LDS hash table
+constexpr int LDS_SPAN2 = 512;          // second-level buckets whose counts one first-level bucket gathers in LDS
+constexpr int GRP_TARGET = 1024;        // records per second-level bucket if every lookup were distinct
+constexpr int GRP_CAP = 1536;           // room of a second-level bucket
+constexpr int GRP_TABLE = 2048;         // entries of its LDS hash table (> GRP_CAP: an insert always ends)
+constexpr int GRP_ITEMS = (GRP_TABLE + 1 + 255) / 256;
+constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
+
+// A distinct (slot, sign) record on its way to the grouping.
+struct GroupRec {
+    uint64_t sign;
+    uint32_t gi;   // position of its first occurrence
+    uint32_t cnt;  // occurrences in its slot
+};
+
+__device__ __forceinline__ uint32_t group_bucket(uint64_t sign, uint32_t nb2) {
+    return (uint32_t)__umul64hi(mix64(sign), (uint64_t)nb2);
+}
 
 // In this mode SlotDesc::tbase is the slot's first bucket and SlotDesc::tcap its number of buckets.
 __device__ __forceinline__ uint32_t bucket_of(const SlotDesc& d, uint64_t sign) {
@@ -159,13 +184,19 @@ __device__ __forceinline__ uint32_t lds_slot(uint64_t sign) { return (uint32_t)(
 
 // One workgroup per bucket.  first_of[gi] = position of the first occurrence
 // of gi's sign in its slot; cnt_at[first position] = occurrences of the sign.
+// With EMIT every distinct sign of the bucket is also appended to its
+// second-level bucket (recs[c * GRP_CAP ...], cursor2[c] = records handed in).
+template <bool EMIT>
 __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
                                                    const uint64_t* __restrict__ pkey, const uint32_t* __restrict__ pgi,
                                                    uint32_t* __restrict__ first_of, uint32_t* __restrict__ cnt_at,
-                                                   DevStatus* status) {
+                                                   DevStatus* status, uint32_t nb2, uint32_t* cursor2,
+                                                   GroupRec* __restrict__ recs) {
     __shared__ unsigned long long keys[LDS_TABLE + 1];  // entry LDS_TABLE: the sign EMPTY_KEY itself
     __shared__ uint32_t minpos[LDS_TABLE + 1];
     __shared__ uint32_t cnts[LDS_TABLE + 1];
+    __shared__ uint32_t hist2[EMIT ? LDS_SPAN2 : 1];
+    __shared__ uint32_t c_lo_sh;
     for (uint32_t b = blockIdx.x; b < nbuckets; b += gridDim.x) {
         const uint32_t lo = bstart[b], hi = bstart[b + 1];
         if (lo == hi) continue;
@@ -174,10 +205,16 @@ __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ 
             minpos[i] = 0xFFFFFFFFu;
             cnts[i] = 0;
         }
+        if (EMIT) {
+            for (int i = threadIdx.x; i < LDS_SPAN2; i += 256) hist2[i] = 0;
+            if (threadIdx.x == 0) c_lo_sh = 0xFFFFFFFFu;
+        }
         __syncthreads();
+        uint32_t c_min = 0xFFFFFFFFu;
         for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
             const uint64_t sign = pkey[i];
             const uint32_t gi = pgi[i];
+            if (EMIT) c_min = min(c_min, group_bucket(sign, nb2));
             uint32_t h = LDS_TABLE;
             if (sign != EMPTY_KEY) {
                 h = lds_slot(sign);
@@ -196,7 +233,12 @@ __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ 
             atomicMin(&minpos[h], gi);
             atomicAdd(&cnts[h], 1u);
         }
+        if (EMIT) {
+            for (int o = 32; o > 0; o >>= 1) c_min = min(c_min, (uint32_t)__shfl_xor((int)c_min, o));
+            if ((threadIdx.x & 63) == 0) atomicMin(&c_lo_sh, c_min);
+        }
         __syncthreads();
+        const uint32_t c_lo = EMIT ? c_lo_sh : 0;
         for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
             const uint64_t sign = pkey[i];
             const uint32_t gi = pgi[i];
@@ -210,7 +252,34 @@ __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ 
             }
             const uint32_t f = found ? minpos[h] : gi;
             first_of[gi] = f;
-            if (f == gi) cnt_at[gi] = found ? cnts[h] : 1u;
+            if (f == gi) {
+                cnt_at[gi] = found ? cnts[h] : 1u;
+                if (EMIT && found) {  // one lookup per occupied entry gets here
+                    const uint32_t local = group_bucket(sign, nb2) - c_lo;
+                    if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
+                }
+            }
+        }
+        if (EMIT) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < LDS_SPAN2; i += 256)
+                if (hist2[i]) hist2[i] = atomicAdd(&cursor2[c_lo + i], hist2[i]);  // this bucket's slice
+            __syncthreads();
+            for (int e = threadIdx.x; e <= LDS_TABLE; e += 256) {
+                const uint32_t cnt = cnts[e];
+                if (cnt == 0) continue;
+                GroupRec r;
+                r.sign = (e == LDS_TABLE) ? EMPTY_KEY : (uint64_t)keys[e];
+                r.gi = minpos[e];
+                r.cnt = cnt;
+                const uint32_t c = group_bucket(r.sign, nb2);
+                const uint32_t local = c - c_lo;
+                const uint32_t at = (local < LDS_SPAN2) ? atomicAdd(&hist2[local], 1u) : atomicAdd(&cursor2[c], 1u);
+                if (at < (uint32_t)GRP_CAP)
+                    recs[(size_t)c * GRP_CAP + at] = r;
+                else
+                    atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+            }
         }
         __syncthreads();
     }
@@ -235,7 +304,10 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const u
     if (threadIdx.x == 0) tilesum[blockIdx.x] = total;
 }
 
-// Ranks of the first occurrences (rank_at[gi]), distinct lists, show counts.
+// Ranks of the first occurrences (rank_at[gi]) and, with LISTS, the distinct
+// lists and show counts.  Each thread owns 8 consecutive lookups; all loads are
+// issued before any dependent store.
+template <bool LISTS>
 __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L,
     const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff, const uint32_t* __restrict__ cnt_at,
@@ -249,20 +321,41 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     if (base < L) bits = flag8[base / REMAP_ITEMS];
     uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256<uint32_t>(__popc(bits), red, nullptr);
     if (base >= L) return;
+    int sls[REMAP_ITEMS];
+    uint64_t vals[REMAP_ITEMS];
+    uint32_t cnts[REMAP_ITEMS];
     int sl = find_slot(lb, N, base);
+#pragma unroll
+    for (int j = 0; j < REMAP_ITEMS; j++) {
+        const uint32_t gi = base + j;
+        sls[j] = sl;
+        vals[j] = 0;
+        cnts[j] = 0;
+        if (gi < L) {
+            while (gi >= lb[sl + 1]) sl++;
+            sls[j] = sl;
+            if (LISTS && (bits & (1u << j))) {
+                vals[j] = (uint64_t)descs[sl].values[gi - lb[sl]];
+                cnts[j] = cnt_at[gi];
+            }
+        }
+    }
+#pragma unroll
     for (int j = 0; j < REMAP_ITEMS; j++) {
         const uint32_t gi = base + j;
         if (gi >= L) break;
-        while (gi >= lb[sl + 1]) sl++;
+        sl = sls[j];
         if (gi == lb[sl]) {
             ubase[sl] = u;
             for (int e = sl - 1; e >= 0 && lb[e] == gi; e--) ubase[e] = u;
         }
         if (bits & (1u << j)) {
             rank_at[gi] = u;
-            uniq_sign[u] = (uint64_t)descs[sl].values[gi - lb[sl]];
-            uniq_slot[u] = (uint32_t)sl;
-            ushow[u] = cnt_at[gi];  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            if (LISTS) {
+                uniq_sign[u] = vals[j];
+                uniq_slot[u] = (uint32_t)sl;
+                ushow[u] = cnts[j];  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            }
             u++;
         }
     }
@@ -284,6 +377,87 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
         u_of_gi[gi] = u | (f == gi ? FIRST_BIT : 0u);
         const int sl = find_slot(lb, N, gi);
         descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+    }
+}
+
+// One workgroup per second-level bucket: groups its records by sign (all slots
+// of a sign meet here), numbers the groups and writes their member lists in
+// ascending slot order -- the place of a record among its group's members is
+// the number of lower slots in the group's slot mask.  At most GRP_SLOTS slots.
+__global__ __launch_bounds__(256) void k_group_lds(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
+                                                   const uint32_t* __restrict__ cursor2,
+                                                   const GroupRec* __restrict__ recs,
+                                                   const uint32_t* __restrict__ rank_at, DevStatus* status,
+                                                   uint32_t ids_cap, uint32_t big_k, uint64_t* __restrict__ grp_sign,
+                                                   uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
+                                                   uint32_t* __restrict__ big_list, Member* __restrict__ list,
+                                                   uint32_t* __restrict__ pos_of_u, uint32_t* __restrict__ g_of_u) {
+    __shared__ unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
+    __shared__ unsigned long long mlo[GRP_TABLE + 1], mhi[GRP_TABLE + 1];
+    __shared__ uint32_t eg[GRP_TABLE + 1], eoff[GRP_TABLE + 1];
+    __shared__ uint16_t rech[GRP_CAP];
+    __shared__ uint32_t lb[GRP_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
+        const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+        if (n == 0) continue;
+        const GroupRec* mine = recs + (size_t)c * GRP_CAP;
+        for (int i = threadIdx.x; i <= GRP_TABLE; i += 256) {
+            keys[i] = EMPTY_KEY;
+            mlo[i] = 0;
+            mhi[i] = 0;
+        }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < n; i += 256) {
+            const GroupRec r = mine[i];
+            uint32_t h = GRP_TABLE;
+            if (r.sign != EMPTY_KEY) {
+                h = (uint32_t)(mix64(r.sign) >> 9) & (GRP_TABLE - 1);
+                for (;;) {  // n <= GRP_CAP < GRP_TABLE: a free entry exists
+                    unsigned long long old = keys[h];
+                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, r.sign);
+                    if (old == EMPTY_KEY || old == r.sign) break;
+                    h = (h + 1) & (GRP_TABLE - 1);
+                }
+            }
+            const uint32_t sl = (uint32_t)find_slot(lb, N, r.gi);
+            atomicOr(sl < 64 ? &mlo[h] : &mhi[h], 1ull << (sl & 63));
+            rech[i] = (uint16_t)h;
+        }
+        __syncthreads();
+        uint32_t ks[GRP_ITEMS];
+        for (int j = 0; j < GRP_ITEMS; j++) {
+            const uint32_t e = j * 256 + threadIdx.x;
+            ks[j] = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
+        }
+        compact_span(status, ks, ids_cap, big_k, big_list, [&](int j, uint32_t g, uint32_t off) {
+            const uint32_t e = j * 256 + threadIdx.x;
+            eg[e] = g;
+            eoff[e] = off;
+            grp_sign[g] = (e == GRP_TABLE) ? EMPTY_KEY : (uint64_t)keys[e];
+            grp_off[g] = off;
+            grp_cnt[g] = ks[j];
+        });
+        for (uint32_t i = threadIdx.x; i < n; i += 256) {
+            const GroupRec r = mine[i];
+            const uint32_t h = rech[i];
+            const uint32_t sl = (uint32_t)find_slot(lb, N, r.gi);
+            uint32_t place;
+            if (sl < 64)
+                place = (uint32_t)__popcll(mlo[h] & ((1ull << sl) - 1ull));
+            else
+                place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (sl - 64)) - 1ull));
+            const uint32_t at = eoff[h] + place;
+            Member m;
+            m.u = rank_at[r.gi];
+            m.slot = sl;
+            m.show = (int32_t)r.cnt;  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            m.click = 0;
+            list[at] = m;
+            pos_of_u[m.u] = at;
+            g_of_u[m.u] = eg[h];
+        }
+        __syncthreads();
     }
 }
 

@@ -727,21 +727,21 @@ constexpr int COMPACT_ITEMS = 16;
 // Signs with big_k records or more are applied by one wavefront each.
 __device__ __forceinline__ bool is_big(uint32_t k, uint32_t big_k) { return k >= big_k; }
 
-// Numbers the groups found in one span of 256 x COMPACT_ITEMS table entries
+// Numbers the groups found in one span of 256 x ITEMS table entries
 // (ks[j] = records of the thread's j-th entry, 0 = unused) and gives each a
 // slice of the member array.  Groups with one record get ids and member places
 // counted up from 0 (place == id); groups with several get ids counted down
 // from ids_cap - 1 and slices carved from the top of the member array; groups
 // with big_k records or more are also listed in big_list.  Four atomics per span.
 // write(j, g, off) stores the result for the thread's j-th entry.
-template <typename W>
-__device__ __forceinline__ void compact_span(DevStatus* status, const uint32_t (&ks)[COMPACT_ITEMS], uint32_t ids_cap,
+template <int ITEMS, typename W>
+__device__ __forceinline__ void compact_span(DevStatus* status, const uint32_t (&ks)[ITEMS], uint32_t ids_cap,
                                              uint32_t big_k, uint32_t* __restrict__ big_list, W write) {
     __shared__ unsigned long long sh[4];
     __shared__ uint32_t bases[4];
     unsigned long long cnt = 0;  // bits 0-31 single groups, 32-63 multi groups
     unsigned long long mem = 0;  // bits 0-39 records of multi groups, 40-63 big groups
-    for (int j = 0; j < COMPACT_ITEMS; j++) {
+    for (int j = 0; j < ITEMS; j++) {
         if (ks[j] == 1) cnt += 1ull;
         if (ks[j] > 1) {
             cnt += 1ull << 32;
@@ -761,7 +761,7 @@ __device__ __forceinline__ void compact_span(DevStatus* status, const uint32_t (
     uint32_t gm = bases[1] + (uint32_t)(ecnt >> 32);                      // multi groups before mine
     uint32_t mm = bases[2] + (uint32_t)(emem & 0xFFFFFFFFFFull);          // multi records before mine
     uint32_t bb = bases[3] + (uint32_t)(emem >> 40);
-    for (int j = 0; j < COMPACT_ITEMS; j++) {
+    for (int j = 0; j < ITEMS; j++) {
         const uint32_t k = ks[j];
         if (k == 0) continue;
         if (k == 1) {
@@ -961,9 +961,10 @@ __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, cons
 template <int VEC>
 __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status, const uint32_t* __restrict__ grp_row,
                                                      const uint32_t* __restrict__ g_of_u,
-                                                     const uint32_t* __restrict__ uniq_slot,
-                                                     const uint32_t* __restrict__ ubase,
+                                                     const uint32_t* __restrict__ ubase, int N,
                                                      const SlotDesc* __restrict__ descs) {
+    __shared__ uint32_t ub[MAX_SLOTS + 1];
+    load_lbase(ub, ubase, N);
     const int chunks = s.wdim / VEC;
     const int64_t total = (int64_t)status->n_unique * chunks;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -971,8 +972,8 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
         const int64_t u = t / chunks;
         const int c = (int)(t - u * chunks);
         const uint32_t row = grp_row[g_of_u[u]];
-        const uint32_t sl = uniq_slot[u];
-        const int64_t r = (int64_t)u - (int64_t)ubase[sl];
+        const int sl = find_slot(ub, N, (uint32_t)u);  // the slot whose window of distinct indices holds u
+        const int64_t r = (int64_t)u - (int64_t)ub[sl];
         const SlotDesc& d = descs[sl];
         if (r >= d.rows) {
             if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);

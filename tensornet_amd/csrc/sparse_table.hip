@@ -332,6 +332,10 @@ struct Scratch {
     uint32_t* first_of;
     uint32_t* cnt_at;
     uint32_t* rank_at;
+    // grouping through LDS (second-level buckets)
+    uint32_t nb2;
+    uint32_t* cursor2;
+    GroupRec* recs;
     void* gt;  // GroupEntry[] or MaskEntry[]
     uint32_t* gidx;
     uint32_t* ord;
@@ -383,7 +387,10 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
     Carver c{base};
     if (use_lds) {
         w.nbuckets = (uint32_t)dt_entries;
-        w.bcount = c.take<uint32_t>(dt_entries + 1);
+        w.nb2 = (uint32_t)std::max<size_t>(1, (L + GRP_TARGET - 1) / GRP_TARGET);
+        w.bcount = c.take<uint32_t>(dt_entries + 1 + w.nb2);  // zeroed together
+        w.cursor2 = w.bcount + dt_entries + 1;
+        w.recs = c.take<GroupRec>((size_t)w.nb2 * GRP_CAP);
         w.bstart = c.take<uint32_t>(dt_entries + 1);
         w.bcursor = c.take<uint32_t>(dt_entries + 1);
         w.pkey = c.take<uint64_t>(L);
@@ -529,19 +536,29 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
     const Store& s = t->store;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, 0u, 0u);
+    const bool lds_groups = use_lds && N <= GRP_SLOTS;
     if (use_lds) {
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
-        TN_LAUNCH(k_zero_u32, dim3(launch_grid(w.nbuckets + 1, 256, 64)), dim3(256), st, w.bcount, w.nbuckets + 1);
+        TN_LAUNCH(k_zero_u32, dim3(launch_grid(w.nbuckets + 1 + w.nb2, 256, 64)), dim3(256), st, w.bcount,
+                  w.nbuckets + 1 + w.nb2);
         TN_LAUNCH(k_lds_hist, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy, w.first_of,
                   ds);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
         TN_LAUNCH(k_lds_scatter, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcursor, w.pkey, w.pgi);
-        TN_LAUNCH(k_lds_dedup, dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart, w.nbuckets,
-                  w.pkey, w.pgi, w.first_of, w.cnt_at, ds);
+        if (lds_groups)
+            TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart,
+                      w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
+        else
+            TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart,
+                      w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
-        TN_LAUNCH(k_lds_assign, dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8, w.tileoff,
-                  w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+        if (lds_groups)
+            TN_LAUNCH((k_lds_assign<false>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
+                      w.tileoff, w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+        else
+            TN_LAUNCH((k_lds_assign<true>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
+                      w.tileoff, w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
         TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.rank_at,
                   p.u_of_gi);
     } else {
@@ -557,7 +574,11 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
                   p.u_of_gi, for_pull ? 1 : 0);
     }
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
-    if (N <= MASK_SLOTS)
+    if (lds_groups)
+        TN_LAUNCH(k_group_lds, dim3(launch_grid(w.nb2, 1, GRID_CAP * 2)), dim3(256), st, p.lbase, N, w.nb2, w.cursor2,
+                  w.recs, w.rank_at, ds, L, big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list,
+                  p.pos_of_u, p.g_of_u);
+    else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
     else
         launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ushow, ds, st);
@@ -594,7 +615,7 @@ void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& 
     }
 #undef TN_LAUNCH_VEC
     if (big_k != 0xFFFFFFFFu)
-        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, GRID_CAP * 2)), dim3(64), st, s, o,
+        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64), st, s, o,
                   src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list);
 }
 
@@ -957,10 +978,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
-                      ds, p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
+                      ds, p.grp_row, p.g_of_u, p.ubase, N, p.descs);
         else
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
-                      p.grp_row, p.g_of_u, p.uniq_slot, p.ubase, p.descs);
+                      p.grp_row, p.g_of_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
         TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
                   reinterpret_cast<uint32_t*>(t->hpull));
