@@ -25,8 +25,9 @@
 // LDS too: k_lds_dedup hands every distinct (slot, sign) record -- sign, first
 // position, occurrences -- to a second level of buckets chosen by the sign's
 // hash alone (fixed room per bucket, one global atomic per touched bucket), and
-// one workgroup per such bucket (k_group_lds) finds the signs shared between
-// slots with an LDS table of slot masks, numbers the groups and writes their
+// one workgroup per such bucket (k_group_count) finds the signs shared between
+// slots with an LDS table of slot masks; a scan over the buckets' counts
+// (k_group_offsets) then numbers the groups, and k_group_emit writes their
 // member lists.
 //
 // If an LDS table ever overflows (more distinct signs in a bucket than it has
@@ -381,27 +382,32 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
 }
 
 // One workgroup per second-level bucket: groups its records by sign (all slots
-// of a sign meet here), numbers the groups and writes their member lists in
-// ascending slot order -- the place of a record among its group's members is
-// the number of lower slots in the group's slot mask.  At most GRP_SLOTS slots.
-__global__ __launch_bounds__(256) void k_group_lds(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
-                                                   const uint32_t* __restrict__ cursor2,
-                                                   const GroupRec* __restrict__ recs,
-                                                   const uint32_t* __restrict__ rank_at, DevStatus* status,
-                                                   uint32_t ids_cap, uint32_t big_k, uint64_t* __restrict__ grp_sign,
-                                                   uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
-                                                   uint32_t* __restrict__ big_list, Member* __restrict__ list,
-                                                   uint32_t* __restrict__ pos_of_u, uint32_t* __restrict__ g_of_u) {
+// of a sign meet here) with an LDS table of slot masks.  The place of a record
+// among its group's members (ascending slot order) is the number of lower
+// slots in the mask.  Per record it leaves
+//   x: bits 0-11 index of its group among the bucket's groups of the same kind
+//      (one record / several), 12-23 index among the bucket's big groups, 24-31 records k of the group
+//   y: bits 0-15 records of the bucket's earlier several-record groups, 16-23 place, 24-31 slot
+// and per bucket the number of groups with one record, with several, the
+// records of the latter, and the big groups.  At most GRP_SLOTS slots.
+__global__ __launch_bounds__(256) void k_group_count(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
+                                                     const uint32_t* __restrict__ cursor2,
+                                                     const GroupRec* __restrict__ recs, uint32_t big_k,
+                                                     uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
     __shared__ unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
     __shared__ unsigned long long mlo[GRP_TABLE + 1], mhi[GRP_TABLE + 1];
-    __shared__ uint32_t eg[GRP_TABLE + 1], eoff[GRP_TABLE + 1];
+    __shared__ uint32_t einfo[GRP_TABLE + 1], eoffs[GRP_TABLE + 1];
     __shared__ uint16_t rech[GRP_CAP];
     __shared__ uint32_t lb[GRP_SLOTS + 1];
+    __shared__ unsigned long long sh[4];
     load_lbase(lb, lbase, N);
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
-        if (n == 0) continue;
-        const GroupRec* mine = recs + (size_t)c * GRP_CAP;
+        if (n == 0) {
+            if (threadIdx.x == 0) bcounts[c] = make_uint4(0, 0, 0, 0);
+            continue;
+        }
+        const size_t first = (size_t)c * GRP_CAP;
         for (int i = threadIdx.x; i <= GRP_TABLE; i += 256) {
             keys[i] = EMPTY_KEY;
             mlo[i] = 0;
@@ -409,7 +415,7 @@ __global__ __launch_bounds__(256) void k_group_lds(const uint32_t* __restrict__ 
         }
         __syncthreads();
         for (uint32_t i = threadIdx.x; i < n; i += 256) {
-            const GroupRec r = mine[i];
+            const GroupRec r = recs[first + i];
             uint32_t h = GRP_TABLE;
             if (r.sign != EMPTY_KEY) {
                 h = (uint32_t)(mix64(r.sign) >> 9) & (GRP_TABLE - 1);
@@ -426,28 +432,122 @@ __global__ __launch_bounds__(256) void k_group_lds(const uint32_t* __restrict__ 
         }
         __syncthreads();
         uint32_t ks[GRP_ITEMS];
+        unsigned long long v = 0;  // 16-bit fields: groups of one record, of several, records of those, big groups
         for (int j = 0; j < GRP_ITEMS; j++) {
             const uint32_t e = j * 256 + threadIdx.x;
-            ks[j] = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
+            const uint32_t k = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
+            ks[j] = k;
+            if (k == 1) v += 1ull;
+            if (k > 1) v += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
         }
-        compact_span(status, ks, ids_cap, big_k, big_list, [&](int j, uint32_t g, uint32_t off) {
+        unsigned long long total;
+        unsigned long long ex = block_excl_scan_256<unsigned long long>(v, sh, &total);
+        if (threadIdx.x == 0)
+            bcounts[c] = make_uint4((uint32_t)(total & 0xFFFF), (uint32_t)((total >> 16) & 0xFFFF),
+                                    (uint32_t)((total >> 32) & 0xFFFF), (uint32_t)(total >> 48));
+        for (int j = 0; j < GRP_ITEMS; j++) {
+            const uint32_t k = ks[j];
+            if (k == 0) continue;
             const uint32_t e = j * 256 + threadIdx.x;
-            eg[e] = g;
-            eoff[e] = off;
-            grp_sign[g] = (e == GRP_TABLE) ? EMPTY_KEY : (uint64_t)keys[e];
-            grp_off[g] = off;
-            grp_cnt[g] = ks[j];
-        });
+            if (k == 1) {
+                einfo[e] = (uint32_t)(ex & 0xFFFF) | (1u << 24);
+                eoffs[e] = 0;
+                ex += 1ull;
+            } else {
+                einfo[e] = (uint32_t)((ex >> 16) & 0xFFFF) | ((uint32_t)(ex >> 48) << 12) | (k << 24);
+                eoffs[e] = (uint32_t)((ex >> 32) & 0xFFFF);
+                ex += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
+            }
+        }
+        __syncthreads();
         for (uint32_t i = threadIdx.x; i < n; i += 256) {
-            const GroupRec r = mine[i];
             const uint32_t h = rech[i];
-            const uint32_t sl = (uint32_t)find_slot(lb, N, r.gi);
+            const uint32_t sl = (uint32_t)find_slot(lb, N, recs[first + i].gi);
             uint32_t place;
             if (sl < 64)
                 place = (uint32_t)__popcll(mlo[h] & ((1ull << sl) - 1ull));
             else
                 place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (sl - 64)) - 1ull));
-            const uint32_t at = eoff[h] + place;
+            aux[first + i] = make_uint2(einfo[h], eoffs[h] | (place << 16) | (sl << 24));
+        }
+        __syncthreads();
+    }
+}
+
+// Exclusive scan of the per-bucket counts (one workgroup); also the totals.
+__global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict__ bcounts, uint4* __restrict__ bbase,
+                                                        uint32_t nb2, DevStatus* status) {
+    __shared__ uint4 wsum[16];
+    __shared__ uint4 carry_sh;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) carry_sh = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+    for (uint32_t start = 0; start < nb2; start += 1024) {
+        const uint32_t i = start + threadIdx.x;
+        const uint4 v = (i < nb2) ? bcounts[i] : make_uint4(0, 0, 0, 0);
+        uint4 inc = v;
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t tx = __shfl_up(inc.x, o), ty = __shfl_up(inc.y, o), tz = __shfl_up(inc.z, o),
+                           tw = __shfl_up(inc.w, o);
+            if (lane >= o) {
+                inc.x += tx;
+                inc.y += ty;
+                inc.z += tz;
+                inc.w += tw;
+            }
+        }
+        if (lane == 63) wsum[wave] = inc;
+        __syncthreads();
+        uint4 base = carry_sh;
+        for (int wv = 0; wv < wave; wv++) {
+            base.x += wsum[wv].x;
+            base.y += wsum[wv].y;
+            base.z += wsum[wv].z;
+            base.w += wsum[wv].w;
+        }
+        if (i < nb2) bbase[i] = make_uint4(base.x + inc.x - v.x, base.y + inc.y - v.y, base.z + inc.z - v.z, base.w + inc.w - v.w);
+        __syncthreads();
+        if (threadIdx.x == 1023) carry_sh = make_uint4(base.x + inc.x, base.y + inc.y, base.z + inc.z, base.w + inc.w);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        status->n_single = carry_sh.x;
+        status->n_multi = carry_sh.y;
+        status->n_members = carry_sh.z;
+        status->n_big = carry_sh.w;
+    }
+}
+
+// Numbers the groups and writes the member lists: groups with one record get
+// ids and member places counted up from 0 (place == id), groups with several
+// get ids counted down from ids_cap - 1 and slices carved from the top of the
+// member array, in bucket order.
+__global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+                                                    const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
+                                                    const uint4* __restrict__ bbase,
+                                                    const uint32_t* __restrict__ rank_at, uint32_t ids_cap,
+                                                    uint32_t big_k, uint64_t* __restrict__ grp_sign,
+                                                    uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
+                                                    uint32_t* __restrict__ big_list, Member* __restrict__ list,
+                                                    uint32_t* __restrict__ pos_of_u, uint32_t* __restrict__ g_of_u) {
+    for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
+        const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+        const size_t first = (size_t)c * GRP_CAP;
+        const uint4 bb = bbase[c];
+        for (uint32_t i = threadIdx.x; i < n; i += 256) {
+            const GroupRec r = recs[first + i];
+            const uint2 a = aux[first + i];
+            const uint32_t k = a.x >> 24, idx = a.x & 0xFFFu, bigidx = (a.x >> 12) & 0xFFFu;
+            const uint32_t place = (a.y >> 16) & 0xFFu, sl = a.y >> 24;
+            uint32_t g, off;
+            if (k == 1) {
+                g = bb.x + idx;
+                off = g;
+            } else {
+                g = ids_cap - 1 - (bb.y + idx);
+                off = ids_cap - (bb.z + (a.y & 0xFFFFu) + k);
+            }
+            const uint32_t at = off + place;
             Member m;
             m.u = rank_at[r.gi];
             m.slot = sl;
@@ -455,9 +555,14 @@ __global__ __launch_bounds__(256) void k_group_lds(const uint32_t* __restrict__ 
             m.click = 0;
             list[at] = m;
             pos_of_u[m.u] = at;
-            g_of_u[m.u] = eg[h];
+            g_of_u[m.u] = g;
+            if (place == 0) {
+                grp_sign[g] = r.sign;
+                grp_off[g] = off;
+                grp_cnt[g] = k;
+                if (is_big(k, big_k)) big_list[bb.w + bigidx] = g;
+            }
         }
-        __syncthreads();
     }
 }
 

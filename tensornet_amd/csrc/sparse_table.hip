@@ -49,10 +49,11 @@ struct SparseTable {
     char* hstage = nullptr;         // pinned staging of slot descriptors
     size_t hstage_bytes = 0;
     hipEvent_t stage_ev = nullptr;  // staging buffer free again
+    hipEvent_t verify_ev = nullptr; // a push's comparison of the signs has been published
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
     bool pull_pending = false;
-    int pending_slots = 0;          // N of the pending calls
+    int pull_slots = 0, push_slots = 0;  // N of the pending calls
     std::vector<int64_t> pending_rows;  // var rows of a pending async pull
     int async_pull = 0;
     int latched = TN_OK;
@@ -144,6 +145,7 @@ int ensure_side_buffers(SparseTable* t) {
     t->hstage_bytes = (size_t)MAX_SLOTS * sizeof(SlotDesc) + (MAX_SLOTS + 1) * sizeof(uint32_t);
     TN_HIP(hipHostMalloc((void**)&t->hstage, t->hstage_bytes, hipHostMallocDefault));
     TN_HIP(hipEventCreateWithFlags(&t->stage_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->verify_ev, hipEventDisableTiming));
     return TN_OK;
 }
 
@@ -183,10 +185,21 @@ void latch(SparseTable* t, int code, const std::string& msg) {
 
 // Examines the status blocks of finished calls (the stream must have been synchronised).
 void harvest(SparseTable* t) {
+    // a pending push is older than a pending pull (a push collects everything before it starts)
+    if (t->push_pending) {
+        t->push_pending = false;
+        const HostStatus& h = *t->hpush;
+        int N = t->push_slots;
+        if (N > 0) {
+            t->last_counts.assign(N, 0);
+            for (int s = 0; s < N; s++) t->last_counts[s] = (int64_t)h.ubase[s + 1] - (int64_t)h.ubase[s];
+        }
+        latch(t, dev_err_code(h.st.err), std::string("sparse push: ") + dev_err_text(h.st.err));
+    }
     if (t->pull_pending) {
         t->pull_pending = false;
         const HostStatus& h = *t->hpull;
-        int N = t->pending_slots;
+        int N = t->pull_slots;
         // the call booked room for every sign it could have inserted; keep what it did insert
         if (t->booked >= h.st.n_new) t->count_upper -= t->booked - h.st.n_new;
         t->booked = 0;
@@ -198,16 +211,6 @@ void harvest(SparseTable* t) {
                 latch(t, TN_ERR_VAR_CAPACITY,
                       "sparse pull: slot " + std::to_string(s) + " has " + std::to_string(t->last_counts[s]) +
                           " distinct signs, its variable only " + std::to_string(t->pending_rows[s]) + " rows");
-    }
-    if (t->push_pending) {
-        t->push_pending = false;
-        const HostStatus& h = *t->hpush;
-        int N = t->pending_slots;
-        if (N > 0) {
-            t->last_counts.assign(N, 0);
-            for (int s = 0; s < N; s++) t->last_counts[s] = (int64_t)h.ubase[s + 1] - (int64_t)h.ubase[s];
-        }
-        latch(t, dev_err_code(h.st.err), std::string("sparse push: ") + dev_err_text(h.st.err));
     }
 }
 
@@ -336,6 +339,9 @@ struct Scratch {
     uint32_t nb2;
     uint32_t* cursor2;
     GroupRec* recs;
+    uint2* aux;
+    uint4* bcounts;
+    uint4* bbase;
     void* gt;  // GroupEntry[] or MaskEntry[]
     uint32_t* gidx;
     uint32_t* ord;
@@ -391,6 +397,9 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.bcount = c.take<uint32_t>(dt_entries + 1 + w.nb2);  // zeroed together
         w.cursor2 = w.bcount + dt_entries + 1;
         w.recs = c.take<GroupRec>((size_t)w.nb2 * GRP_CAP);
+        w.aux = c.take<uint2>((size_t)w.nb2 * GRP_CAP);
+        w.bcounts = c.take<uint4>(w.nb2);
+        w.bbase = c.take<uint4>(w.nb2);
         w.bstart = c.take<uint32_t>(dt_entries + 1);
         w.bcursor = c.take<uint32_t>(dt_entries + 1);
         w.pkey = c.take<uint64_t>(L);
@@ -574,11 +583,14 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
                   p.u_of_gi, for_pull ? 1 : 0);
     }
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
-    if (lds_groups)
-        TN_LAUNCH(k_group_lds, dim3(launch_grid(w.nb2, 1, GRID_CAP * 2)), dim3(256), st, p.lbase, N, w.nb2, w.cursor2,
-                  w.recs, w.rank_at, ds, L, big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list,
-                  p.pos_of_u, p.g_of_u);
-    else if (N <= MASK_SLOTS)
+    if (lds_groups) {
+        const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
+        TN_LAUNCH(k_group_count, dim3(bblocks), dim3(256), st, p.lbase, N, w.nb2, w.cursor2, w.recs, big_threshold(s),
+                  w.aux, w.bcounts);
+        TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), st, w.bcounts, w.bbase, w.nb2, ds);
+        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.rank_at, L,
+                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.pos_of_u, p.g_of_u);
+    } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
     else
         launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ushow, ds, st);
@@ -806,7 +818,7 @@ int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int 
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->hpull->ubase[0] = 0;
     t->pull_pending = true;
-    t->pending_slots = 0;
+    t->pull_slots = 0;
     t->pending_rows.clear();
     return sync_table(t, st);
 }
@@ -854,7 +866,7 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->push_pending = true;
-    t->pending_slots = 0;
+    t->push_slots = 0;
     return TN_OK;
 }
 
@@ -887,7 +899,7 @@ int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const floa
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->pull_pending = true;
-    t->pending_slots = 0;
+    t->pull_slots = 0;
     t->pending_rows.clear();
     return sync_table(t, st);
 }
@@ -932,11 +944,15 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     if (var_dim != wdim)
         return fail(TN_ERR_DIM_MISMATCH, "SparseTablePull: variable dim " + std::to_string(var_dim) +
                                              " but table rows hold " + std::to_string(wdim));
-    t->last_stream = st;
-    if (t->push_pending || t->pull_pending) {
+    // An earlier push on the same stream need not be waited for: this call runs behind it and
+    // collects its status when it waits for its own work.
+    const bool same_stream = !t->last_stream || t->last_stream == st;
+    if (t->pull_pending || (t->push_pending && (t->async_pull || !same_stream))) {
+        if (!same_stream) TN_HIP(hipStreamSynchronize(t->last_stream));
         TN_HIP(hipStreamSynchronize(st));
         harvest(t);
     }
+    t->last_stream = st;
     // The remap through LDS needs the call's status on the host to fall back if a
     // bucket overflowed, so it is only used when the pull waits for its stream anyway.
     bool use_lds = !t->async_pull;
@@ -986,7 +1002,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
                   reinterpret_cast<uint32_t*>(t->hpull));
         t->pull_pending = true;
-        t->pending_slots = N;
+        t->pull_slots = N;
         t->pending_rows.assign(var_rows, var_rows + N);
         // a push of the same batch may reuse the analysis
         t->plan_valid = true;
@@ -1050,6 +1066,24 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     bool reuse = t->plan_valid && t->plan_epoch == t->epoch && t->plan_N == N &&
                  std::equal(value_lens, value_lens + N, t->plan_lens.begin());
     DevStatus* ds = t->dplan;
+    const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
+    const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
+    // show / click counts of the batch into the member lists of plan p
+    auto launch_counts = [&](bool has_show) -> int {
+        if (has_show) {
+            if (with_click) {
+                TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
+                TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
+                          p.pos_of_u, p.list);
+            }
+        } else {
+            TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
+            TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)),
+                      dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.pos_of_u, p.list,
+                      with_click ? 1 : 0);
+        }
+        return TN_OK;
+    };
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(upload_slots(t, p, descs, lbase, st));
@@ -1057,10 +1091,13 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
                   (uint32_t)L, p.vals_copy, &ds->mismatch);
         TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush));
-        TN_HIP(hipStreamSynchronize(st));
+        TN_HIP(hipEventRecord(t->verify_ev, st));
+        // The counts only touch the plan's member lists, which a mismatch discards anyway:
+        // they run while the host waits for the comparison.
+        TN_TRY(launch_counts(t->plan_has_show));
+        TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
-    bool has_show = reuse && t->plan_has_show;
     if (!reuse) {
         // another batch than the last pull's: analyse it here, on the global-table path
         // (its status cannot be waited for, a push only enqueues)
@@ -1071,25 +1108,13 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
         TN_TRY(upload_slots(t, p, descs, lbase, st));
         launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
-    }
-    const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
-    const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
-    if (has_show) {
-        if (with_click) {
-            TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
-            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
-                      p.pos_of_u, p.list);
-        }
-    } else {
-        TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
-        TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256),
-                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.pos_of_u, p.list, with_click ? 1 : 0);
+        TN_TRY(launch_counts(false));
     }
     launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
     TN_HIP(hipGetLastError());
     TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush));
     t->push_pending = true;
-    t->pending_slots = N;
+    t->push_slots = N;
     return TN_OK;
 }
 

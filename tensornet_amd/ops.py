@@ -28,84 +28,108 @@ def _require(t, dtype, what):
         raise ValueError("%s must be contiguous" % what)
 
 
+class BoundSparseTablePull:
+    """SparseTablePull bound to fixed tensors, the way an op kernel of a built
+    graph sees its inputs: arguments are validated and marshalled once, the
+    mapped-id outputs allocated once; every call only crosses the C ABI (with the
+    stream current at that moment).  Calling it returns the N mapped-id tensors."""
+
+    def __init__(self, resources, values, table_handle):
+        n = len(values)
+        if len(resources) != n:
+            raise ValueError("SparseTable pull num_inputs: %d not equal: %d" % (len(resources) + n, n * 2))
+        if n == 0:
+            raise ValueError("SparseTable pull needs at least one slot")
+        dim = None
+        for i in range(n):
+            _require(resources[i], torch.float32, "resources[%d]" % i)
+            _require(values[i], torch.int64, "values[%d]" % i)
+            if resources[i].dim() != 2:
+                raise ValueError(
+                    "sparse pull variable must Matrix(sign_id_cnt, dim), saw: %s" % (tuple(resources[i].shape),)
+                )
+            if values[i].dim() != 1:
+                raise ValueError("values[%d] must have rank 1" % i)
+            if dim is None:
+                dim = resources[i].shape[1]
+            elif dim != resources[i].shape[1]:
+                raise _lib.TensorNetError(3, "all variables of one pull must have the same dim")
+        lens = [v.numel() for v in values]
+        # one allocation for all mapped ids, handed out as per-slot views
+        flat = torch.empty(sum(lens), dtype=torch.int64, device=values[0].device)
+        self.mapped = list(flat.split(lens)) if sum(lens) > 0 else [torch.empty_like(v) for v in values]
+        self._keep = (list(resources), list(values), flat)
+        self._fn = _lib.load().tn_sparse_table_pull_op
+        self._args = (
+            table_handle,
+            n,
+            _lib.ptr_array([v.data_ptr() for v in values]),
+            _lib.i64_array(lens),
+            _lib.ptr_array([r.data_ptr() for r in resources]),
+            _lib.i64_array([r.shape[0] for r in resources]),
+            int(dim),
+            _lib.ptr_array([m.data_ptr() for m in self.mapped]),
+        )
+
+    def __call__(self):
+        _lib.check(self._fn(*self._args, _stream()))
+        return self.mapped
+
+
+class BoundSparseTablePush:
+    """SparseTablePush bound to fixed tensors (see BoundSparseTablePull)."""
+
+    def __init__(self, values, grads, feature_labels, table_handle):
+        n = len(values)
+        if len(grads) != n or len(feature_labels) != n:
+            raise ValueError(
+                "SparseTable push num_inputs: %d not equal: %d" % (n + len(grads) + len(feature_labels), n * 3)
+            )
+        if n == 0:
+            raise ValueError("SparseTable push needs at least one slot")
+        dim = None
+        for i in range(n):
+            _require(values[i], torch.int64, "values[%d]" % i)
+            _require(grads[i], torch.float32, "grads[%d]" % i)
+            _require(feature_labels[i], torch.int64, "feature_labels[%d]" % i)
+            if grads[i].dim() != 2:
+                raise ValueError("sparse push grad must Matrix(sign_id_cnt, dim), saw: %s" % (tuple(grads[i].shape),))
+            if feature_labels[i].numel() != values[i].numel():
+                raise ValueError("feature_labels[%d] must have one label per lookup" % i)
+            if dim is None:
+                dim = grads[i].shape[1]
+            elif dim != grads[i].shape[1]:
+                raise _lib.TensorNetError(3, "all gradients of one push must have the same dim")
+        self._keep = (list(values), list(grads), list(feature_labels))
+        self._fn = _lib.load().tn_sparse_table_push_op
+        self._args = (
+            table_handle,
+            n,
+            _lib.ptr_array([v.data_ptr() for v in values]),
+            _lib.i64_array([v.numel() for v in values]),
+            _lib.ptr_array([g.data_ptr() for g in grads]),
+            _lib.i64_array([g.shape[0] for g in grads]),
+            int(dim),
+            _lib.ptr_array([l.data_ptr() for l in feature_labels]),
+        )
+
+    def __call__(self):
+        _lib.check(self._fn(*self._args, _stream()))
+
+
 def sparse_table_pull(resources, values, table_handle):
     """SparseTablePull.  resources: N float32 variables [rows, dim] (updated in
     place: row j <- embedding of the j-th distinct sign of the slot);
     values: N int64 rank-1 tensors of signs.  Returns N int64 tensors of mapped
     ids (same shapes as values)."""
-    n = len(values)
-    if len(resources) != n:
-        raise ValueError("SparseTable pull num_inputs: %d not equal: %d" % (len(resources) + n, n * 2))
-    if n == 0:
-        raise ValueError("SparseTable pull needs at least one slot")
-    dim = None
-    for i in range(n):
-        _require(resources[i], torch.float32, "resources[%d]" % i)
-        _require(values[i], torch.int64, "values[%d]" % i)
-        if resources[i].dim() != 2:
-            raise ValueError(
-                "sparse pull variable must Matrix(sign_id_cnt, dim), saw: %s" % (tuple(resources[i].shape),)
-            )
-        if values[i].dim() != 1:
-            raise ValueError("values[%d] must have rank 1" % i)
-        if dim is None:
-            dim = resources[i].shape[1]
-        elif dim != resources[i].shape[1]:
-            raise _lib.TensorNetError(3, "all variables of one pull must have the same dim")
-    mapped = [torch.empty_like(v) for v in values]
-    lib = _lib.load()
-    rc = lib.tn_sparse_table_pull_op(
-        table_handle,
-        n,
-        _lib.ptr_array([v.data_ptr() for v in values]),
-        _lib.i64_array([v.numel() for v in values]),
-        _lib.ptr_array([r.data_ptr() for r in resources]),
-        _lib.i64_array([r.shape[0] for r in resources]),
-        int(dim),
-        _lib.ptr_array([m.data_ptr() for m in mapped]),
-        _stream(),
-    )
-    _lib.check(rc)
-    return mapped
+    return BoundSparseTablePull(resources, values, table_handle)()
 
 
 def sparse_table_push(values, grads, feature_labels, table_handle):
     """SparseTablePush.  grads[i] is [U_i, dim] with row j the gradient of the
     j-th distinct sign of values[i]; feature_labels[i] has one int64 label per
     lookup.  Returns nothing (the update is enqueued on the current stream)."""
-    n = len(values)
-    if len(grads) != n or len(feature_labels) != n:
-        raise ValueError(
-            "SparseTable push num_inputs: %d not equal: %d" % (n + len(grads) + len(feature_labels), n * 3)
-        )
-    if n == 0:
-        raise ValueError("SparseTable push needs at least one slot")
-    dim = None
-    for i in range(n):
-        _require(values[i], torch.int64, "values[%d]" % i)
-        _require(grads[i], torch.float32, "grads[%d]" % i)
-        _require(feature_labels[i], torch.int64, "feature_labels[%d]" % i)
-        if grads[i].dim() != 2:
-            raise ValueError("sparse push grad must Matrix(sign_id_cnt, dim), saw: %s" % (tuple(grads[i].shape),))
-        if feature_labels[i].numel() != values[i].numel():
-            raise ValueError("feature_labels[%d] must have one label per lookup" % i)
-        if dim is None:
-            dim = grads[i].shape[1]
-        elif dim != grads[i].shape[1]:
-            raise _lib.TensorNetError(3, "all gradients of one push must have the same dim")
-    lib = _lib.load()
-    rc = lib.tn_sparse_table_push_op(
-        table_handle,
-        n,
-        _lib.ptr_array([v.data_ptr() for v in values]),
-        _lib.i64_array([v.numel() for v in values]),
-        _lib.ptr_array([g.data_ptr() for g in grads]),
-        _lib.i64_array([g.shape[0] for g in grads]),
-        int(dim),
-        _lib.ptr_array([l.data_ptr() for l in feature_labels]),
-        _stream(),
-    )
-    _lib.check(rc)
+    BoundSparseTablePush(values, grads, feature_labels, table_handle)()
 
 
 def sparse_table_sync(table_handle):

@@ -414,6 +414,54 @@ def test_push_of_another_batch_than_the_last_pull(tn, oracle):
     pair.assert_rows_match(base)
 
 
+def test_bound_ops_over_several_steps_without_waiting(tn, oracle):
+    """Ops bound to their tensors once and called step after step: a pull runs behind
+    the push before it without the host waiting in between, and a push whose signs were
+    overwritten in place since the pull notices it."""
+    D = 16
+    rng = np.random.default_rng(33)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000)
+    vocab = 30000
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    batches = [random_batch(rng, 6, 9000, vocab) for _ in range(3)]  # large enough for the remap through LDS
+    bound = []
+    for values in batches:
+        gvalues = [dev(v) for v in values]
+        gvars = [torch.zeros((len(v) + 1, D), device="cuda") for v in values]
+        counts = [len(np.unique(v)) for v in values]
+        grads = synth.make_grads(counts, D, 0.01, seed=len(bound))
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        pull = tn.ops.BoundSparseTablePull(gvars, gvalues, pair.h)
+        push = tn.ops.BoundSparseTablePush(gvalues, [dev(g) for g in grads], [dev(l) for l in labels], pair.h)
+        bound.append((values, gvalues, gvars, grads, labels, pull, push))
+    for step in range(6):
+        values, gvalues, gvars, grads, labels, pull, push = bound[step % 3]
+        cvars = [np.zeros((len(v) + 1, D), np.float32) for v in values]
+        rc, cmapped, counts = pair.o.pull_op(values, cvars)
+        assert rc == 0
+        gmapped = pull()
+        for s in range(len(values)):
+            assert (gmapped[s].cpu().numpy() == cmapped[s]).all()
+            np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
+        assert pair.o.push_op(values, grads, labels)[0] == 0
+        push()
+    tn.ops.sparse_table_sync(pair.h)
+    pair.assert_rows_match(base)
+    # same tensors, other signs in two places: the push must not use the pull's analysis
+    values, gvalues, gvars, grads, labels, pull, push = bound[0]
+    pull()
+    pair.o.pull_op(values, [np.zeros((len(v) + 1, D), np.float32) for v in values])
+    changed = [v.copy() for v in values]
+    s0 = max(range(len(values)), key=lambda s: len(values[s]))
+    other = int(np.flatnonzero(changed[s0] != changed[s0][0])[0])
+    changed[s0][0], changed[s0][other] = changed[s0][other], changed[s0][0]  # same distinct signs, other order
+    gvalues[s0].copy_(dev(changed[s0]))
+    assert pair.o.push_op(changed, grads, labels)[0] == 0
+    push()
+    tn.ops.sparse_table_sync(pair.h)
+    pair.assert_rows_match(base)
+
+
 @pytest.mark.parametrize("opt,hyper", [("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP)])
 def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper):
     """SparseTable::Push applies records in array order however often a sign repeats:
