@@ -46,11 +46,17 @@ constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
 constexpr int LDS_BUCKET_TARGET = 1536; // average lookups per bucket
 constexpr int LDS_MAX_SUB = 2048;       // buckets per slot at most
 constexpr int LDS_TABLE = 4096;         // entries of a bucket's LDS hash table
+constexpr int DEDUP_THREADS = 1024;     // a bucket's phases are short and separated by barriers: many wavefronts hide them
+constexpr int DEDUP_ITEMS = 2;          // lookups a thread of k_lds_dedup holds in registers
 constexpr int LDS_SPAN2 = 512;          // second-level buckets whose counts one first-level bucket gathers in LDS
 constexpr int GRP_TARGET = 1024;        // records per second-level bucket if every lookup were distinct
 constexpr int GRP_CAP = 1536;           // room of a second-level bucket
 constexpr int GRP_TABLE = 2048;         // entries of its LDS hash table (> GRP_CAP: an insert always ends)
-constexpr int GRP_ITEMS = (GRP_TABLE + 1 + 255) / 256;
+constexpr int GRP_THREADS = 512;        // threads of k_group_count
+constexpr int GRP_RECS = GRP_CAP / GRP_THREADS;  // records per thread of a second-level bucket's workgroup
+static_assert(GRP_CAP % GRP_THREADS == 0 && GRP_CAP % 256 == 0 && GRP_CAP < GRP_TABLE, "a bucket fits its table and the registers of one workgroup");
+constexpr int EMIT_RECS = GRP_CAP / 256;  // records per thread of k_group_emit (256 threads)
+constexpr int GRP_ITEMS = (GRP_TABLE + 1 + GRP_THREADS - 1) / GRP_THREADS;
 constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
 
 // A distinct (slot, sign) record on its way to the grouping.
@@ -188,7 +194,7 @@ __device__ __forceinline__ uint32_t lds_slot(uint64_t sign) { return (uint32_t)(
 // With EMIT every distinct sign of the bucket is also appended to its
 // second-level bucket (recs[c * GRP_CAP ...], cursor2[c] = records handed in).
 template <bool EMIT>
-__global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
+__global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
                                                    const uint64_t* __restrict__ pkey, const uint32_t* __restrict__ pgi,
                                                    uint32_t* __restrict__ first_of, uint32_t* __restrict__ cnt_at,
                                                    DevStatus* status, uint32_t nb2, uint32_t* cursor2,
@@ -201,38 +207,79 @@ __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ 
     for (uint32_t b = blockIdx.x; b < nbuckets; b += gridDim.x) {
         const uint32_t lo = bstart[b], hi = bstart[b + 1];
         if (lo == hi) continue;
-        for (int i = threadIdx.x; i <= LDS_TABLE; i += 256) {
+        for (int i = threadIdx.x; i <= LDS_TABLE; i += DEDUP_THREADS) {
             keys[i] = EMPTY_KEY;
             minpos[i] = 0xFFFFFFFFu;
             cnts[i] = 0;
         }
         if (EMIT) {
-            for (int i = threadIdx.x; i < LDS_SPAN2; i += 256) hist2[i] = 0;
+            for (int i = threadIdx.x; i < LDS_SPAN2; i += DEDUP_THREADS) hist2[i] = 0;
             if (threadIdx.x == 0) c_lo_sh = 0xFFFFFFFFu;
         }
         __syncthreads();
-        uint32_t c_min = 0xFFFFFFFFu;
-        for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
-            const uint64_t sign = pkey[i];
-            const uint32_t gi = pgi[i];
-            if (EMIT) c_min = min(c_min, group_bucket(sign, nb2));
-            uint32_t h = LDS_TABLE;
-            if (sign != EMPTY_KEY) {
-                h = lds_slot(sign);
-                int tries = 0;
-                for (; tries < LDS_TABLE; tries++) {
-                    unsigned long long old = keys[h];
-                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
-                    if (old == EMPTY_KEY || old == sign) break;
-                    h = (h + 1) & (LDS_TABLE - 1);
-                }
-                if (tries == LDS_TABLE) {  // table full: keep indices in bounds, let the host fall back
-                    atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
-                    continue;
-                }
+        // The bucket's lookups are taken DEDUP_ITEMS per thread at a time, all loads of a round
+        // issued together; a bucket that fits one round (the usual case) is read once.
+        uint64_t sg[DEDUP_ITEMS];
+        uint32_t gp[DEDUP_ITEMS];
+        const uint32_t round = DEDUP_THREADS * DEDUP_ITEMS;
+        const bool one_round = hi - lo <= round;
+        auto load_round = [&](uint32_t base) {
+#pragma unroll
+            for (int j = 0; j < DEDUP_ITEMS; j++) {
+                const uint32_t i = base + j * DEDUP_THREADS + threadIdx.x;
+                sg[j] = (i < hi) ? pkey[i] : 0;
+                gp[j] = (i < hi) ? pgi[i] : 0xFFFFFFFFu;  // no position: nothing to do
             }
-            atomicMin(&minpos[h], gi);
-            atomicAdd(&cnts[h], 1u);
+        };
+        uint32_t c_min = 0xFFFFFFFFu;
+        for (uint32_t base = lo; base < hi; base += round) {
+            load_round(base);
+#pragma unroll
+            for (int j = 0; j < DEDUP_ITEMS; j++) {
+                const uint64_t sign = sg[j];
+                uint32_t gi = gp[j];
+                uint32_t mult = 1;
+                bool valid = gi != 0xFFFFFFFFu;
+                // A frequent sign fills whole wavefronts: the lanes that hold the same sign as the
+                // first valid lane hand their smallest position and their number to that lane,
+                // instead of queueing up on one LDS address.
+                const unsigned long long vmask = __ballot(valid);
+                if (vmask == 0) continue;
+                const int leader = __ffsll((long long)vmask) - 1;
+                const uint64_t lead_sign = ((uint64_t)(uint32_t)__shfl((int)(sign >> 32), leader) << 32) |
+                                           (uint32_t)__shfl((int)(uint32_t)sign, leader);
+                const bool same = valid && sign == lead_sign;
+                const unsigned long long smask = __ballot(same);
+                if (__popcll(smask) >= 8) {
+                    uint32_t m = same ? gi : 0xFFFFFFFFu;
+                    for (int o = 32; o > 0; o >>= 1) m = min(m, (uint32_t)__shfl_xor((int)m, o));
+                    if ((int)(threadIdx.x & 63) == leader) {
+                        gi = m;
+                        mult = (uint32_t)__popcll(smask);
+                    } else if (same) {
+                        valid = false;
+                    }
+                }
+                if (!valid) continue;
+                if (EMIT) c_min = min(c_min, group_bucket(sign, nb2));
+                uint32_t h = LDS_TABLE;
+                if (sign != EMPTY_KEY) {
+                    h = lds_slot(sign);
+                    int tries = 0;
+                    for (; tries < LDS_TABLE; tries++) {
+                        unsigned long long old = keys[h];
+                        if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
+                        if (old == EMPTY_KEY || old == sign) break;
+                        h = (h + 1) & (LDS_TABLE - 1);
+                    }
+                    if (tries == LDS_TABLE) {  // table full: keep indices in bounds, let the host fall back
+                        atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+                        continue;
+                    }
+                }
+                atomicMin(&minpos[h], gi);
+                atomicAdd(&cnts[h], mult);
+            }
         }
         if (EMIT) {
             for (int o = 32; o > 0; o >>= 1) c_min = min(c_min, (uint32_t)__shfl_xor((int)c_min, o));
@@ -240,33 +287,38 @@ __global__ __launch_bounds__(256) void k_lds_dedup(const uint32_t* __restrict__ 
         }
         __syncthreads();
         const uint32_t c_lo = EMIT ? c_lo_sh : 0;
-        for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
-            const uint64_t sign = pkey[i];
-            const uint32_t gi = pgi[i];
-            uint32_t h = LDS_TABLE;
-            bool found = true;
-            if (sign != EMPTY_KEY) {
-                h = lds_slot(sign);
-                int tries = 0;
-                for (; tries < LDS_TABLE && keys[h] != sign; tries++) h = (h + 1) & (LDS_TABLE - 1);
-                found = tries < LDS_TABLE;
-            }
-            const uint32_t f = found ? minpos[h] : gi;
-            first_of[gi] = f;
-            if (f == gi) {
-                cnt_at[gi] = found ? cnts[h] : 1u;
-                if (EMIT && found) {  // one lookup per occupied entry gets here
-                    const uint32_t local = group_bucket(sign, nb2) - c_lo;
-                    if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
+        for (uint32_t base = lo; base < hi; base += round) {
+            if (!one_round) load_round(base);
+#pragma unroll
+            for (int j = 0; j < DEDUP_ITEMS; j++) {
+                const uint64_t sign = sg[j];
+                const uint32_t gi = gp[j];
+                if (gi == 0xFFFFFFFFu) continue;
+                uint32_t h = LDS_TABLE;
+                bool found = true;
+                if (sign != EMPTY_KEY) {
+                    h = lds_slot(sign);
+                    int tries = 0;
+                    for (; tries < LDS_TABLE && keys[h] != sign; tries++) h = (h + 1) & (LDS_TABLE - 1);
+                    found = tries < LDS_TABLE;
+                }
+                const uint32_t f = found ? minpos[h] : gi;
+                first_of[gi] = f;
+                if (f == gi) {
+                    cnt_at[gi] = found ? cnts[h] : 1u;
+                    if (EMIT && found) {  // one lookup per occupied entry gets here
+                        const uint32_t local = group_bucket(sign, nb2) - c_lo;
+                        if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
+                    }
                 }
             }
         }
         if (EMIT) {
             __syncthreads();
-            for (int i = threadIdx.x; i < LDS_SPAN2; i += 256)
+            for (int i = threadIdx.x; i < LDS_SPAN2; i += DEDUP_THREADS)
                 if (hist2[i]) hist2[i] = atomicAdd(&cursor2[c_lo + i], hist2[i]);  // this bucket's slice
             __syncthreads();
-            for (int e = threadIdx.x; e <= LDS_TABLE; e += 256) {
+            for (int e = threadIdx.x; e <= LDS_TABLE; e += DEDUP_THREADS) {
                 const uint32_t cnt = cnts[e];
                 if (cnt == 0) continue;
                 GroupRec r;
@@ -390,7 +442,7 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
 //   y: bits 0-15 records of the bucket's earlier several-record groups, 16-23 place, 24-31 slot
 // and per bucket the number of groups with one record, with several, the
 // records of the latter, and the big groups.  At most GRP_SLOTS slots.
-__global__ __launch_bounds__(256) void k_group_count(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
+__global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
                                                      const uint32_t* __restrict__ cursor2,
                                                      const GroupRec* __restrict__ recs, uint32_t big_k,
                                                      uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
@@ -399,7 +451,7 @@ __global__ __launch_bounds__(256) void k_group_count(const uint32_t* __restrict_
     __shared__ uint32_t einfo[GRP_TABLE + 1], eoffs[GRP_TABLE + 1];
     __shared__ uint16_t rech[GRP_CAP];
     __shared__ uint32_t lb[GRP_SLOTS + 1];
-    __shared__ unsigned long long sh[4];
+    __shared__ unsigned long long sh[GRP_THREADS / 64];
     load_lbase(lb, lbase, N);
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
@@ -408,47 +460,63 @@ __global__ __launch_bounds__(256) void k_group_count(const uint32_t* __restrict_
             continue;
         }
         const size_t first = (size_t)c * GRP_CAP;
-        for (int i = threadIdx.x; i <= GRP_TABLE; i += 256) {
+        for (int i = threadIdx.x; i <= GRP_TABLE; i += GRP_THREADS) {
             keys[i] = EMPTY_KEY;
             mlo[i] = 0;
             mhi[i] = 0;
         }
         __syncthreads();
-        for (uint32_t i = threadIdx.x; i < n; i += 256) {
-            const GroupRec r = recs[first + i];
+        // all records of the bucket sit in registers (GRP_CAP = GRP_THREADS x GRP_RECS), loaded together
+        uint64_t sg[GRP_RECS];
+        uint32_t sl[GRP_RECS];  // slot of the record, 0xFFFFFFFF = no record
+#pragma unroll
+        for (int j = 0; j < GRP_RECS; j++) {
+            const uint32_t i = j * GRP_THREADS + threadIdx.x;
+            sg[j] = 0;
+            sl[j] = 0xFFFFFFFFu;
+            if (i < n) {
+                const GroupRec r = recs[first + i];
+                sg[j] = r.sign;
+                sl[j] = r.gi;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < GRP_RECS; j++) {
+            if (sl[j] == 0xFFFFFFFFu) continue;
+            const uint64_t sign = sg[j];
             uint32_t h = GRP_TABLE;
-            if (r.sign != EMPTY_KEY) {
-                h = (uint32_t)(mix64(r.sign) >> 9) & (GRP_TABLE - 1);
+            if (sign != EMPTY_KEY) {
+                h = (uint32_t)(mix64(sign) >> 9) & (GRP_TABLE - 1);
                 for (;;) {  // n <= GRP_CAP < GRP_TABLE: a free entry exists
                     unsigned long long old = keys[h];
-                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, r.sign);
-                    if (old == EMPTY_KEY || old == r.sign) break;
+                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
                     h = (h + 1) & (GRP_TABLE - 1);
                 }
             }
-            const uint32_t sl = (uint32_t)find_slot(lb, N, r.gi);
-            atomicOr(sl < 64 ? &mlo[h] : &mhi[h], 1ull << (sl & 63));
-            rech[i] = (uint16_t)h;
+            sl[j] = (uint32_t)find_slot(lb, N, sl[j]);
+            atomicOr(sl[j] < 64 ? &mlo[h] : &mhi[h], 1ull << (sl[j] & 63));
+            rech[j * GRP_THREADS + threadIdx.x] = (uint16_t)h;
         }
         __syncthreads();
         uint32_t ks[GRP_ITEMS];
         unsigned long long v = 0;  // 16-bit fields: groups of one record, of several, records of those, big groups
         for (int j = 0; j < GRP_ITEMS; j++) {
-            const uint32_t e = j * 256 + threadIdx.x;
+            const uint32_t e = j * GRP_THREADS + threadIdx.x;
             const uint32_t k = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
             ks[j] = k;
             if (k == 1) v += 1ull;
             if (k > 1) v += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
         }
         unsigned long long total;
-        unsigned long long ex = block_excl_scan_256<unsigned long long>(v, sh, &total);
+        unsigned long long ex = block_excl_scan<unsigned long long, GRP_THREADS / 64>(v, sh, &total);
         if (threadIdx.x == 0)
             bcounts[c] = make_uint4((uint32_t)(total & 0xFFFF), (uint32_t)((total >> 16) & 0xFFFF),
                                     (uint32_t)((total >> 32) & 0xFFFF), (uint32_t)(total >> 48));
         for (int j = 0; j < GRP_ITEMS; j++) {
             const uint32_t k = ks[j];
             if (k == 0) continue;
-            const uint32_t e = j * 256 + threadIdx.x;
+            const uint32_t e = j * GRP_THREADS + threadIdx.x;
             if (k == 1) {
                 einfo[e] = (uint32_t)(ex & 0xFFFF) | (1u << 24);
                 eoffs[e] = 0;
@@ -460,15 +528,18 @@ __global__ __launch_bounds__(256) void k_group_count(const uint32_t* __restrict_
             }
         }
         __syncthreads();
-        for (uint32_t i = threadIdx.x; i < n; i += 256) {
+#pragma unroll
+        for (int j = 0; j < GRP_RECS; j++) {
+            const uint32_t s1 = sl[j];
+            if (s1 == 0xFFFFFFFFu) continue;
+            const uint32_t i = j * GRP_THREADS + threadIdx.x;
             const uint32_t h = rech[i];
-            const uint32_t sl = (uint32_t)find_slot(lb, N, recs[first + i].gi);
             uint32_t place;
-            if (sl < 64)
-                place = (uint32_t)__popcll(mlo[h] & ((1ull << sl) - 1ull));
+            if (s1 < 64)
+                place = (uint32_t)__popcll(mlo[h] & ((1ull << s1) - 1ull));
             else
-                place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (sl - 64)) - 1ull));
-            aux[first + i] = make_uint2(einfo[h], eoffs[h] | (place << 16) | (sl << 24));
+                place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (s1 - 64)) - 1ull));
+            aux[first + i] = make_uint2(einfo[h], eoffs[h] | (place << 16) | (s1 << 24));
         }
         __syncthreads();
     }
@@ -534,9 +605,25 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
         const uint4 bb = bbase[c];
-        for (uint32_t i = threadIdx.x; i < n; i += 256) {
-            const GroupRec r = recs[first + i];
-            const uint2 a = aux[first + i];
+        GroupRec rs[EMIT_RECS];
+        uint2 as[EMIT_RECS];
+        uint32_t us[EMIT_RECS];
+#pragma unroll
+        for (int j = 0; j < EMIT_RECS; j++) {
+            const uint32_t i = j * 256 + threadIdx.x;
+            if (i < n) {
+                rs[j] = recs[first + i];
+                as[j] = aux[first + i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < EMIT_RECS; j++)
+            if (j * 256 + threadIdx.x < n) us[j] = rank_at[rs[j].gi];
+#pragma unroll
+        for (int j = 0; j < EMIT_RECS; j++) {
+            if (j * 256 + threadIdx.x >= n) continue;
+            const GroupRec r = rs[j];
+            const uint2 a = as[j];
             const uint32_t k = a.x >> 24, idx = a.x & 0xFFFu, bigidx = (a.x >> 12) & 0xFFFu;
             const uint32_t place = (a.y >> 16) & 0xFFu, sl = a.y >> 24;
             uint32_t g, off;
@@ -549,7 +636,7 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
             }
             const uint32_t at = off + place;
             Member m;
-            m.u = rank_at[r.gi];
+            m.u = us[j];
             m.slot = sl;
             m.show = (int32_t)r.cnt;  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             m.click = 0;

@@ -447,8 +447,9 @@ __device__ __forceinline__ uint32_t block_sum_256(uint32_t v, uint32_t* sh /*4*/
 }
 
 // exclusive prefix of v over the 256 threads of the block; *total = block sum
-template <typename T>
-__device__ __forceinline__ T block_excl_scan_256(T v, T* sh /*4*/, T* total) {
+// Exclusive scan over a workgroup of WAVES wavefronts (sh: WAVES entries of LDS).
+template <typename T, int WAVES>
+__device__ __forceinline__ T block_excl_scan(T v, T* sh, T* total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     T inc = v;
     for (int o = 1; o < 64; o <<= 1) {
@@ -457,11 +458,20 @@ __device__ __forceinline__ T block_excl_scan_256(T v, T* sh /*4*/, T* total) {
     }
     if (lane == 63) sh[wave] = inc;
     __syncthreads();
-    T base = 0;
-    for (int wv = 0; wv < wave; wv++) base += sh[wv];
-    if (total) *total = sh[0] + sh[1] + sh[2] + sh[3];
+    T base = 0, all = 0;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; wv++) {
+        if (wv < wave) base += sh[wv];
+        all += sh[wv];
+    }
+    if (total) *total = all;
     __syncthreads();
     return base + inc - v;
+}
+
+template <typename T>
+__device__ __forceinline__ T block_excl_scan_256(T v, T* sh /*4*/, T* total) {
+    return block_excl_scan<T, 4>(v, sh, total);
 }
 
 // Step 2: a lookup is a first occurrence iff its position equals its entry's

@@ -50,6 +50,8 @@ struct SparseTable {
     size_t hstage_bytes = 0;
     hipEvent_t stage_ev = nullptr;  // staging buffer free again
     hipEvent_t verify_ev = nullptr; // a push's comparison of the signs has been published
+    hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
+    hipEvent_t fork_ev = nullptr, join_ev = nullptr;
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
     bool pull_pending = false;
@@ -146,6 +148,9 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipHostMalloc((void**)&t->hstage, t->hstage_bytes, hipHostMallocDefault));
     TN_HIP(hipEventCreateWithFlags(&t->stage_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->verify_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->fork_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->join_ev, hipEventDisableTiming));
+    TN_HIP(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));  // default priority
     return TN_OK;
 }
 
@@ -555,10 +560,10 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
         TN_LAUNCH(k_lds_scatter, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcursor, w.pkey, w.pgi);
         if (lds_groups)
-            TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart,
+            TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
                       w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         else
-            TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(256), st, w.bstart,
+            TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
                       w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
@@ -585,7 +590,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
-        TN_LAUNCH(k_group_count, dim3(bblocks), dim3(256), st, p.lbase, N, w.nb2, w.cursor2, w.recs, big_threshold(s),
+        TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), st, p.lbase, N, w.nb2, w.cursor2, w.recs, big_threshold(s),
                   w.aux, w.bcounts);
         TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), st, w.bcounts, w.bbase, w.nb2, ds);
         TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.rank_at, L,
@@ -602,11 +607,22 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
                   (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
 }
 
+// The three kernels touch disjoint rows.  k_apply_big is latency-bound (few wavefronts, long
+// dependent chains) while the other two saturate the memory system, so it runs beside them on
+// the table's side stream, forked from and joined back into the caller's stream by events.
 template <int KIND>
-void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds, const Plan& p,
-                       int64_t n_upper, hipStream_t st) {
+int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
+                      const Plan& p, int64_t n_upper, hipStream_t st) {
     const uint32_t big_k = big_threshold(s);
     const uint32_t ids_cap = (uint32_t)n_upper;
+    const bool with_big = big_k != 0xFFFFFFFFu;
+    if (with_big) {
+        TN_HIP(hipEventRecord(t->fork_ev, st));
+        TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64), t->side, s, o,
+                  src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list);
+        TN_HIP(hipEventRecord(t->join_ev, t->side));
+    }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
         TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
@@ -626,14 +642,13 @@ void launch_apply_kind(int lpg, const Store& s, const OptDev& o, const PushSrc& 
                       p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);
     }
 #undef TN_LAUNCH_VEC
-    if (big_k != 0xFFFFFFFFu)
-        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64), st, s, o,
-                  src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list);
+    if (with_big) TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
+    return TN_OK;
 }
 
 // Applies the grouped records; n_upper bounds the number of records.
-void launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
-                  hipStream_t st) {
+int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
+                 hipStream_t st) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     int lpg = 0;
@@ -642,9 +657,9 @@ void launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* 
         if (q >= 1 && q <= 32 && (q & (q - 1)) == 0) lpg = q;
     }
     switch (o.kind) {
-        case OPT_ADAGRAD: launch_apply_kind<OPT_ADAGRAD>(lpg, s, o, src, ds, p, n_upper, st); break;
-        case OPT_ADAM: launch_apply_kind<OPT_ADAM>(lpg, s, o, src, ds, p, n_upper, st); break;
-        default: launch_apply_kind<OPT_FTRL>(lpg, s, o, src, ds, p, n_upper, st); break;
+        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st);
+        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st);
+        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st);
     }
 }
 
@@ -862,7 +877,7 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
     launch_grouping(p, w, src, n, n, big_threshold(t->store), nullptr, ds, st);
     TN_LAUNCH((k_probe<false>), dim3(launch_grid(n, 256, GRID_CAP * 2)), dim3(256), st, t->store, p.grp_sign,
               (int64_t)0, ds, (uint32_t)n, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
-    launch_apply(t, p, src, ds, n, aligned16(grads) && dim % 4 == 0, st);
+    TN_TRY(launch_apply(t, p, src, ds, n, aligned16(grads) && dim % 4 == 0, st));
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
     t->push_pending = true;
@@ -1110,7 +1125,7 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
         TN_TRY(launch_counts(false));
     }
-    launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st);
+    TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
     TN_HIP(hipGetLastError());
     TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush));
     t->push_pending = true;
