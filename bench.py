@@ -27,6 +27,11 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
+# HBM bytes per launch (read + written) of the cfg3 kernels from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# scaled by what the same counters read for the dense Adam stream of known size; see profiles/.
+MEASURED_TRAFFIC = {}
+
+
 def state_bytes(opt, dim):
     """Optimizer state bytes read+written per applied row (beyond w and the gradient)."""
     return 28 if opt == "AdaGrad" else 16 * dim + 8
@@ -39,32 +44,66 @@ def step_algorithmic_bytes(opt, dim, L, U):
     return 32 * L + U * (8 + 8 * dim + 4 * dim + 8 + 8 * dim + state_bytes(opt, dim))
 
 
-def kernel_algorithmic_bytes(name, opt, dim, L, U, G):
-    """Algorithmic bytes of one launch of each kernel of the step (L lookups, U
-    per-slot distinct signs, G distinct signs of the whole push)."""
+# Launched on the table's side stream, concurrently with the other apply kernels: its
+# duration is not part of the step's critical path.
+SIDE_STREAM_KERNELS = ("k_apply_big",)
+BIG_GROUP = 16  # records from which a sign is applied by k_apply_big (sparse_table.hip)
+
+
+def kernel_algorithmic_bytes(name, opt, dim, shape):
+    """Algorithmic bytes of one launch of each kernel of the step: what the kernel has to
+    read and write once, from the sizes of the batch.  shape: L lookups, U per-slot distinct
+    signs (records), G distinct signs of the whole batch (groups); G1 groups with one record,
+    Rm / Gm records / groups with 2..15 records, Rb / Gb records / groups with 16 or more."""
+    L, U, G = shape["L"], shape["U"], shape["G"]
     row = 4 * dim
+    st = state_bytes(opt, dim)
+
+    def apply_bytes(records, groups):  # gradient + member entry per record; row and state read and written per group
+        return records * (row + 16) + groups * (2 * row + st)
+
     table = {
-        "k_fill_ff": 0,
-        "k_remap_insert": 8 * L,                      # reads every sign once
-        "k_flag_count": 0,
-        "k_scan_tiles": 0,
-        "k_assign_rank": 8 * U,                       # writes the distinct sign lists
-        "k_write_mapped": 8 * L,                      # writes every mapped id
-        "k_count_show": 8 * L,                        # reads every label
-        "k_probe<true>": 8 * U,                       # one stored-key compare per row
-        "k_probe<false>": 8 * G,
-        "k_init_rows": 0,
-        "k_finish_insert": 0,
-        "k_gather_vars<4>": U * 2 * row,              # row read + variable row write
-        "k_gather_vars<1>": U * 2 * row,
-        "k_fill_groups": 0,
-        "k_group_insert": 8 * U,
-        "k_group_compact": 0,
-        "k_group_fill": 0,
+        # remap through LDS
+        "k_lds_hist": 16 * L,                  # reads every sign, keeps a copy for the push
+        "k_lds_scatter": 20 * L,               # reads every sign, writes {sign, position} by bucket
+        "k_lds_dedup": 16 * L + 16 * U,        # reads {sign, position}, writes first positions and the distinct records
+        "k_lds_flags": 4 * L,
+        "k_lds_assign": 4 * U,
+        "k_lds_mapped": 12 * L,                # first position in, mapped id out
+        "k_group_count": 24 * U,               # distinct records in, per-record placement out
+        "k_group_emit": 48 * U + 16 * G,       # records + placement in; member lists, per-record index, groups out
+        # global-table fallback
+        "k_remap_insert": 8 * L, "k_assign_rank": 8 * U, "k_write_mapped": 8 * L, "k_count_show": 8 * L,
+        "k_mask_insert": 16 * U, "k_mask_compact": 16 * G, "k_mask_fill": 32 * U,
+        "k_group_insert": 16 * U,
+        # table
+        "k_probe": 8 * G + 4 * G,              # one stored-key compare per distinct sign, row number out
+        "k_gather_vars": U * (2 * row + 4),    # row read + variable row write
+        # push
+        "k_verify_values": 16 * L,             # the op's signs against the pull's copy
+        "k_count_click": 8 * L,                # labels
+        "k_reset_counts": 8 * U,
+        "k_apply_single": apply_bytes(shape["G1"], shape["G1"]),
+        "k_apply_vec": apply_bytes(shape["Rm"], shape["Gm"]),
+        "k_apply_big": apply_bytes(shape["Rb"], shape["Gb"]),
+        "k_apply_scalar": apply_bytes(U, G),
     }
-    if name.startswith("k_apply"):
-        return U * row + G * (2 * row + state_bytes(opt, dim))
-    return table.get(name, 0)
+    return table.get(name.split("<")[0], 0)
+
+
+def batch_shape(values):
+    """Sizes of one batch (torch on the GPU, harness only): see kernel_algorithmic_bytes."""
+    import torch
+
+    per_slot = [torch.unique(v) for v in values]
+    _, k = torch.unique(torch.cat(per_slot), return_counts=True)
+    mid = (k > 1) & (k < BIG_GROUP)
+    big = k >= BIG_GROUP
+    return {
+        "L": sum(v.numel() for v in values), "U": sum(u.numel() for u in per_slot), "G": int(k.numel()),
+        "G1": int((k == 1).sum()), "Gm": int(mid.sum()), "Rm": int(k[mid].sum()),
+        "Gb": int(big.sum()), "Rb": int(k[big].sum()),
+    }
 
 
 def populate(tn, handle, resident, dim, chunk=1 << 23):
@@ -200,7 +239,8 @@ def main():
         tn.ops.sparse_table_pull(vars_, values, h)
         Us.append(sum(tn.ops.sparse_table_last_unique_counts(h, n_slots)))
         Ls.append(sum(v.numel() for v in values))
-    G0 = int(torch.unique(torch.cat(batches[0][0])).numel())
+    shapes = [batch_shape(b[0]) for b in batches]
+    G0 = shapes[0]["G"]
     torch.cuda.synchronize()
 
     # ---- timed region ------------------------------------------------------------
@@ -237,11 +277,14 @@ def main():
     lib.tn_profile_reset()
     per_step = {k: (c / psteps, ms / psteps) for k, (c, ms) in prof.items()}
     kernel_ms = sum(ms for _, ms in per_step.values())
-    dominant = max(per_step.items(), key=lambda kv: kv[1][1])
+    # the dominant kernel of the step's critical path
+    dominant = max((kv for kv in per_step.items() if not kv[0].startswith(SIDE_STREAM_KERNELS)),
+                   key=lambda kv: kv[1][1])
     dname, (dcount, dms) = dominant
     avg_launch_s = dms / dcount * 1e-3
     mean_L, mean_U = total_L / args.steps, total_U / args.steps
-    dbytes = kernel_algorithmic_bytes(dname, opt_name, dim, mean_L, mean_U, G0)
+    mean_shape = {k: sum(sh[k] for sh in shapes) / len(shapes) for k in shapes[0]}
+    dbytes = kernel_algorithmic_bytes(dname, opt_name, dim, mean_shape)
     achieved = dbytes / avg_launch_s
     for k, (c, ms) in sorted(per_step.items(), key=lambda kv: -kv[1][1]):
         log("  %-28s %5.1f launches/step %9.3f ms/step" % (k, c, ms))
@@ -279,11 +322,16 @@ def main():
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get(dname.split("<")[0]) if args.config == "cfg3" else None,
             "avg_launch_us": avg_launch_s * 1e6,
             "algorithmic_bytes_per_launch": dbytes,
         },
         "kernels_ms_per_step": {k: round(ms, 4) for k, (c, ms) in per_step.items()},
+        "kernels_frac_of_hbm_peak": {
+            k: round(kernel_algorithmic_bytes(k, opt_name, dim, mean_shape) / (ms / c * 1e-3) / HBM_PEAK, 4)
+            for k, (c, ms) in per_step.items() if kernel_algorithmic_bytes(k, opt_name, dim, mean_shape) > 0},
+        "side_stream_kernels": [k for k in per_step if k.startswith(SIDE_STREAM_KERNELS)],
+        "batch_shape": mean_shape,
     }
 
     # ---- dense Adam side measurement (cfg5's flat array) --------------------------

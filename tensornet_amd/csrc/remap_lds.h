@@ -43,10 +43,10 @@ namespace tn {
 constexpr int LDS_TILE = 4096;          // lookups per tile of the partition kernels
 constexpr int LDS_TILE_ITEMS = LDS_TILE / 256;
 constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
-constexpr int LDS_BUCKET_TARGET = 1536; // average lookups per bucket
-constexpr int LDS_MAX_SUB = 2048;       // buckets per slot at most
-constexpr int LDS_TABLE = 4096;         // entries of a bucket's LDS hash table
-constexpr int DEDUP_THREADS = 1024;     // a bucket's phases are short and separated by barriers: many wavefronts hide them
+constexpr int LDS_BUCKET_TARGET = 768;  // average lookups per bucket
+constexpr int LDS_MAX_SUB = 4096;       // buckets per slot at most
+constexpr int LDS_TABLE = 2048;         // entries of a bucket's LDS hash table
+constexpr int DEDUP_THREADS = 512;      // a bucket's phases are short and separated by barriers: many wavefronts hide them
 constexpr int DEDUP_ITEMS = 2;          // lookups a thread of k_lds_dedup holds in registers
 constexpr int LDS_SPAN2 = 512;          // second-level buckets whose counts one first-level bucket gathers in LDS
 constexpr int GRP_TARGET = 1024;        // records per second-level bucket if every lookup were distinct
