@@ -303,9 +303,9 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                     found = tries < LDS_TABLE;
                 }
                 const uint32_t f = found ? minpos[h] : gi;
-                first_of[gi] = f;
+                if (f != gi) first_of[gi] = f;  // k_lds_hist preset first_of[gi] = gi
                 if (f == gi) {
-                    cnt_at[gi] = found ? cnts[h] : 1u;
+                    if (!EMIT) cnt_at[gi] = found ? cnts[h] : 1u;  // with EMIT the record carries the count
                     if (EMIT && found) {  // one lookup per occupied entry gets here
                         const uint32_t local = group_bucket(sign, nb2) - c_lo;
                         if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
@@ -600,7 +600,7 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
                                                     uint32_t big_k, uint64_t* __restrict__ grp_sign,
                                                     uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
-                                                    uint32_t* __restrict__ pos_of_u, uint32_t* __restrict__ g_of_u) {
+                                                    uint2* __restrict__ where_u) {
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
@@ -641,8 +641,7 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
             m.show = (int32_t)r.cnt;  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             m.click = 0;
             list[at] = m;
-            pos_of_u[m.u] = at;
-            g_of_u[m.u] = g;
+            where_u[m.u] = make_uint2(at, g);
             if (place == 0) {
                 grp_sign[g] = r.sign;
                 grp_off[g] = off;
@@ -659,14 +658,14 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
 __global__ __launch_bounds__(256) void k_count_click(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                      const uint32_t* __restrict__ u_of_gi,
-                                                     const uint32_t* __restrict__ pos_of_u, Member* list) {
+                                                     const uint2* __restrict__ where_u, Member* list) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
         const int label = (int)descs[sl].labels[gi - lb[sl]];
-        if (label != 0) atomicAdd(&list[pos_of_u[u_of_gi[gi] & ~FIRST_BIT]].click, label);
+        if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
     }
 }
 

@@ -636,7 +636,7 @@ constexpr int COUNT_SLOTS = 4096;  // LDS table entries per tile (load factor <=
 __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__ descs,
                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                     const uint32_t* __restrict__ u_of_gi,
-                                                    const uint32_t* __restrict__ pos_of_u, Member* list,
+                                                    const uint2* __restrict__ where_u, Member* list,
                                                     int with_click) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t keys[COUNT_SLOTS];
@@ -676,7 +676,7 @@ __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__
         for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
             const uint32_t u = keys[i];
             if (u == 0xFFFFFFFFu) continue;
-            Member* m = &list[pos_of_u[u]];
+            Member* m = &list[where_u[u].x];
             if (cnts[i]) atomicAdd(&m->show, cnts[i]);
             if (clks[i]) atomicAdd(&m->click, clks[i]);
         }
@@ -833,7 +833,7 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
                                                     const uint32_t* __restrict__ arrival,
                                                     const uint32_t* __restrict__ uniq_slot,
                                                     const uint32_t* __restrict__ ushow, Member* __restrict__ list,
-                                                    uint32_t* __restrict__ g_of_u, uint32_t* __restrict__ pos_of_u) {
+                                                    uint2* __restrict__ where_u) {
     const int64_t n = n_dev ? (int64_t)*n_dev : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
@@ -851,8 +851,7 @@ __global__ __launch_bounds__(256) void k_group_rank(int64_t n_host, const uint32
         m.show = ushow ? (int32_t)ushow[u] : 1;
         m.click = 0;
         list[off + pos] = m;
-        g_of_u[u] = en.g;
-        pos_of_u[u] = off + pos;
+        where_u[u] = make_uint2(off + pos, en.g);
     }
 }
 
@@ -941,7 +940,7 @@ __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, cons
                                                    const uint32_t* __restrict__ gidx,
                                                    const uint32_t* __restrict__ uniq_slot,
                                                    const uint32_t* __restrict__ ushow, Member* __restrict__ list,
-                                                   uint32_t* __restrict__ g_of_u, uint32_t* __restrict__ pos_of_u) {
+                                                   uint2* __restrict__ where_u) {
     const uint32_t n = status->n_unique;
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t u = blockIdx.x * blockDim.x + threadIdx.x; u < n; u += stride) {
@@ -961,8 +960,7 @@ __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, cons
         m.show = ushow ? (int32_t)ushow[u] : 1;
         m.click = 0;
         list[go.y + pos] = m;
-        g_of_u[u] = go.x;
-        pos_of_u[u] = go.y + pos;
+        where_u[u] = make_uint2(go.y + pos, go.x);
     }
 }
 
@@ -970,7 +968,7 @@ __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, cons
 // every slot (PopulatePulledVariable_, sparse_table_ops.cc:244-265).
 template <int VEC>
 __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status, const uint32_t* __restrict__ grp_row,
-                                                     const uint32_t* __restrict__ g_of_u,
+                                                     const uint2* __restrict__ where_u,
                                                      const uint32_t* __restrict__ ubase, int N,
                                                      const SlotDesc* __restrict__ descs) {
     __shared__ uint32_t ub[MAX_SLOTS + 1];
@@ -981,7 +979,7 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
         const int64_t u = t / chunks;
         const int c = (int)(t - u * chunks);
-        const uint32_t row = grp_row[g_of_u[u]];
+        const uint32_t row = grp_row[where_u[u].y];
         const int sl = find_slot(ub, N, (uint32_t)u);  // the slot whose window of distinct indices holds u
         const int64_t r = (int64_t)u - (int64_t)ub[sl];
         const SlotDesc& d = descs[sl];

@@ -315,8 +315,7 @@ struct Plan {
     uint32_t* grp_off;
     uint32_t* grp_cnt;
     Member* list;          // members of every group, ascending (with their show / click counts)
-    uint32_t* pos_of_u;    // record -> its place in `list`
-    uint32_t* g_of_u;      // record -> its group
+    uint2* where_u;        // record -> {its place in `list`, its group}
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     uint32_t* newlist;     // groups whose row was inserted by the pull
 };
@@ -366,8 +365,7 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_off = c.take<uint32_t>(n);
     p.grp_cnt = c.take<uint32_t>(n);
     p.list = c.take<Member>(n);
-    p.pos_of_u = c.take<uint32_t>(n);
-    p.g_of_u = c.take<uint32_t>(n);
+    p.where_u = c.take<uint2>(n);
     p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
     p.newlist = c.take<uint32_t>(n);
 }
@@ -521,7 +519,7 @@ void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_
               dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k, (uint32_t)n_upper);
     TN_LAUNCH(k_group_fill, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.ord, w.arrival);
     TN_LAUNCH(k_group_rank, dim3(gblocks), dim3(256), st, n_host, n_dev, gt, p.grp_off, w.gidx, w.arrival,
-              src.uniq_slot, ushow, p.list, p.g_of_u, p.pos_of_u);
+              src.uniq_slot, ushow, p.list, p.where_u);
 }
 
 constexpr int MASK_SLOTS = 128;
@@ -537,8 +535,7 @@ void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint
     TN_LAUNCH(k_mask_insert, dim3(gblocks), dim3(256), st, p.uniq_sign, p.uniq_slot, ds, gt, w.gidx);
     TN_LAUNCH(k_mask_compact, dim3(launch_grid((int64_t)group_cap(n_upper) / COMPACT_ITEMS + 1, 256, GRID_CAP)),
               dim3(256), st, ds, gt, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, big_k, (uint32_t)n_upper);
-    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, ushow, p.list, p.g_of_u,
-              p.pos_of_u);
+    TN_LAUNCH(k_mask_fill, dim3(gblocks), dim3(256), st, ds, gt, w.gidx, p.uniq_slot, ushow, p.list, p.where_u);
 }
 
 // Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids,
@@ -594,7 +591,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
                   w.aux, w.bcounts);
         TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), st, w.bcounts, w.bbase, w.nb2, ds);
         TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.rank_at, L,
-                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.pos_of_u, p.g_of_u);
+                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u);
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
     else
@@ -1009,10 +1006,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
-                      ds, p.grp_row, p.g_of_u, p.ubase, N, p.descs);
+                      ds, p.grp_row, p.where_u, p.ubase, N, p.descs);
         else
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
-                      p.grp_row, p.g_of_u, p.ubase, N, p.descs);
+                      p.grp_row, p.where_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
         TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
                   reinterpret_cast<uint32_t*>(t->hpull));
@@ -1089,12 +1086,12 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
             if (with_click) {
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
                 TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
-                          p.pos_of_u, p.list);
+                          p.where_u, p.list);
             }
         } else {
             TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
             TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)),
-                      dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.pos_of_u, p.list,
+                      dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.where_u, p.list,
                       with_click ? 1 : 0);
         }
         return TN_OK;
