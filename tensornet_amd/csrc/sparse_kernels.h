@@ -5,6 +5,9 @@
 //     keys[cap + 1]              uint64 sign, EMPTY_KEY where free
 //     w   [cap + 1][wstride]     embedding weights (+2 cvm columns)
 //     st  [cap + 1][sstride]     optimizer state
+// When a weight row and its state fit one 128-byte line together, the two are
+// interleaved (st = w + wlen, both strides 32 floats): an update then touches
+// one line of the table instead of two.
 // Slot `cap` is reserved for the one sign whose value equals EMPTY_KEY.
 // A pull touches keys and w only (one 64-byte granule each for dim 16); the
 // optimizer state is touched by push alone.
@@ -35,7 +38,9 @@ struct Store {
     float* st;
     uint32_t* special;            // 1 when the sign EMPTY_KEY itself is resident
     unsigned long long* count;    // resident keys
-    int D, wdim, wstride, sstride;
+    int D, wdim;
+    int wlen, slen;        // floats of a weight / state row (incl. padding to a multiple of 4)
+    int wstride, sstride;  // distance between consecutive rows, in floats (>= wlen / slen)
 };
 
 // One slot (input tensor pair) of a pull / push op.  64 bytes.
@@ -245,7 +250,7 @@ __device__ __forceinline__ void init_state(const Store& s, const OptDev& o, floa
         st[2] = 0.f;
         st[3] = 0.f;  // no_show_days = 0 (int bits)
     } else {
-        for (int i = 0; i < s.sstride; i++) st[i] = 0.f;  // m=v=0 / z=n=0, show, delta_show
+        for (int i = 0; i < s.slen; i++) st[i] = 0.f;  // m=v=0 / z=n=0, show, delta_show
     }
 }
 
@@ -273,7 +278,7 @@ __global__ __launch_bounds__(256) void k_init_rows(Store s, OptDev o, uint64_t s
                 if (c + 1 < s.D) w[c + 1] = (z.y * stddev) * o.initial_scale;
             }
         }
-        for (int c = s.D; c < s.wstride; c++) w[c] = 0.f;  // cvm columns / padding
+        for (int c = s.D; c < s.wlen; c++) w[c] = 0.f;  // cvm columns / padding
         init_state(s, o, s.st + row * s.sstride);
     }
 }
@@ -309,12 +314,12 @@ __global__ __launch_bounds__(256) void k_load_rows(Store s, OptDev o, const uint
         if (row == NO_ROW) continue;
         float* dw = s.w + (uint64_t)row * s.wstride;
         for (int c = 0; c < s.wdim; c++) dw[c] = w[i * s.wdim + c];
-        for (int c = s.wdim; c < s.wstride; c++) dw[c] = 0.f;
+        for (int c = s.wdim; c < s.wlen; c++) dw[c] = 0.f;
         float* ds = s.st + (uint64_t)row * s.sstride;
         if (state) {
             const int sf = (o.kind == OPT_ADAGRAD) ? 4 : 2 * s.D + 2;
             for (int c = 0; c < sf; c++) ds[c] = state[i * sf + c];
-            for (int c = sf; c < s.sstride; c++) ds[c] = 0.f;
+            for (int c = sf; c < s.slen; c++) ds[c] = 0.f;
         } else {
             init_state(s, o, ds);
         }
@@ -367,10 +372,10 @@ __global__ __launch_bounds__(256) void k_rehash(Store from, Store to, DevStatus*
         }
         const float* sw = from.w + i * from.wstride;
         float* dw = to.w + dst * to.wstride;
-        for (int c = 0; c < from.wstride; c++) dw[c] = sw[c];
+        for (int c = 0; c < from.wlen; c++) dw[c] = sw[c];
         const float* ss = from.st + i * from.sstride;
         float* ds = to.st + dst * to.sstride;
-        for (int c = 0; c < from.sstride; c++) ds[c] = ss[c];
+        for (int c = 0; c < from.slen; c++) ds[c] = ss[c];
     }
 }
 
