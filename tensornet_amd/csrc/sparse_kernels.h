@@ -128,31 +128,47 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
     }
 }
 
-// start of a push that reuses the plan: keep the counts, clear the flags
-__global__ void k_begin_push(DevStatus* status) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        status->err = 0;
-        status->mismatch = 0;
-    }
-}
-
 // Small host<->device transfers done by kernels on the stream (pinned host
-// memory is device-accessible): cheaper than a copy command each.
+// memory is device-accessible): cheaper than a copy command each.  The same
+// launch prepares the call's status block (STATUS_NEW_PLAN: everything cleared;
+// STATUS_REUSE_PLAN: a push on the last pull's plan keeps the counts and clears
+// the flags) and clears `zero[0 .. n_zero)`.
+enum { STATUS_KEEP = 0, STATUS_NEW_PLAN = 1, STATUS_REUSE_PLAN = 2 };
+
 __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ host_src, uint32_t* __restrict__ dst_a,
-                                                  uint32_t words_a, uint32_t* __restrict__ dst_b, uint32_t words_b) {
+                                                  uint32_t words_a, uint32_t* __restrict__ dst_b, uint32_t words_b,
+                                                  DevStatus* status, int status_mode, uint32_t* __restrict__ zero,
+                                                  uint32_t n_zero) {
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < words_a + words_b; i += stride) {
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint32_t i = tid; i < words_a + words_b; i += stride) {
         if (i < words_a)
             dst_a[i] = host_src[i];
         else
             dst_b[i - words_a] = host_src[i];
     }
+    for (uint32_t i = tid; i < n_zero; i += stride) zero[i] = 0;
+    if (tid == 0 && status_mode != STATUS_KEEP) {
+        status->err = 0;
+        status->mismatch = 0;
+        if (status_mode == STATUS_NEW_PLAN) {
+            status->n_unique = 0;
+            status->n_single = 0;
+            status->n_multi = 0;
+            status->n_new = 0;
+            status->gcap = 0;
+            status->n_members = 0;
+            status->n_big = 0;
+        }
+    }
 }
 
-// host_dst: a DevStatus followed by n_ubase words
+// host_dst: a DevStatus followed by n_ubase words.  With count != nullptr the rows the call
+// inserted are added to the table's number of resident keys.
 __global__ __launch_bounds__(256) void k_publish(const DevStatus* __restrict__ status,
                                                  const uint32_t* __restrict__ ubase, uint32_t n_ubase,
-                                                 uint32_t* __restrict__ host_dst) {
+                                                 uint32_t* __restrict__ host_dst, unsigned long long* count) {
+    if (count && threadIdx.x == 0) *count += status->n_new;
     const uint32_t sw = sizeof(DevStatus) / 4;
     const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
     for (uint32_t i = threadIdx.x; i < sw + n_ubase; i += blockDim.x)
@@ -167,19 +183,24 @@ __global__ void k_finish_insert(Store s, const DevStatus* status) {
 // One thread per sign.  rows[i] = slot of signs[i] (NO_ROW if absent / full).
 // With INSERT an absent sign claims the first free slot of its probe sequence
 // (SparseKernelBlock::GetWeight's insert, optimizer_kernel.h:299-308) and the
-// index i of every claim is appended to newlist.
+// index i of every claim is appended to newlist (or, without a newlist, the
+// claiming thread initialises the row on the spot).
 // Groups with one record are numbered upwards from 0, groups with several
 // downwards from ids_cap - 1: the i-th group in enumeration order.
 __device__ __forceinline__ uint32_t group_id(uint32_t i, uint32_t n_single, uint32_t n_multi, uint32_t ids_cap) {
     return i < n_single ? i : ids_cap - n_multi + (i - n_single);
 }
 
+constexpr int PROBE_WIDTH = 4;
+
+__device__ __forceinline__ void init_row(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row);
+
 // With groups_of != nullptr the signs are those of its groups (ids_cap = size of the id space).
 template <bool INSERT>
 __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restrict__ signs, int64_t n_host,
                                                const DevStatus* groups_of, uint32_t ids_cap,
                                                uint32_t* __restrict__ rows, uint32_t* __restrict__ newlist,
-                                               DevStatus* status, uint32_t miss_err) {
+                                               DevStatus* status, uint32_t miss_err, OptDev o, uint64_t seed) {
     const uint32_t n_single = groups_of ? groups_of->n_single : 0, n_multi = groups_of ? groups_of->n_multi : 0;
     const int64_t n = groups_of ? (int64_t)n_single + n_multi : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -196,34 +217,50 @@ __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restri
                 row = (uint32_t)s.cap;
             }
         } else {
+            // PROBE_WIDTH consecutive slots per round trip: their loads are issued together, so a
+            // probe sequence of a few slots costs one memory latency instead of one per slot.
             uint64_t idx = slot_of(sign, s.cap);
-            for (uint64_t p = 0; p < s.cap; ++p) {
-                uint64_t k = ld_relaxed(&s.keys[idx]);
-                if (k == sign) {
-                    row = (uint32_t)idx;
-                    break;
+            bool done = false;
+            for (uint64_t p = 0; p < s.cap && !done; p += PROBE_WIDTH) {
+                uint64_t at[PROBE_WIDTH], k[PROBE_WIDTH];
+#pragma unroll
+                for (int j = 0; j < PROBE_WIDTH; j++) {
+                    at[j] = idx + j;
+                    if (at[j] >= s.cap) at[j] -= s.cap;
+                    k[j] = s.keys[at[j]];  // plain load: a key never changes once set, and a stale free slot is settled by the compare-and-swap
                 }
-                if (k == EMPTY_KEY) {
-                    if (!INSERT) break;
-                    uint64_t old = atomicCAS(ull(&s.keys[idx]), EMPTY_KEY, sign);
-                    if (old == EMPTY_KEY) {
-                        row = (uint32_t)idx;
-                        is_new = true;
-                        break;
-                    }
-                    if (old == sign) {
-                        row = (uint32_t)idx;
-                        break;
+#pragma unroll
+                for (int j = 0; j < PROBE_WIDTH; j++) {
+                    if (done) break;
+                    if (k[j] == sign) {
+                        row = (uint32_t)at[j];
+                        done = true;
+                    } else if (k[j] == EMPTY_KEY) {  // possibly stale: the compare-and-swap decides
+                        if (!INSERT) {
+                            done = true;
+                        } else {
+                            uint64_t old = atomicCAS(ull(&s.keys[at[j]]), EMPTY_KEY, sign);
+                            if (old == EMPTY_KEY || old == sign) {
+                                row = (uint32_t)at[j];
+                                is_new = old == EMPTY_KEY;
+                                done = true;
+                            }
+                        }
                     }
                 }
-                idx = (idx + 1 == s.cap) ? 0 : idx + 1;
+                idx = at[PROBE_WIDTH - 1] + 1 == s.cap ? 0 : at[PROBE_WIDTH - 1] + 1;
             }
         }
         rows[i] = row;
         if (row == NO_ROW && miss_err) atomicOr(&status->err, miss_err);
         if (INSERT) {
             uint32_t j = wave_alloc(is_new, &status->n_new);
-            if (is_new) newlist[j] = (uint32_t)i;
+            if (is_new) {
+                if (newlist)
+                    newlist[j] = (uint32_t)i;  // initialised by k_init_rows
+                else
+                    init_row(s, o, seed, sign, row);  // the thread that claimed the row fills it
+            }
         }
     }
 }
@@ -258,28 +295,30 @@ __device__ __forceinline__ void init_state(const Store& s, const OptDev& o, floa
 // sparse_zero_init; fresh optimizer state (ada_grad_kernel.cc:78-103,
 // adam_kernel.cc:89-110, ftrl_kernel.cc:34-55).  The draw is a pure function
 // of (seed, sign, element).  One thread per new row.
+__device__ __forceinline__ void init_row(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row) {
+    const float stddev = (float)(1.0 / sqrt((double)s.D));
+    float* w = s.w + row * s.wstride;
+    if (o.zero_init) {
+        for (int c = 0; c < s.D; c++) w[c] = 0.f;
+    } else {
+        for (int c = 0; c < s.D; c += 2) {
+            float2 z = normal_pair(rnd64(seed, sign, (uint64_t)(c >> 1)));
+            w[c] = (z.x * stddev) * o.initial_scale;
+            if (c + 1 < s.D) w[c + 1] = (z.y * stddev) * o.initial_scale;
+        }
+    }
+    for (int c = s.D; c < s.wlen; c++) w[c] = 0.f;  // cvm columns / padding
+    init_state(s, o, s.st + row * s.sstride);
+}
+
 __global__ __launch_bounds__(256) void k_init_rows(Store s, OptDev o, uint64_t seed, const uint64_t* __restrict__ signs,
                                                    const uint32_t* __restrict__ rows,
                                                    const uint32_t* __restrict__ newlist, const DevStatus* status) {
     const uint32_t n_new = status->n_new;
     const uint32_t stride = gridDim.x * blockDim.x;
-    const float stddev = (float)(1.0 / sqrt((double)s.D));
     for (uint32_t j = blockIdx.x * blockDim.x + threadIdx.x; j < n_new; j += stride) {
         const uint32_t i = newlist[j];
-        const uint64_t sign = signs[i];
-        const uint64_t row = rows[i];
-        float* w = s.w + row * s.wstride;
-        if (o.zero_init) {
-            for (int c = 0; c < s.D; c++) w[c] = 0.f;
-        } else {
-            for (int c = 0; c < s.D; c += 2) {
-                float2 z = normal_pair(rnd64(seed, sign, (uint64_t)(c >> 1)));
-                w[c] = (z.x * stddev) * o.initial_scale;
-                if (c + 1 < s.D) w[c + 1] = (z.y * stddev) * o.initial_scale;
-            }
-        }
-        for (int c = s.D; c < s.wlen; c++) w[c] = 0.f;  // cvm columns / padding
-        init_state(s, o, s.st + row * s.sstride);
+        init_row(s, o, seed, signs[i], rows[i]);
     }
 }
 

@@ -499,8 +499,11 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
     return TN_OK;
 }
 
+// Slot descriptors to the device; the same launch prepares the plan's status block
+// (status_mode) and clears `zero[0 .. n_zero)`.
 int upload_slots(SparseTable* t, const Plan& p, const std::vector<SlotDesc>& descs,
-                 const std::vector<uint32_t>& lbase, hipStream_t st) {
+                 const std::vector<uint32_t>& lbase, hipStream_t st, int status_mode, uint32_t* zero = nullptr,
+                 uint32_t n_zero = 0) {
     if (t->stage_pending) {
         TN_HIP(hipEventSynchronize(t->stage_ev));
         t->stage_pending = false;
@@ -509,9 +512,9 @@ int upload_slots(SparseTable* t, const Plan& p, const std::vector<SlotDesc>& des
     const size_t lb = lbase.size() * sizeof(uint32_t);
     std::memcpy(t->hstage, descs.data(), db);
     std::memcpy(t->hstage + db, lbase.data(), lb);
-    TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)(db + lb) / 4, 256, 64)), dim3(256), st,
+    TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)std::max<size_t>((db + lb) / 4, n_zero), 256, 64)), dim3(256), st,
               reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(p.descs), (uint32_t)(db / 4),
-              p.lbase, (uint32_t)(lb / 4));
+              p.lbase, (uint32_t)(lb / 4), t->dplan, status_mode, zero, n_zero);
     TN_HIP(hipEventRecord(t->stage_ev, st));
     t->stage_pending = true;
     return TN_OK;
@@ -563,18 +566,17 @@ void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint
 
 // Analyses the batch staged in p.descs: per-slot distinct signs and mapped ids,
 // groups of equal signs, and the table row of every group (inserting absent
-// signs for a pull).  use_lds picks the remap through LDS (pull only).
+// signs for a pull).  use_lds picks the remap through LDS (pull only).  The
+// upload of the descriptors has cleared the status block and, for the LDS path,
+// the bucket counters.
 void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull, bool use_lds,
                        hipStream_t st) {
     DevStatus* ds = t->dplan;
     const Store& s = t->store;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
-    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, 0u, 0u);
     const bool lds_groups = use_lds && N <= GRP_SLOTS;
     if (use_lds) {
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
-        TN_LAUNCH(k_zero_u32, dim3(launch_grid(w.nbuckets + 1 + w.nb2, 256, 64)), dim3(256), st, w.bcount,
-                  w.nbuckets + 1 + w.nb2);
         TN_LAUNCH(k_lds_hist, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy, w.first_of,
                   ds);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
@@ -620,11 +622,11 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
     else
         launch_grouping(p, w, op_source(p, 0), 0, (int64_t)L, big_threshold(s), ushow, ds, st);
     if (for_pull)
-        TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row, p.newlist,
-                  ds, (uint32_t)DEV_ERR_TABLE_FULL);
+        TN_LAUNCH((k_probe<true>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row,
+                  (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_TABLE_FULL, make_optdev(t), t->seed);
     else
         TN_LAUNCH((k_probe<false>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row,
-                  (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+                  (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY, make_optdev(t), t->seed);
 }
 
 // The three kernels touch disjoint rows.  k_apply_big is latency-bound (few wavefronts, long
@@ -842,7 +844,7 @@ int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int 
     const OptDev o = make_optdev(t);
     const int blocks = launch_grid(n, 256, GRID_CAP * 2);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
-    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL, make_optdev(t), t->seed);
     TN_LAUNCH(k_init_rows, dim3(blocks), dim3(256), st, s, o, t->seed, signs, rows, newlist, t->dstatus);
     TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     if (wdim % 4 == 0 && s.wstride % 4 == 0 && aligned16(out))
@@ -896,7 +898,7 @@ int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, (uint32_t)n, (uint32_t)group_cap((size_t)n));
     launch_grouping(p, w, src, n, n, big_threshold(t->store), nullptr, ds, st);
     TN_LAUNCH((k_probe<false>), dim3(launch_grid(n, 256, GRID_CAP * 2)), dim3(256), st, t->store, p.grp_sign,
-              (int64_t)0, ds, (uint32_t)n, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY);
+              (int64_t)0, ds, (uint32_t)n, p.grp_row, (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY, make_optdev(t), t->seed);
     TN_TRY(launch_apply(t, p, src, ds, n, aligned16(grads) && dim % 4 == 0, st));
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpush->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
@@ -928,7 +930,7 @@ int tn_sparse_table_load_rows(uint32_t handle, const uint64_t* signs, const floa
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
     TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, (uint32_t)n, 0u);
-    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, t->dstatus, (uint32_t)DEV_ERR_TABLE_FULL, make_optdev(t), t->seed);
     TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, t->dstatus);
     TN_LAUNCH(k_load_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state);
     TN_HIP(hipGetLastError());
@@ -958,7 +960,7 @@ int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t 
     uint32_t* rows = (uint32_t*)t->ws.p;
     const Store& s = t->store;
     const int blocks = launch_grid(n, 256, GRID_CAP * 4);
-    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, (uint32_t*)nullptr, t->dstatus, 0u);
+    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, (uint32_t*)nullptr, t->dstatus, 0u, make_optdev(t), t->seed);
     TN_LAUNCH(k_export_rows, dim3(blocks), dim3(256), st, s, make_optdev(t), rows, n, w, state, found);
     TN_HIP(hipGetLastError());
     TN_HIP(hipStreamSynchronize(st));
@@ -1018,15 +1020,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds);
         t->plan_valid = false;
-        TN_TRY(upload_slots(t, p, descs, lbase, st));
+        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN, use_lds ? w.bcount : nullptr,
+                            use_lds ? w.nbuckets + 1 + w.nb2 : 0));
 
         const Store& s = t->store;
         const OptDev o = make_optdev(t);
         DevStatus* ds = t->dplan;
         launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st);
         const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
-        TN_LAUNCH(k_init_rows, dim3(gblocks), dim3(256), st, s, o, t->seed, p.grp_sign, p.grp_row, p.newlist, ds);
-        TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
                       ds, p.grp_row, p.where_u, p.ubase, N, p.descs);
@@ -1035,7 +1036,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                       p.grp_row, p.where_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
         TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
-                  reinterpret_cast<uint32_t*>(t->hpull));
+                  reinterpret_cast<uint32_t*>(t->hpull), s.count);
         t->pull_pending = true;
         t->pull_slots = N;
         t->pending_rows.assign(var_rows, var_rows + N);
@@ -1121,11 +1122,11 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     };
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
-        TN_TRY(upload_slots(t, p, descs, lbase, st));
-        TN_LAUNCH(k_begin_push, dim3(1), dim3(64), st, ds);
+        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_REUSE_PLAN));
         TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
                   (uint32_t)L, p.vals_copy, &ds->mismatch);
-        TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush));
+        TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush),
+                  (unsigned long long*)nullptr);
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // The counts only touch the plan's member lists, which a mismatch discards anyway:
         // they run while the host waits for the comparison.
@@ -1141,13 +1142,14 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, false)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
-        TN_TRY(upload_slots(t, p, descs, lbase, st));
+        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
         launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
         TN_TRY(launch_counts(false));
     }
     TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
     TN_HIP(hipGetLastError());
-    TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush));
+    TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush),
+              (unsigned long long*)nullptr);
     t->push_pending = true;
     t->push_slots = N;
     return TN_OK;
