@@ -75,16 +75,32 @@ __device__ __forceinline__ uint32_t bucket_of(const SlotDesc& d, uint64_t sign) 
     return d.tbase + (uint32_t)__umul64hi(mix64(sign), (uint64_t)d.tcap);
 }
 
-// One pass over a tile: calls f(gi, slot, sign) for each of its lookups.
+// One pass over a tile: calls f(gi, slot, descriptor, sign) for each of its
+// lookups.  A tile usually lies inside one slot: then the slot is looked up
+// once, its descriptor sits in registers and the loads of the signs do not
+// depend on anything.
 template <typename F>
 __device__ __forceinline__ void for_tile(uint32_t tile, const SlotDesc* descs, const uint32_t* lb, int N, uint32_t L,
                                          F f) {
+    const uint32_t g0 = tile * LDS_TILE;
+    const uint32_t g1 = min(L, g0 + (uint32_t)LDS_TILE) - 1;
+    const int s0 = find_slot(lb, N, g0);
+    if (g1 < lb[s0 + 1]) {
+        const SlotDesc d = descs[s0];
+        const uint32_t base = lb[s0];
+#pragma unroll
+        for (int j = 0; j < LDS_TILE_ITEMS; j++) {
+            const uint32_t gi = g0 + j * 256 + threadIdx.x;
+            if (gi <= g1) f(gi, s0, d, (uint64_t)d.values[gi - base]);
+        }
+    } else {
 #pragma unroll 4
-    for (int j = 0; j < LDS_TILE_ITEMS; j++) {
-        const uint32_t gi = tile * LDS_TILE + j * 256 + threadIdx.x;
-        if (gi >= L) break;
-        const int sl = find_slot(lb, N, gi);
-        f(gi, sl, (uint64_t)descs[sl].values[gi - lb[sl]]);
+        for (int j = 0; j < LDS_TILE_ITEMS; j++) {
+            const uint32_t gi = g0 + j * 256 + threadIdx.x;
+            if (gi > g1) break;
+            const int sl = find_slot(lb, N, gi);
+            f(gi, sl, descs[sl], (uint64_t)descs[sl].values[gi - lb[sl]]);
+        }
     }
 }
 
@@ -108,10 +124,10 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
         for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
         __syncthreads();
         const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;  // lowest bucket the tile can touch
-        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, uint64_t sign) {
+        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
             vals_copy[gi] = sign;
             first_of[gi] = gi;
-            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+            const uint32_t local = bucket_of(d, sign) - b0;
             if (local < LDS_SPAN)
                 atomicAdd(&hist[local], 1u);
             else
@@ -167,16 +183,16 @@ __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict_
         for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
         __syncthreads();
         const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;
-        for_tile(tile, descs, lb, N, L, [&](uint32_t, int sl, uint64_t sign) {
-            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+        for_tile(tile, descs, lb, N, L, [&](uint32_t, int, const SlotDesc& d, uint64_t sign) {
+            const uint32_t local = bucket_of(d, sign) - b0;
             if (local < LDS_SPAN) atomicAdd(&hist[local], 1u);
         });
         __syncthreads();
         for (int i = threadIdx.x; i < LDS_SPAN; i += 256)
             if (hist[i]) hist[i] = atomicAdd(&bcursor[b0 + i], hist[i]);  // the tile's slice of the bucket
         __syncthreads();
-        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, uint64_t sign) {
-            const uint32_t local = bucket_of(descs[sl], sign) - b0;
+        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
+            const uint32_t local = bucket_of(d, sign) - b0;
             if (local < LDS_SPAN) {
                 const uint32_t at = atomicAdd(&hist[local], 1u);
                 pkey[at] = sign;

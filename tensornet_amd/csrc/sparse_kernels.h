@@ -642,19 +642,24 @@ __global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict
     }
 }
 
-// Push: are the signs of this call the ones the plan was built from?
+// Push: are the signs of this call the ones the plan was built from?  With
+// list != nullptr the same pass starts the click sums of the plan's member
+// lists at zero (the show counts of the pull stay), as k_reset_counts would.
 __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                       const uint64_t* __restrict__ vals_copy, uint32_t* mismatch) {
+                                                       const uint64_t* __restrict__ vals_copy, DevStatus* status,
+                                                       Member* __restrict__ list) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
+    const uint32_t n_single = status->n_single, n_members = status->n_members;
     bool bad = false;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
         bad |= (uint64_t)descs[sl].values[gi - lb[sl]] != vals_copy[gi];
+        if (list && gi < n_single + n_members) list[group_id(gi, n_single, n_members, L)].click = 0;
     }
-    if (bad) atomicOr(mismatch, 1u);
+    if (bad) atomicOr(&status->mismatch, 1u);
 }
 
 // Push: batch_show = occurrences, batch_click = sum of labels per distinct sign

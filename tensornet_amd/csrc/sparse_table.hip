@@ -1123,14 +1123,19 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_REUSE_PLAN));
+        const bool clicks = t->plan_has_show && with_click;  // the verify pass also clears the click sums
         TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
-                  (uint32_t)L, p.vals_copy, &ds->mismatch);
+                  (uint32_t)L, p.vals_copy, ds, clicks ? p.list : (Member*)nullptr);
         TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush),
                   (unsigned long long*)nullptr);
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // The counts only touch the plan's member lists, which a mismatch discards anyway:
         // they run while the host waits for the comparison.
-        TN_TRY(launch_counts(t->plan_has_show));
+        if (clicks)
+            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
+                      p.where_u, p.list);
+        else
+            TN_TRY(launch_counts(t->plan_has_show));
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
