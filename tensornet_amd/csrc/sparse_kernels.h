@@ -1098,6 +1098,7 @@ template <int KIND, int LPG>
 __global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc src, DevStatus* status,
                                                       const uint32_t* __restrict__ grp_row,
                                                       const Member* __restrict__ list) {
+    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
     const uint32_t n_single = status->n_single;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;
@@ -1178,6 +1179,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                                                    const uint32_t* __restrict__ grp_cnt,
                                                    const Member* __restrict__ list, uint32_t big_k,
                                                    uint32_t ids_cap) {
+    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
     const uint32_t n_multi = status->n_multi;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;                       // my float4 inside the row
@@ -1305,6 +1307,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
     const int D = s.D;
     const int Dp = D + 1;  // padded staging row: lanes walking down a column hit different banks
     const int lane = threadIdx.x;
+    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
     const uint32_t n_big = status->n_big;
     const int per_chunk = (BIG_GBUF / Dp) < 64 ? (BIG_GBUF / Dp) : 64;
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
@@ -1441,6 +1444,7 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
                                                       const uint32_t* __restrict__ grp_cnt,
                                                       const Member* __restrict__ list, uint32_t big_k,
                                                       uint32_t ids_cap) {
+    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
     const uint32_t n_single = status->n_single, n_multi = status->n_multi;
     const int D = s.D;
     const uint32_t stride = gridDim.x * blockDim.x;

@@ -1129,13 +1129,15 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush),
                   (unsigned long long*)nullptr);
         TN_HIP(hipEventRecord(t->verify_ev, st));
-        // The counts only touch the plan's member lists, which a mismatch discards anyway:
-        // they run while the host waits for the comparison.
+        // Counts and apply kernels are queued before the host knows the outcome: the counts only
+        // touch the plan's member lists, which a mismatch discards anyway, and the apply kernels
+        // return at once when the mismatch flag is set.  The device never waits for the host.
         if (clicks)
             TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
                       p.where_u, p.list);
         else
             TN_TRY(launch_counts(t->plan_has_show));
+        TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
@@ -1150,8 +1152,8 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
         launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
         TN_TRY(launch_counts(false));
+        TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
     }
-    TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
     TN_HIP(hipGetLastError());
     TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush),
               (unsigned long long*)nullptr);
