@@ -569,8 +569,8 @@ void launch_mask_grouping(const Plan& p, const Scratch& w, int64_t n_upper, uint
 // signs for a pull).  use_lds picks the remap through LDS (pull only).  The
 // upload of the descriptors has cleared the status block and, for the LDS path,
 // the bucket counters.
-void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull, bool use_lds,
-                       hipStream_t st) {
+int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, uint32_t L, bool for_pull, bool use_lds,
+                      hipStream_t st) {
     DevStatus* ds = t->dplan;
     const Store& s = t->store;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
@@ -587,6 +587,18 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
         else
             TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
                       w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
+        if (lds_groups) {
+            // The grouping of the distinct records only needs what the dedup handed over: it runs on
+            // the side stream beside the ranking of the first occurrences (LDS / latency bound
+            // against streaming kernels) and joins before the member lists are written.
+            const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
+            TN_HIP(hipEventRecord(t->fork_ev, st));
+            TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), t->side, p.lbase, N, w.nb2, w.cursor2, w.recs,
+                      big_threshold(s), w.aux, w.bcounts);
+            TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
+            TN_HIP(hipEventRecord(t->join_ev, t->side));
+        }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
         if (lds_groups)
@@ -612,9 +624,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
-        TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), st, p.lbase, N, w.nb2, w.cursor2, w.recs, big_threshold(s),
-                  w.aux, w.bcounts);
-        TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), st, w.bcounts, w.bbase, w.nb2, ds);
+        TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
         TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.rank_at, L,
                   big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u);
     } else if (N <= MASK_SLOTS)
@@ -627,6 +637,7 @@ void launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, u
     else
         TN_LAUNCH((k_probe<false>), dim3(lblocks), dim3(256), st, s, p.grp_sign, (int64_t)0, ds, L, p.grp_row,
                   (uint32_t*)nullptr, ds, (uint32_t)DEV_ERR_UNKNOWN_KEY, make_optdev(t), t->seed);
+    return TN_OK;
 }
 
 // The three kernels touch disjoint rows.  k_apply_big is latency-bound (few wavefronts, long
@@ -1026,7 +1037,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         const Store& s = t->store;
         const OptDev o = make_optdev(t);
         DevStatus* ds = t->dplan;
-        launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st);
+        TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st));
         const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
@@ -1150,7 +1161,7 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, false)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
-        launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st);
+        TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st));
         TN_TRY(launch_counts(false));
         TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
     }
