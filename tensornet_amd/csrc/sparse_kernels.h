@@ -195,6 +195,48 @@ constexpr int PROBE_WIDTH = 4;
 
 __device__ __forceinline__ void init_row(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row);
 
+// Slot of `sign` in the table, NO_ROW if absent (or, with INSERT, if the table
+// is full).  With INSERT an absent sign claims the first free slot of its probe
+// sequence and is_new tells whether this call made the claim.
+template <bool INSERT>
+__device__ __forceinline__ uint32_t probe_slot(const Store& s, uint64_t sign, bool& is_new) {
+    is_new = false;
+    if (sign == EMPTY_KEY) {
+        if (INSERT) {
+            is_new = atomicCAS(s.special, 0u, 1u) == 0u;
+            return (uint32_t)s.cap;
+        }
+        return ld_relaxed(s.special) ? (uint32_t)s.cap : NO_ROW;
+    }
+    // PROBE_WIDTH consecutive slots per round trip: their loads are issued together, so a
+    // probe sequence of a few slots costs one memory latency instead of one per slot.
+    uint64_t idx = slot_of(sign, s.cap);
+    for (uint64_t p = 0; p < s.cap; p += PROBE_WIDTH) {
+        uint64_t at[PROBE_WIDTH], k[PROBE_WIDTH];
+#pragma unroll
+        for (int j = 0; j < PROBE_WIDTH; j++) {
+            at[j] = idx + j;
+            if (at[j] >= s.cap) at[j] -= s.cap;
+            // plain load: a key never changes once set, and a stale free slot is settled by the compare-and-swap
+            k[j] = s.keys[at[j]];
+        }
+#pragma unroll
+        for (int j = 0; j < PROBE_WIDTH; j++) {
+            if (k[j] == sign) return (uint32_t)at[j];
+            if (k[j] == EMPTY_KEY) {
+                if (!INSERT) return NO_ROW;
+                uint64_t old = atomicCAS(ull(&s.keys[at[j]]), EMPTY_KEY, sign);
+                if (old == EMPTY_KEY || old == sign) {
+                    is_new = old == EMPTY_KEY;
+                    return (uint32_t)at[j];
+                }
+            }
+        }
+        idx = at[PROBE_WIDTH - 1] + 1 == s.cap ? 0 : at[PROBE_WIDTH - 1] + 1;
+    }
+    return NO_ROW;
+}
+
 // With groups_of != nullptr the signs are those of its groups (ids_cap = size of the id space).
 template <bool INSERT>
 __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restrict__ signs, int64_t n_host,
@@ -207,50 +249,8 @@ __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restri
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride) {
         const int64_t i = groups_of ? (int64_t)group_id((uint32_t)t, n_single, n_multi, ids_cap) : t;
         const uint64_t sign = signs[i];
-        uint32_t row = NO_ROW;
-        bool is_new = false;
-        if (sign == EMPTY_KEY) {
-            if (INSERT) {
-                is_new = atomicCAS(s.special, 0u, 1u) == 0u;
-                row = (uint32_t)s.cap;
-            } else if (ld_relaxed(s.special)) {
-                row = (uint32_t)s.cap;
-            }
-        } else {
-            // PROBE_WIDTH consecutive slots per round trip: their loads are issued together, so a
-            // probe sequence of a few slots costs one memory latency instead of one per slot.
-            uint64_t idx = slot_of(sign, s.cap);
-            bool done = false;
-            for (uint64_t p = 0; p < s.cap && !done; p += PROBE_WIDTH) {
-                uint64_t at[PROBE_WIDTH], k[PROBE_WIDTH];
-#pragma unroll
-                for (int j = 0; j < PROBE_WIDTH; j++) {
-                    at[j] = idx + j;
-                    if (at[j] >= s.cap) at[j] -= s.cap;
-                    k[j] = s.keys[at[j]];  // plain load: a key never changes once set, and a stale free slot is settled by the compare-and-swap
-                }
-#pragma unroll
-                for (int j = 0; j < PROBE_WIDTH; j++) {
-                    if (done) break;
-                    if (k[j] == sign) {
-                        row = (uint32_t)at[j];
-                        done = true;
-                    } else if (k[j] == EMPTY_KEY) {  // possibly stale: the compare-and-swap decides
-                        if (!INSERT) {
-                            done = true;
-                        } else {
-                            uint64_t old = atomicCAS(ull(&s.keys[at[j]]), EMPTY_KEY, sign);
-                            if (old == EMPTY_KEY || old == sign) {
-                                row = (uint32_t)at[j];
-                                is_new = old == EMPTY_KEY;
-                                done = true;
-                            }
-                        }
-                    }
-                }
-                idx = at[PROBE_WIDTH - 1] + 1 == s.cap ? 0 : at[PROBE_WIDTH - 1] + 1;
-            }
-        }
+        bool is_new;
+        const uint32_t row = probe_slot<INSERT>(s, sign, is_new);
         rows[i] = row;
         if (row == NO_ROW && miss_err) atomicOr(&status->err, miss_err);
         if (INSERT) {
@@ -1282,7 +1282,10 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
 }
 
 constexpr int BIG_DIM_MAX = 128;    // largest dim k_apply_big stages in LDS
-constexpr int BIG_GBUF = 2176;      // floats of gradient staging per wavefront
+constexpr int BIG_GBUF = 2176;      // floats of gradient staging per wavefront at most (dynamic LDS: big_gbuf_floats)
+
+// Staging for up to 64 records of dim D (rows padded by one float), capped at BIG_GBUF.
+inline int big_gbuf_floats(int D) { return 64 * (D + 1) < BIG_GBUF ? 64 * (D + 1) : BIG_GBUF; }
 
 // A sign with many records (it occurs in many slots) would make one lane
 // group chase a long chain of dependent loads.  Here one wavefront owns the
@@ -1297,9 +1300,9 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                                                   const uint32_t* __restrict__ grp_row,
                                                   const uint32_t* __restrict__ grp_off,
                                                   const uint32_t* __restrict__ grp_cnt,
-                                                  const Member* __restrict__ list) {
+                                                  const Member* __restrict__ list, int gbuf_floats) {
     __shared__ float rw[BIG_DIM_MAX], ra[BIG_DIM_MAX], rb[BIG_DIM_MAX];
-    __shared__ float gbuf[BIG_GBUF];
+    extern __shared__ float gbuf[];  // gbuf_floats floats
     __shared__ const float* gptr[64];
     __shared__ int gshow[64], gclick[64], gok[64];
     __shared__ double msq[64];
@@ -1309,7 +1312,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
     const int lane = threadIdx.x;
     if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
     const uint32_t n_big = status->n_big;
-    const int per_chunk = (BIG_GBUF / Dp) < 64 ? (BIG_GBUF / Dp) : 64;
+    const int per_chunk = (gbuf_floats / Dp) < 64 ? (gbuf_floats / Dp) : 64;
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
     const bool pow2 = (D & (D - 1)) == 0;
     const double inv_d = 1.0 / (double)D;  // exact when D is a power of two

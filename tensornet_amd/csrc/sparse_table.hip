@@ -652,8 +652,10 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
     if (with_big) {
         TN_HIP(hipEventRecord(t->fork_ev, st));
         TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
-        TN_LAUNCH((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64), t->side, s, o,
-                  src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list);
+        const int gfloats = big_gbuf_floats(s.D);
+        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
+                      gfloats * sizeof(float), t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
+                      p.list, gfloats);
         TN_HIP(hipEventRecord(t->join_ev, t->side));
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \

@@ -130,12 +130,14 @@ extern bool g_profile_on;
 void prof_begin(const char* name, hipStream_t st);
 void prof_end(hipStream_t st);
 
-#define TN_LAUNCH(KERNEL, GRID, BLOCK, STREAM, ...)                            \
+#define TN_LAUNCH_LDS(KERNEL, GRID, BLOCK, LDS_BYTES, STREAM, ...)              \
     do {                                                                       \
         if (::tn::g_profile_on) ::tn::prof_begin(#KERNEL, STREAM);             \
-        hipLaunchKernelGGL(KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__);       \
+        hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS_BYTES, STREAM, __VA_ARGS__); \
         if (::tn::g_profile_on) ::tn::prof_end(STREAM);                        \
     } while (0)
+
+#define TN_LAUNCH(KERNEL, GRID, BLOCK, STREAM, ...) TN_LAUNCH_LDS(KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__)
 
 }  // namespace tn
 
