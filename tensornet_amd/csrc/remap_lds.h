@@ -40,7 +40,7 @@
 
 namespace tn {
 
-constexpr int LDS_TILE = 4096;          // lookups per tile of the partition kernels
+constexpr int LDS_TILE = 2048;          // lookups per tile of the partition kernels
 constexpr int LDS_TILE_ITEMS = LDS_TILE / 256;
 constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
 constexpr int LDS_BUCKET_TARGET = 768;  // average lookups per bucket
@@ -104,6 +104,19 @@ __device__ __forceinline__ void for_tile(uint32_t tile, const SlotDesc* descs, c
     }
 }
 
+// Buckets a tile can touch: from the first bucket of its first slot (b0) up to the
+// last bucket of its last slot, span_cap at most (the host sizes the LDS histogram for the
+// widest tile of the call, LDS_SPAN at most).
+__device__ __forceinline__ uint32_t tile_span(uint32_t tile, const SlotDesc* descs, const uint32_t* lb, int N,
+                                              uint32_t L, uint32_t span_cap, uint32_t& b0) {
+    const uint32_t g0 = tile * LDS_TILE;
+    const uint32_t g1 = min(L, g0 + (uint32_t)LDS_TILE) - 1;
+    const SlotDesc& first = descs[find_slot(lb, N, g0)];
+    const SlotDesc& last = descs[find_slot(lb, N, g1)];
+    b0 = first.tbase;
+    return min(span_cap, last.tbase + last.tcap - b0);
+}
+
 __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
@@ -115,26 +128,28 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
 __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
                                                   int N, uint32_t L, uint32_t* bcount,
                                                   uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ first_of,
-                                                  DevStatus* status) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
-    __shared__ uint32_t hist[LDS_SPAN];
+                                                  DevStatus* status, uint32_t span_cap) {
+    extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]
+    uint32_t* lb = smem;
+    uint32_t* hist = smem + N + 1;
     load_lbase(lb, lbase, N);
     const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
+        uint32_t b0;  // lowest bucket the tile can touch
+        const uint32_t span = tile_span(tile, descs, lb, N, L, span_cap, b0);
+        for (uint32_t i = threadIdx.x; i < span; i += 256) hist[i] = 0;
         __syncthreads();
-        const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;  // lowest bucket the tile can touch
         for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
             vals_copy[gi] = sign;
             first_of[gi] = gi;
             const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < LDS_SPAN)
+            if (local < span)
                 atomicAdd(&hist[local], 1u);
             else
                 atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
         });
         __syncthreads();
-        for (int i = threadIdx.x; i < LDS_SPAN; i += 256)
+        for (uint32_t i = threadIdx.x; i < span; i += 256)
             if (hist[i]) atomicAdd(&bcount[b0 + i], hist[i]);
         __syncthreads();
     }
@@ -174,26 +189,41 @@ __global__ __launch_bounds__(1024) void k_lds_offsets(const uint32_t* __restrict
 __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                      uint32_t* bcursor, uint64_t* __restrict__ pkey,
-                                                     uint32_t* __restrict__ pgi) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
-    __shared__ uint32_t hist[LDS_SPAN];  // first the tile's count per bucket, then its write cursor
+                                                     uint32_t* __restrict__ pgi, uint32_t span_cap) {
+    extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]: first the tile's count per bucket, then its write cursor
+    uint32_t* lb = smem;
+    uint32_t* hist = smem + N + 1;
     load_lbase(lb, lbase, N);
     const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        for (int i = threadIdx.x; i < LDS_SPAN; i += 256) hist[i] = 0;
+        uint32_t b0;
+        const uint32_t span = tile_span(tile, descs, lb, N, L, span_cap, b0);
+        for (uint32_t i = threadIdx.x; i < span; i += 256) hist[i] = 0;
         __syncthreads();
-        const uint32_t b0 = descs[find_slot(lb, N, tile * LDS_TILE)].tbase;
         for_tile(tile, descs, lb, N, L, [&](uint32_t, int, const SlotDesc& d, uint64_t sign) {
             const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < LDS_SPAN) atomicAdd(&hist[local], 1u);
+            if (local < span) atomicAdd(&hist[local], 1u);
         });
         __syncthreads();
-        for (int i = threadIdx.x; i < LDS_SPAN; i += 256)
-            if (hist[i]) hist[i] = atomicAdd(&bcursor[b0 + i], hist[i]);  // the tile's slice of the bucket
+        // the tile's slice of every bucket it touches; all atomics of a thread are in flight together
+        for (uint32_t i0 = 0; i0 < span; i0 += 256 * 4) {
+            uint32_t got[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t i = i0 + q * 256 + threadIdx.x;
+                const uint32_t cnt = i < span ? hist[i] : 0;
+                got[q] = cnt ? atomicAdd(&bcursor[b0 + i], cnt) : 0;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t i = i0 + q * 256 + threadIdx.x;
+                if (i < span) hist[i] = got[q];
+            }
+        }
         __syncthreads();
         for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
             const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < LDS_SPAN) {
+            if (local < span) {
                 const uint32_t at = atomicAdd(&hist[local], 1u);
                 pkey[at] = sign;
                 pgi[at] = gi;

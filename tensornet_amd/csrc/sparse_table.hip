@@ -354,6 +354,7 @@ struct Scratch {
     uint32_t ntiles;
     // LDS remap
     uint32_t nbuckets;
+    uint32_t span_cap;  // buckets the widest tile touches (entries of the partition kernels' LDS histogram)
     uint32_t* bcount;
     uint32_t* bstart;
     uint32_t* bcursor;
@@ -455,7 +456,8 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
 // number of buckets); otherwise *use_lds comes back false and tbase/tcap describe the
 // slot's region of the global dedup table.
 int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64_t* lens, std::vector<SlotDesc>& descs,
-                std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what, bool* use_lds) {
+                std::vector<uint32_t>& lbase, size_t& L, size_t& dt_entries, const char* what, bool* use_lds,
+                uint32_t* span_cap = nullptr) {
     if (N <= 0 || !values || !lens) return fail(TN_ERR_INVALID_ARGUMENT, std::string(what) + ": no slots");
     if (N > MAX_SLOTS)
         return fail(TN_ERR_UNSUPPORTED, std::string(what) + ": more than " + std::to_string(MAX_SLOTS) + " slots");
@@ -494,6 +496,18 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
                 nb += sub;
             }
             dt_entries = nb;
+            // buckets the widest tile of the partition kernels touches: first bucket of the slot of
+            // its first lookup .. last bucket of the slot of its last lookup
+            size_t widest = 1;
+            int s0 = 0, s1 = 0;
+            for (size_t g0 = 0; g0 < l; g0 += LDS_TILE) {
+                const size_t g1 = std::min(l, g0 + (size_t)LDS_TILE) - 1;
+                while (s0 + 1 < N && lbase[s0 + 1] <= g0) s0++;
+                if (s1 < s0) s1 = s0;
+                while (s1 + 1 < N && lbase[s1 + 1] <= g1) s1++;
+                widest = std::max<size_t>(widest, (size_t)descs[s1].tbase + descs[s1].tcap - descs[s0].tbase);
+            }
+            if (span_cap) *span_cap = (uint32_t)std::min<size_t>(widest, LDS_SPAN);
         }
     }
     return TN_OK;
@@ -577,10 +591,12 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     const bool lds_groups = use_lds && N <= GRP_SLOTS;
     if (use_lds) {
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
-        TN_LAUNCH(k_lds_hist, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy, w.first_of,
-                  ds);
+        const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
+        TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy,
+                      w.first_of, ds, w.span_cap);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
-        TN_LAUNCH(k_lds_scatter, dim3(tiles), dim3(256), st, p.descs, p.lbase, N, L, w.bcursor, w.pkey, w.pgi);
+        TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.pkey,
+                      w.pgi, w.span_cap);
         if (lds_groups)
             TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
                       w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
@@ -1010,7 +1026,9 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         std::vector<SlotDesc> descs;
         std::vector<uint32_t> lbase;
         size_t L = 0, dt_entries = 0;
-        TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePull", &use_lds));
+        uint32_t span_cap = 0;
+        TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePull", &use_lds,
+                           &span_cap));
         bool vec = (wdim % 4 == 0) && (t->store.wstride % 4 == 0);
         for (int s = 0; s < N; s++) {
             if (var_rows[s] < 0 || !vars[s] || (value_lens[s] > 0 && !mapped_values[s]))
@@ -1032,6 +1050,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds);
+        w.span_cap = span_cap;
         t->plan_valid = false;
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN, use_lds ? w.bcount : nullptr,
                             use_lds ? w.nbuckets + 1 + w.nb2 : 0));
