@@ -414,6 +414,35 @@ def test_push_of_another_batch_than_the_last_pull(tn, oracle):
     pair.assert_rows_match(base)
 
 
+@pytest.mark.parametrize("slots,opt,hyper", [(40, "AdaGrad", ADAGRAD_HP), (128, "Adam", ADAM_HP),
+                                             (130, "AdaGrad", ADAGRAD_HP)])
+def test_large_ragged_batches_take_the_lds_path(tn, oracle, slots, opt, hyper):
+    """More than 32768 lookups in ragged slots (some empty, some with a handful of lookups,
+    so that tiles of the partition kernels straddle many slots), non-zero labels, signs shared
+    between slots, new signs in the second batch: remap and grouping through LDS (arrival-order
+    grouping above 128 slots) against the oracle."""
+    D = 8
+    rng = np.random.default_rng(100 + slots)
+    pair = Pair(tn, oracle, opt, D, hyper, reserve=400000, zero_init=True)
+    vocab = 40000
+    pool = synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool[:30000].view(np.uint64))
+    for step in range(2):
+        values = []
+        for s in range(slots):
+            kind = s % 5
+            n = 0 if kind == 0 else int(rng.integers(1, 8)) if kind == 1 else int(rng.integers(500, 4000))
+            hot = pool[rng.integers(0, 50, n)]                 # a few signs everywhere
+            cold = pool[rng.integers(0, vocab if step else 30000, n)]
+            values.append(np.where(rng.random(n) < 0.3, hot, cold))
+        assert sum(len(v) for v in values) > 40000
+        counts = check_pull(pair, values)
+        grads = synth.make_grads(counts, D, 0.01, seed=step)
+        labels = [rng.integers(0, 3, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+        assert pair.assert_rows_match(all_signs(values)) > 0.99
+
+
 def test_bound_ops_over_several_steps_without_waiting(tn, oracle):
     """Ops bound to their tensors once and called step after step: a pull runs behind
     the push before it without the host waiting in between, and a push whose signs were
