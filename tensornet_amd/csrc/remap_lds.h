@@ -160,30 +160,11 @@ __global__ __launch_bounds__(1024) void k_lds_offsets(const uint32_t* __restrict
                                                       uint32_t* __restrict__ bcursor, uint32_t nbuckets) {
     __shared__ uint32_t wsum[16];
     __shared__ uint32_t carry_sh;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) carry_sh = 0;
-    __syncthreads();
-    for (uint32_t start = 0; start < nbuckets; start += 1024) {
-        const uint32_t i = start + threadIdx.x;
-        const uint32_t v = (i < nbuckets) ? bcount[i] : 0;
-        uint32_t inc = v;
-        for (int o = 1; o < 64; o <<= 1) {
-            uint32_t t = __shfl_up(inc, o);
-            if (lane >= o) inc += t;
-        }
-        if (lane == 63) wsum[wave] = inc;
-        __syncthreads();
-        uint32_t base = carry_sh;
-        for (int wv = 0; wv < wave; wv++) base += wsum[wv];
-        if (i < nbuckets) {
-            bstart[i] = base + inc - v;
-            bcursor[i] = base + inc - v;
-        }
-        __syncthreads();
-        if (threadIdx.x == 1023) carry_sh = base + inc;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) bstart[nbuckets] = carry_sh;
+    const uint32_t total = scan_u32_1024(bcount, nbuckets, wsum, &carry_sh, [&](uint32_t i, uint32_t v) {
+        bstart[i] = v;
+        bcursor[i] = v;
+    });
+    if (threadIdx.x == 0) bstart[nbuckets] = total;
 }
 
 __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict__ descs,
@@ -594,37 +575,40 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
 // Exclusive scan of the per-bucket counts (one workgroup); also the totals.
 __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict__ bcounts, uint4* __restrict__ bbase,
                                                         uint32_t nb2, DevStatus* status) {
+    constexpr int ITEMS = 8;
     __shared__ uint4 wsum[16];
     __shared__ uint4 carry_sh;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    auto add = [](uint4 a, uint4 b) { return make_uint4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); };
     if (threadIdx.x == 0) carry_sh = make_uint4(0, 0, 0, 0);
     __syncthreads();
-    for (uint32_t start = 0; start < nb2; start += 1024) {
-        const uint32_t i = start + threadIdx.x;
-        const uint4 v = (i < nb2) ? bcounts[i] : make_uint4(0, 0, 0, 0);
-        uint4 inc = v;
+    for (uint32_t start = 0; start < nb2; start += 1024 * ITEMS) {
+        const uint32_t i0 = start + threadIdx.x * ITEMS;
+        uint4 v[ITEMS];
+        uint4 mine = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < ITEMS; j++) {
+            v[j] = (i0 + j < nb2) ? bcounts[i0 + j] : make_uint4(0, 0, 0, 0);
+            mine = add(mine, v[j]);
+        }
+        uint4 inc = mine;
         for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t tx = __shfl_up(inc.x, o), ty = __shfl_up(inc.y, o), tz = __shfl_up(inc.z, o),
-                           tw = __shfl_up(inc.w, o);
-            if (lane >= o) {
-                inc.x += tx;
-                inc.y += ty;
-                inc.z += tz;
-                inc.w += tw;
-            }
+            const uint4 t = make_uint4(__shfl_up(inc.x, o), __shfl_up(inc.y, o), __shfl_up(inc.z, o), __shfl_up(inc.w, o));
+            if (lane >= o) inc = add(inc, t);
         }
         if (lane == 63) wsum[wave] = inc;
         __syncthreads();
         uint4 base = carry_sh;
-        for (int wv = 0; wv < wave; wv++) {
-            base.x += wsum[wv].x;
-            base.y += wsum[wv].y;
-            base.z += wsum[wv].z;
-            base.w += wsum[wv].w;
+        for (int wv = 0; wv < wave; wv++) base = add(base, wsum[wv]);
+        uint4 run = make_uint4(base.x + inc.x - mine.x, base.y + inc.y - mine.y, base.z + inc.z - mine.z,
+                               base.w + inc.w - mine.w);
+#pragma unroll
+        for (int j = 0; j < ITEMS; j++) {
+            if (i0 + j < nb2) bbase[i0 + j] = run;
+            run = add(run, v[j]);
         }
-        if (i < nb2) bbase[i] = make_uint4(base.x + inc.x - v.x, base.y + inc.y - v.y, base.z + inc.z - v.z, base.w + inc.w - v.w);
         __syncthreads();
-        if (threadIdx.x == 1023) carry_sh = make_uint4(base.x + inc.x, base.y + inc.y, base.z + inc.z, base.w + inc.w);
+        if (threadIdx.x == 1023) carry_sh = add(base, inc);
         __syncthreads();
     }
     if (threadIdx.x == 0) {

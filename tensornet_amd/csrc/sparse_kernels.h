@@ -545,6 +545,48 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_flag_count(const uint32_t* __
     if (threadIdx.x == 0) tilesum[blockIdx.x] = total;
 }
 
+// Exclusive scan of in[0 .. n) by one workgroup of 1024 threads: out[i] = sum of in[0 .. i);
+// returns the total.  Every thread takes SCAN_ITEMS consecutive entries, so arrays of a few
+// thousand entries need one round of barriers.  wsum: 16 entries of LDS, carry: one.
+constexpr int SCAN_ITEMS = 8;
+
+template <typename Out>
+__device__ __forceinline__ uint32_t scan_u32_1024(const uint32_t* __restrict__ in, uint32_t n, uint32_t* wsum,
+                                                  uint32_t* carry, Out out) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) *carry = 0;
+    __syncthreads();
+    for (uint32_t start = 0; start < n; start += 1024 * SCAN_ITEMS) {
+        const uint32_t i0 = start + threadIdx.x * SCAN_ITEMS;
+        uint32_t v[SCAN_ITEMS];
+        uint32_t mine = 0;
+#pragma unroll
+        for (int j = 0; j < SCAN_ITEMS; j++) {
+            v[j] = (i0 + j < n) ? in[i0 + j] : 0;
+            mine += v[j];
+        }
+        uint32_t inc = mine;
+        for (int o = 1; o < 64; o <<= 1) {
+            uint32_t t = __shfl_up(inc, o);
+            if (lane >= o) inc += t;
+        }
+        if (lane == 63) wsum[wave] = inc;
+        __syncthreads();
+        uint32_t base = *carry;
+        for (int wv = 0; wv < wave; wv++) base += wsum[wv];
+        uint32_t run = base + inc - mine;
+#pragma unroll
+        for (int j = 0; j < SCAN_ITEMS; j++) {
+            if (i0 + j < n) out(i0 + j, run);
+            run += v[j];
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) *carry = base + inc;
+        __syncthreads();
+    }
+    return *carry;
+}
+
 // Step 3 (one workgroup): exclusive scan of the tile counts; total distinct
 // count U; size of the group table; ubase of trailing empty slots.
 __global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict__ tilesum,
@@ -553,27 +595,7 @@ __global__ __launch_bounds__(1024) void k_scan_tiles(const uint32_t* __restrict_
                                                      int N, uint32_t L, DevStatus* status) {
     __shared__ uint32_t wsum[16];
     __shared__ uint32_t carry_sh;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) carry_sh = 0;
-    __syncthreads();
-    for (uint32_t start = 0; start < ntiles; start += 1024) {
-        const uint32_t i = start + threadIdx.x;
-        const uint32_t v = (i < ntiles) ? tilesum[i] : 0;
-        uint32_t inc = v;
-        for (int o = 1; o < 64; o <<= 1) {
-            uint32_t t = __shfl_up(inc, o);
-            if (lane >= o) inc += t;
-        }
-        if (lane == 63) wsum[wave] = inc;
-        __syncthreads();
-        uint32_t base = carry_sh;
-        for (int wv = 0; wv < wave; wv++) base += wsum[wv];
-        if (i < ntiles) tileoff[i] = base + inc - v;
-        __syncthreads();
-        if (threadIdx.x == 1023) carry_sh = base + inc;
-        __syncthreads();
-    }
-    const uint32_t U = carry_sh;
+    const uint32_t U = scan_u32_1024(tilesum, ntiles, wsum, &carry_sh, [&](uint32_t i, uint32_t v) { tileoff[i] = v; });
     if (threadIdx.x == 0) {
         status->n_unique = U;
         uint32_t g = U + U / 2;
