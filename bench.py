@@ -27,9 +27,26 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-# HBM bytes per launch (read + written) of the cfg3 kernels from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
-# scaled by what the same counters read for the dense Adam stream of known size; see profiles/.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch (read + written) of the cfg3 kernels at 5e8 resident keys, from the rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs summarised in profiles/cfg3_adagrad_dim16_pull_push.md (FETCH_SIZE x 2.0 and
+# WRITE_SIZE x 1.0: the factors that make the counters reproduce the known traffic of the dense Adam stream).
+# Counters cannot be read from inside this script; the figures are refreshed together with that summary.
+MEASURED_TRAFFIC = {
+    "k_gather_vars": 506400000,
+    "k_group_emit": 454300000,
+    "k_apply_single": 340600000,
+    "k_lds_scatter": 205200000,
+    "k_lds_dedup": 203400000,
+    "k_lds_mapped": 139000000,
+    "k_apply_vec": 117400000,
+    "k_verify_values": 114600000,
+    "k_lds_hist": 101300000,
+    "k_apply_big": 89000000,
+    "k_group_count": 49300000,
+    "k_count_click": 42400000,
+    "k_lds_flags": 20700000,
+    "k_lds_assign": 20500000,
+}
 
 
 def state_bytes(opt, dim):
