@@ -226,6 +226,43 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
                             const float* const* grads, const int64_t* grad_rows, int grad_dim,
                             const int64_t* const* feature_labels, void* stream);
 
+/*
+ * The step TensorFlow runs between the two ops for every slot -- the combiner
+ * of tf.nn.embedding_lookup_sparse, reached by the reference through
+ * embedding_column.get_dense_tensor (tensornet/layers/embedding_features.py:278-280)
+ * with the mapped ids of tensornet/feature_column/category_column.py:42-51 --
+ * done on the device on both sides of the table.
+ *
+ * Forward: out[s] is a device matrix [batch, dim]; example_ids[s] holds, for
+ * every lookup of slot s, the index of its example (SparseTensor.indices[:, 0]:
+ * non-decreasing, in [0, batch)); mapped_values[s] are the ids the pull op
+ * returned and vars[s] ([var_rows[s], dim]) the variable it filled.
+ *   out[s][b, :] = (sum over the lookups of example b, in order, of vars[s][mapped, :]) / d(n_b)
+ *   d(n) = 1 (TN_COMBINER_SUM), n (MEAN), sqrt(n) (SQRTN); examples without lookups give zeros.
+ * Returns after the stream work has completed; ids outside the variable are
+ * TN_ERR_VAR_CAPACITY, unsorted or out-of-range example ids TN_ERR_INVALID_ARGUMENT.
+ */
+enum { TN_COMBINER_SUM = 0, TN_COMBINER_MEAN = 1, TN_COMBINER_SQRTN = 2 };
+int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* const* mapped_values,
+                               const int64_t* value_lens, const int64_t* const* example_ids, const float* const* vars,
+                               const int64_t* var_rows, int dim, int64_t batch, int combiner, float* const* out,
+                               void* stream);
+
+/*
+ * Backward: SparseTablePush (as tn_sparse_table_push_op) fed with the gradient
+ * of the combiner's output instead of per-distinct-sign rows.  pooled_grads[s]
+ * is a device matrix [batch, grad_dim]; the gradient row of the j-th distinct
+ * sign of slot s -- what TensorFlow hands the reference's op as grads[s][j, :],
+ * core/kernels/sparse_table_ops.cc:336-352 -- is
+ *   sum over the lookups of that sign, in order, of pooled_grads[s][example, :] * (1 / d(n_example))
+ * computed on the device (the segmented reduction of the per-lookup gradients)
+ * and applied like a push.  Enqueues and returns like tn_sparse_table_push_op.
+ */
+int tn_sparse_table_push_pooled_op(uint32_t table_handle, int N, const int64_t* const* values,
+                                   const int64_t* value_lens, const int64_t* const* example_ids,
+                                   const float* const* pooled_grads, int64_t batch, int grad_dim, int combiner,
+                                   const int64_t* const* feature_labels, void* stream);
+
 /* Wait for the table's enqueued work and return (and clear) its latched error. */
 int tn_sparse_table_sync(uint32_t handle);
 

@@ -109,6 +109,10 @@ SIGNATURES = {
     "tn_sparse_table_export_rows": (C.c_int, [C.c_uint32, _P, C.c_int64, _P, _P, _P, _P]),
     "tn_sparse_table_pull_op": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _PP, _I64P, C.c_int, _PP, _P]),
     "tn_sparse_table_push_op": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _PP, _I64P, C.c_int, _PP, _P]),
+    "tn_sparse_table_combine_op": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _PP, _PP, _I64P, C.c_int, C.c_int64,
+                                             C.c_int, _PP, _P]),
+    "tn_sparse_table_push_pooled_op": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _PP, _PP, C.c_int64, C.c_int,
+                                                 C.c_int, _PP, _P]),
     "tn_sparse_table_sync": (C.c_int, [C.c_uint32]),
     "tn_sparse_table_last_unique_counts": (C.c_int, [C.c_uint32, C.c_int, _I64P]),
     "tn_sparse_table_set_async": (C.c_int, [C.c_uint32, C.c_int]),

@@ -767,6 +767,8 @@ struct PushSrc {
     const uint32_t* ubase;
     const SlotDesc* descs;
     int dim;
+    // op-level push of pooled gradients: one reduced gradient row per distinct sign, record order
+    const float* flat;
 };
 
 __device__ __forceinline__ uint64_t src_sign(const PushSrc& p, uint32_t u) {
@@ -1077,6 +1079,12 @@ __device__ __forceinline__ bool src_record(const PushSrc& p, Member member, cons
         g = p.grads + (uint64_t)u * p.dim;
         show = p.infos[u].batch_show;
         click = p.infos[u].batch_click;
+        return true;
+    }
+    show = member.show;
+    click = member.click;
+    if (p.flat) {
+        g = p.flat + (uint64_t)u * p.dim;
         return true;
     }
     const uint32_t sl = member.slot;

@@ -1,12 +1,18 @@
 // SparseTable host side: registry, HBM storage management and the launch
 // sequences of pull / push at table level (core/ps/table/sparse_table.cc:52-83)
 // and at operator level (core/kernels/sparse_table_ops.cc:170-265,317-368).
+#include "combine_kernels.h"
 #include "remap_lds.h"
 
 #include <algorithm>
 #include <cstring>
 
 namespace tn {
+
+// sort_pairs.hip
+int sort_pairs_temp_bytes(size_t n, int key_bits, size_t* bytes);
+int sort_pairs_u32(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out, const uint32_t* vals_in,
+                   uint32_t* vals_out, size_t n, int key_bits, hipStream_t st);
 
 namespace {
 
@@ -50,6 +56,8 @@ struct SparseTable {
     size_t hstage_bytes = 0;
     hipEvent_t stage_ev = nullptr;  // staging buffer free again
     hipEvent_t verify_ev = nullptr; // a push's comparison of the signs has been published
+    DevBuf comb_buf;                // slot descriptors of a combine op
+    DevBuf pooled_ws;               // scratch of a push of pooled gradients (sort buffers, reduced rows)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipEvent_t fork_ev = nullptr, join_ev = nullptr;
     bool stage_pending = false;
@@ -1056,10 +1064,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                             use_lds ? w.nbuckets + 1 + w.nb2 : 0));
 
         const Store& s = t->store;
-        const OptDev o = make_optdev(t);
         DevStatus* ds = t->dplan;
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st));
-        const int gblocks = launch_grid(L, 256, GRID_CAP * 2);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
                       ds, p.grp_row, p.where_u, p.ubase, N, p.descs);
@@ -1094,12 +1100,23 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     return fail(TN_ERR_HIP, "SparseTablePull: remap fell back twice");
 }
 
-int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
-                            const float* const* grads, const int64_t* grad_rows, int grad_dim,
-                            const int64_t* const* feature_labels, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// SparseTablePush.  With example_ids the gradients are pooled ([batch, dim] per slot, one row per
+// example): they are first reduced to one row per distinct sign (the gradient of the combiner).
+int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                 const float* const* grads, const int64_t* grad_rows, int grad_dim,
+                 const int64_t* const* feature_labels, const int64_t* const* example_ids, int64_t batch, int combiner,
+                 void* stream) {
     SparseTable* t = get_table(table_handle);
     if (!t) return fail(TN_ERR_BAD_HANDLE, "SparseTablePush: bad table handle " + std::to_string(table_handle));
-    if (!grads || !grad_rows || !feature_labels) return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush: NULL argument");
+    if (!grads || (!grad_rows && !example_ids) || !feature_labels)
+        return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush: NULL argument");
+    const bool pooled = example_ids != nullptr;
+    if (pooled && (batch <= 0 || combiner < COMBINE_SUM || combiner > COMBINE_SQRTN))
+        return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush (pooled): bad batch size or combiner");
     std::lock_guard<std::mutex> lk(t->mu);
     hipStream_t st = (hipStream_t)stream;
     TN_TRY(ensure_allocated(t, st));
@@ -1113,12 +1130,15 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
     TN_TRY(stage_slots(t, N, values, value_lens, descs, lbase, L, dt_entries, "SparseTablePush", nullptr));
     bool vec = (grad_dim % 4 == 0);
     for (int s = 0; s < N; s++) {
-        if (grad_rows[s] < 0 || (grad_rows[s] > 0 && !grads[s]) || (value_lens[s] > 0 && !feature_labels[s]))
+        const int64_t rows = pooled ? batch : grad_rows[s];
+        if (rows < 0 || (rows > 0 && !grads[s]) || (value_lens[s] > 0 && !feature_labels[s]) ||
+            (pooled && value_lens[s] > 0 && !example_ids[s]))
             return fail(TN_ERR_INVALID_ARGUMENT,
                         "sparse push grad must Matrix(sign_id_cnt, dim), slot " + std::to_string(s));
         descs[s].grads = grads[s];
-        descs[s].rows = grad_rows[s];
+        descs[s].rows = rows;
         descs[s].labels = feature_labels[s];
+        if (pooled) descs[s].mapped = const_cast<int64_t*>(example_ids[s]);  // example index of every lookup
         vec = vec && aligned16(grads[s]);
     }
     t->last_stream = st;
@@ -1152,6 +1172,49 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         }
         return TN_OK;
     };
+    // Where the apply kernels find the gradient of a record.  Pooled gradients are first reduced
+    // to one row per distinct sign: stable sort of (distinct index, position) pairs, then one
+    // ordered sum per distinct index.
+    PushSrc src = op_source(p, grad_dim);
+    auto prepare_src = [&]() -> int {
+        src = op_source(p, grad_dim);
+        if (!pooled) return TN_OK;
+        int bits = 1;
+        while (bits < 32 && (1ull << bits) < L) bits++;
+        size_t temp_bytes = 0;
+        TN_TRY(sort_pairs_temp_bytes(L, bits, &temp_bytes));
+        Carver c{nullptr};
+        auto carve = [&](Carver& cv, uint32_t*& keys, uint32_t*& vals, uint32_t*& skeys, uint32_t*& svals,
+                         uint32_t*& nlook, uint32_t*& seg_off, float*& flat, char*& temp) {
+            keys = cv.take<uint32_t>(L);
+            vals = cv.take<uint32_t>(L);
+            skeys = cv.take<uint32_t>(L);
+            svals = cv.take<uint32_t>(L);
+            nlook = cv.take<uint32_t>(L);
+            seg_off = cv.take<uint32_t>(L + 1);
+            flat = cv.take<float>(L * (size_t)grad_dim);
+            temp = cv.take<char>(temp_bytes);
+        };
+        uint32_t *keys, *vals, *skeys, *svals, *nlook, *seg_off;
+        float* flat;
+        char* temp;
+        carve(c, keys, vals, skeys, svals, nlook, seg_off, flat, temp);
+        TN_TRY(t->pooled_ws.ensure(align_up(c.off, 256)));
+        Carver c2{(char*)t->pooled_ws.p};
+        carve(c2, keys, vals, skeys, svals, nlook, seg_off, flat, temp);
+        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, batch,
+                  combiner, keys, vals, nlook, ds);
+        TN_TRY(sort_pairs_u32(temp, temp_bytes, keys, skeys, vals, svals, L, bits, st));
+        TN_LAUNCH(k_segment_starts, dim3(lblocks), dim3(256), st, skeys, (uint32_t)L, ds, seg_off);
+        if (vec)
+            TN_LAUNCH((k_reduce_pooled<4>), dim3(launch_grid((int64_t)L * (grad_dim / 4), 256, GRID_CAP * 4)), dim3(256),
+                      st, p.descs, p.lbase, N, grad_dim, batch, combiner, ds, seg_off, svals, nlook, flat);
+        else
+            TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * grad_dim, 256, GRID_CAP * 4)), dim3(256), st,
+                      p.descs, p.lbase, N, grad_dim, batch, combiner, ds, seg_off, svals, nlook, flat);
+        src.flat = flat;
+        return TN_OK;
+    };
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_REUSE_PLAN));
@@ -1169,7 +1232,8 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
                       p.where_u, p.list);
         else
             TN_TRY(launch_counts(t->plan_has_show));
-        TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
+        TN_TRY(prepare_src());
+        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
@@ -1184,13 +1248,113 @@ int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* 
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st));
         TN_TRY(launch_counts(false));
-        TN_TRY(launch_apply(t, p, op_source(p, grad_dim), ds, (int64_t)L, vec, st));
+        TN_TRY(prepare_src());
+        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
     }
     TN_HIP(hipGetLastError());
     TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush),
               (unsigned long long*)nullptr);
     t->push_pending = true;
     t->push_slots = N;
+    return TN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
+                            const float* const* grads, const int64_t* grad_rows, int grad_dim,
+                            const int64_t* const* feature_labels, void* stream) {
+    return push_op_impl(table_handle, N, values, value_lens, grads, grad_rows, grad_dim, feature_labels, nullptr, 0, 0,
+                        stream);
+}
+
+int tn_sparse_table_push_pooled_op(uint32_t table_handle, int N, const int64_t* const* values,
+                                   const int64_t* value_lens, const int64_t* const* example_ids,
+                                   const float* const* pooled_grads, int64_t batch, int grad_dim, int combiner,
+                                   const int64_t* const* feature_labels, void* stream) {
+    if (!example_ids) return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush (pooled): NULL argument");
+    return push_op_impl(table_handle, N, values, value_lens, pooled_grads, nullptr, grad_dim, feature_labels, example_ids,
+                        batch, combiner, stream);
+}
+
+int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* const* mapped_values,
+                               const int64_t* value_lens, const int64_t* const* example_ids, const float* const* vars,
+                               const int64_t* var_rows, int dim, int64_t batch, int combiner, float* const* out,
+                               void* stream) {
+    SparseTable* t = get_table(table_handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "embedding combine: bad table handle " + std::to_string(table_handle));
+    if (!mapped_values || !value_lens || !example_ids || !vars || !var_rows || !out || N <= 0)
+        return fail(TN_ERR_INVALID_ARGUMENT, "embedding combine: NULL argument");
+    if (N > MAX_SLOTS) return fail(TN_ERR_UNSUPPORTED, "embedding combine: too many slots");
+    if (dim <= 0 || batch <= 0 || combiner < COMBINE_SUM || combiner > COMBINE_SQRTN)
+        return fail(TN_ERR_INVALID_ARGUMENT, "embedding combine: bad dim, batch size or combiner");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    std::vector<SlotDesc> descs(N, SlotDesc{});
+    std::vector<uint32_t> lbase(N + 1, 0);
+    size_t L = 0;
+    bool vec = dim % 4 == 0;
+    for (int s = 0; s < N; s++) {
+        if (value_lens[s] < 0 || var_rows[s] < 0 || !out[s] ||
+            (value_lens[s] > 0 && (!mapped_values[s] || !example_ids[s] || !vars[s])))
+            return fail(TN_ERR_INVALID_ARGUMENT, "embedding combine: bad tensors of slot " + std::to_string(s));
+        SlotDesc& d = descs[s];
+        d.values = mapped_values[s];
+        d.mapped = const_cast<int64_t*>(example_ids[s]);
+        d.grads = vars[s];
+        d.var = out[s];
+        d.rows = var_rows[s];
+        d.len = (uint32_t)value_lens[s];
+        d.lbase = (uint32_t)L;
+        lbase[s] = (uint32_t)L;
+        L += (size_t)value_lens[s];
+        if (L > 0x7FFFFFF0ull) return fail(TN_ERR_UNSUPPORTED, "embedding combine: more than 2^31 lookups in one call");
+        vec = vec && aligned16(vars[s]) && aligned16(out[s]);
+    }
+    lbase[N] = (uint32_t)L;
+    // an earlier call's status is collected first: this call uses the table's status block
+    if (t->push_pending || t->pull_pending) {
+        if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    t->last_stream = st;
+    for (int s = 0; s < N; s++)
+        if (value_lens[s] == 0)  // no lookups: every example of the slot gets zeros
+            TN_LAUNCH(k_zero_f32, dim3(launch_grid(batch * dim, 256, GRID_CAP)), dim3(256), st, out[s], batch * dim);
+    if (L > 0) {
+        const size_t db = (size_t)N * sizeof(SlotDesc), lb = (size_t)(N + 1) * sizeof(uint32_t);
+        TN_TRY(t->comb_buf.ensure(align_up(db, 256) + lb));
+        SlotDesc* ddescs = (SlotDesc*)t->comb_buf.p;
+        uint32_t* dlbase = (uint32_t*)((char*)t->comb_buf.p + align_up(db, 256));
+        if (t->stage_pending) {
+            TN_HIP(hipEventSynchronize(t->stage_ev));
+            t->stage_pending = false;
+        }
+        std::memcpy(t->hstage, descs.data(), db);
+        std::memcpy(t->hstage + db, lbase.data(), lb);
+        TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)(db + lb) / 4, 256, 64)), dim3(256), st,
+                  reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(ddescs), (uint32_t)(db / 4),
+                  dlbase, (uint32_t)(lb / 4), t->dstatus, (int)STATUS_NEW_PLAN, (uint32_t*)nullptr, 0u);
+        TN_HIP(hipEventRecord(t->stage_ev, st));
+        t->stage_pending = true;
+        if (vec)
+            TN_LAUNCH((k_combine_fwd<4>), dim3(launch_grid((int64_t)L * (dim / 4), 256, GRID_CAP * 4)), dim3(256), st,
+                      ddescs, dlbase, N, (uint32_t)L, dim, batch, combiner, t->dstatus);
+        else
+            TN_LAUNCH((k_combine_fwd<1>), dim3(launch_grid((int64_t)L * dim, 256, GRID_CAP * 4)), dim3(256), st, ddescs,
+                      dlbase, N, (uint32_t)L, dim, batch, combiner, t->dstatus);
+    }
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipStreamSynchronize(st));
+    const uint32_t err = t->hpull->st.err;
+    if (err & DEV_ERR_VAR_CAPACITY) return fail(TN_ERR_VAR_CAPACITY, "embedding combine: a mapped id is not a row of its variable");
+    if (err & DEV_ERR_GRAD_ROWS)
+        return fail(TN_ERR_INVALID_ARGUMENT, "embedding combine: example ids must be non-decreasing and in [0, batch)");
     return TN_OK;
 }
 

@@ -132,6 +132,95 @@ def sparse_table_push(values, grads, feature_labels, table_handle):
     BoundSparseTablePush(values, grads, feature_labels, table_handle)()
 
 
+COMBINERS = {"sum": 0, "mean": 1, "sqrtn": 2}
+
+
+def _combiner(combiner):
+    if combiner not in COMBINERS:
+        raise ValueError("combiner must be one of 'sum', 'mean', 'sqrtn', got %r" % (combiner,))
+    return COMBINERS[combiner]
+
+
+def embedding_lookup_sparse(resources, mapped_values, example_ids, batch_size, table_handle, combiner="mean"):
+    """What TensorFlow does with the pull's results for every slot
+    (tf.nn.embedding_lookup_sparse behind embedding_column.get_dense_tensor,
+    tensornet/layers/embedding_features.py:278-280): out[s][b] = combiner over
+    the rows resources[s][mapped_values[s][i]] of the lookups i of example b.
+    example_ids[s][i] is the example of lookup i (SparseTensor.indices[:, 0]).
+    Returns N float32 tensors [batch_size, dim]."""
+    n = len(mapped_values)
+    if len(resources) != n or len(example_ids) != n or n == 0:
+        raise ValueError("embedding_lookup_sparse needs one variable, id tensor and example-id tensor per slot")
+    for i in range(n):
+        _require(resources[i], torch.float32, "resources[%d]" % i)
+        _require(mapped_values[i], torch.int64, "mapped_values[%d]" % i)
+        _require(example_ids[i], torch.int64, "example_ids[%d]" % i)
+        if example_ids[i].numel() != mapped_values[i].numel():
+            raise ValueError("example_ids[%d] must have one entry per lookup" % i)
+    dim = resources[0].shape[1]
+    flat = torch.empty((n, batch_size, dim), dtype=torch.float32, device=resources[0].device)
+    out = list(flat.unbind(0))
+    rc = _lib.load().tn_sparse_table_combine_op(
+        table_handle,
+        n,
+        _lib.ptr_array([v.data_ptr() for v in mapped_values]),
+        _lib.i64_array([v.numel() for v in mapped_values]),
+        _lib.ptr_array([e.data_ptr() for e in example_ids]),
+        _lib.ptr_array([r.data_ptr() for r in resources]),
+        _lib.i64_array([r.shape[0] for r in resources]),
+        int(dim),
+        int(batch_size),
+        _combiner(combiner),
+        _lib.ptr_array([o.data_ptr() for o in out]),
+        _stream(),
+    )
+    _lib.check(rc)
+    return out
+
+
+class BoundSparseTablePushPooled:
+    """SparseTablePush fed with the gradients of the combiner's outputs
+    (pooled_grads[s]: [batch_size, dim]) instead of per-distinct-sign rows; the
+    reduction TensorFlow performs in between (gradient of embedding_lookup_sparse
+    summed per distinct id) runs on the device.  Bound to fixed tensors like
+    BoundSparseTablePush."""
+
+    def __init__(self, values, example_ids, pooled_grads, feature_labels, table_handle, combiner="mean"):
+        n = len(values)
+        if len(example_ids) != n or len(pooled_grads) != n or len(feature_labels) != n or n == 0:
+            raise ValueError("SparseTable push (pooled) needs values, example ids, gradients and labels per slot")
+        for i in range(n):
+            _require(values[i], torch.int64, "values[%d]" % i)
+            _require(example_ids[i], torch.int64, "example_ids[%d]" % i)
+            _require(pooled_grads[i], torch.float32, "pooled_grads[%d]" % i)
+            _require(feature_labels[i], torch.int64, "feature_labels[%d]" % i)
+            if pooled_grads[i].dim() != 2 or pooled_grads[i].shape != pooled_grads[0].shape:
+                raise ValueError("pooled_grads must all be Matrix(batch_size, dim)")
+            if example_ids[i].numel() != values[i].numel() or feature_labels[i].numel() != values[i].numel():
+                raise ValueError("example_ids / feature_labels of slot %d must have one entry per lookup" % i)
+        self._keep = (list(values), list(example_ids), list(pooled_grads), list(feature_labels))
+        self._fn = _lib.load().tn_sparse_table_push_pooled_op
+        self._args = (
+            table_handle,
+            n,
+            _lib.ptr_array([v.data_ptr() for v in values]),
+            _lib.i64_array([v.numel() for v in values]),
+            _lib.ptr_array([e.data_ptr() for e in example_ids]),
+            _lib.ptr_array([g.data_ptr() for g in pooled_grads]),
+            int(pooled_grads[0].shape[0]),
+            int(pooled_grads[0].shape[1]),
+            _combiner(combiner),
+            _lib.ptr_array([l.data_ptr() for l in feature_labels]),
+        )
+
+    def __call__(self):
+        _lib.check(self._fn(*self._args, _stream()))
+
+
+def sparse_table_push_pooled(values, example_ids, pooled_grads, feature_labels, table_handle, combiner="mean"):
+    BoundSparseTablePushPooled(values, example_ids, pooled_grads, feature_labels, table_handle, combiner)()
+
+
 def sparse_table_sync(table_handle):
     """Waits for enqueued pushes of the table and raises their latched error."""
     _lib.check(_lib.load().tn_sparse_table_sync(table_handle))
