@@ -191,6 +191,7 @@ def main():
     ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated batches cycled through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
+    ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -295,12 +296,12 @@ def main():
     per_step = {k: (c / psteps, ms / psteps) for k, (c, ms) in prof.items()}
     kernel_ms = sum(ms for _, ms in per_step.values())
     # the dominant kernel of the step's critical path
-    dominant = max((kv for kv in per_step.items() if not kv[0].startswith(SIDE_STREAM_KERNELS)),
-                   key=lambda kv: kv[1][1])
+    mean_shape = {k: sum(sh[k] for sh in shapes) / len(shapes) for k in shapes[0]}
+    dominant = max((kv for kv in per_step.items() if not kv[0].startswith(SIDE_STREAM_KERNELS)
+                    and kernel_algorithmic_bytes(kv[0], opt_name, dim, mean_shape) > 0), key=lambda kv: kv[1][1])
     dname, (dcount, dms) = dominant
     avg_launch_s = dms / dcount * 1e-3
     mean_L, mean_U = total_L / args.steps, total_U / args.steps
-    mean_shape = {k: sum(sh[k] for sh in shapes) / len(shapes) for k in shapes[0]}
     dbytes = kernel_algorithmic_bytes(dname, opt_name, dim, mean_shape)
     achieved = dbytes / avg_launch_s
     for k, (c, ms) in sorted(per_step.items(), key=lambda kv: -kv[1][1]):
@@ -350,6 +351,65 @@ def main():
         "side_stream_kernels": [k for k in per_step if k.startswith(SIDE_STREAM_KERNELS)],
         "batch_shape": mean_shape,
     }
+
+    # ---- side measurement: the combiner around the ops on the device ---------------
+    # pull -> embedding_lookup_sparse (mean) -> push of the pooled gradients, same batches
+    if not args.no_combiner:
+        crng = np.random.default_rng(0)
+        cb = []
+        for values, labels, grads, vars_ in batches:
+            ex = [torch.from_numpy(np.sort(crng.integers(0, cfg["batch"], v.numel()))).cuda() for v in values]
+            pooled = [torch.randn((cfg["batch"], dim), device="cuda", generator=rng) * cfg["grad_sigma"] for _ in values]
+            pull = tn.ops.BoundSparseTablePull(vars_, values, h)
+            push = tn.ops.BoundSparseTablePushPooled(values, ex, pooled, labels, h, "mean")
+            cb.append((pull, push, vars_, ex))
+
+        def cstep(i):
+            pull, push, vars_, ex = cb[i % nb]
+            mapped = pull()
+            tn.ops.embedding_lookup_sparse(vars_, mapped, ex, cfg["batch"], h, "mean")
+            push()
+
+        for i in range(2):
+            cstep(i)
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        csteps = min(args.steps, 10)
+        t0 = time.perf_counter()
+        for i in range(csteps):
+            cstep(i)
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        cms = (time.perf_counter() - t0) * 1e3 / csteps
+        lib.tn_profile_reset()
+        lib.tn_profile_enable(1)
+        for i in range(csteps):
+            cstep(i)
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        lib.tn_profile_enable(0)
+        cprof = {k: ms / csteps for k, (c, ms) in _lib.profile_summary().items()}
+        lib.tn_profile_reset()
+        comb_bytes = {
+            # signs' ids + example ids in, one output row per (slot, example) out, variable rows read once
+            "k_combine_fwd": 16 * mean_L + 4 * dim * (cfg["batch"] * n_slots + mean_U),
+            # example ids + distinct index in, sort key + value out
+            "k_lookup_keys": 24 * mean_L,
+            # sorted values in, pooled rows read once, one reduced row per distinct sign out
+            "k_reduce_pooled": 8 * mean_L + 4 * dim * (cfg["batch"] * n_slots + mean_U),
+        }
+        out["combiner_step"] = {
+            "what": "pull + embedding_lookup_sparse(mean) + push of pooled gradients, same workload",
+            "ms_per_step": cms,
+            "keys_per_s": mean_L / (cms * 1e-3),
+            "kernels_ms_per_step": {k: round(v, 4) for k, v in cprof.items()
+                                    if k.startswith(("k_combine", "k_example", "k_lookup_keys", "k_segment", "k_reduce"))},
+            "kernels_frac_of_hbm_peak": {k: round(comb_bytes[k.split("<")[0]] / (v * 1e-3) / HBM_PEAK, 4)
+                                         for k, v in cprof.items() if k.split("<")[0] in comb_bytes},
+            "note": "the stable radix sort between k_lookup_keys and k_segment_starts is rocPRIM's; its time is "
+                    "in ms_per_step only",
+        }
+        log("combiner step: %.3f ms/step; %s" % (cms, out["combiner_step"]["kernels_ms_per_step"]))
 
     # ---- dense Adam side measurement (cfg5's flat array) --------------------------
     if not args.no_dense:

@@ -19,6 +19,7 @@
 namespace tn {
 
 enum { COMBINE_SUM = 0, COMBINE_MEAN = 1, COMBINE_SQRTN = 2 };
+constexpr int COMBINE_WINDOW = 8;  // lookups of an example / of a distinct sign read ahead with independent loads
 
 // In these kernels a SlotDesc carries: values = mapped ids (forward) / signs (backward),
 // mapped = example index of every lookup, grads = rows to read (variable / pooled gradient),
@@ -30,21 +31,16 @@ __device__ __forceinline__ float combine_divisor(uint32_t n, int combiner) {
     return combiner == COMBINE_MEAN ? (float)n : sqrtf((float)n);
 }
 
-// One group of `chunks` threads per lookup; the group of the first lookup of an example
-// sums the example's rows, divides, writes the output row, and clears the rows of the
-// examples without lookups before it (after it, for the slot's last example).
-template <int VEC>
-__global__ __launch_bounds__(256) void k_combine_fwd(const SlotDesc* __restrict__ descs,
-                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L, int dim,
-                                                     int64_t batch, int combiner, DevStatus* status) {
+// Forward, step 1: where the lookups of every example start (rowptr[s * (batch + 1) + b], with
+// rowptr[.. + batch] = lookups of the slot), from the sorted example ids; also checks them.
+__global__ __launch_bounds__(256) void k_example_rowptr(const SlotDesc* __restrict__ descs,
+                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                        int64_t batch, uint32_t* __restrict__ rowptr,
+                                                        DevStatus* status) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
-    const int chunks = dim / VEC;
-    const int64_t total = (int64_t)L * chunks;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
-        const uint32_t gi = (uint32_t)(t / chunks);
-        const int c = (int)(t - (int64_t)gi * chunks);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
         const SlotDesc& d = descs[sl];
         const int64_t* ex = example_of(d);
@@ -52,50 +48,77 @@ __global__ __launch_bounds__(256) void k_combine_fwd(const SlotDesc* __restrict_
         const int64_t b = ex[i];
         const int64_t prev = i > 0 ? ex[i - 1] : -1;
         if (b < 0 || b >= batch || prev > b) {
-            if (c == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+            atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
             continue;
         }
-        if (prev == b) continue;  // not the first lookup of its example
+        uint32_t* rp = rowptr + (size_t)sl * (batch + 1);
+        for (int64_t r = prev + 1; r <= b; r++) rp[r] = i;  // example b starts here; the ones skipped are empty
+        if (i == d.len - 1)
+            for (int64_t r = b + 1; r <= batch; r++) rp[r] = d.len;
+    }
+}
+
+// Forward, step 2: one group of `chunks` threads per (slot, example) sums the rows of the example's
+// lookups in order, divides, and writes the output row (zeros for an example without lookups).
+template <int VEC>
+__global__ __launch_bounds__(256) void k_combine_fwd(const SlotDesc* __restrict__ descs, int N, int dim, int64_t batch,
+                                                     int combiner, const uint32_t* __restrict__ rowptr,
+                                                     DevStatus* status) {
+    const int chunks = dim / VEC;
+    const int64_t per_slot = batch * chunks;
+    const int64_t total = (int64_t)N * per_slot;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const int sl = (int)(t / per_slot);
+        const int64_t rest = t - (int64_t)sl * per_slot;
+        const int64_t b = rest / chunks;
+        const int c = (int)(rest - b * chunks);
+        const SlotDesc& d = descs[sl];
+        const uint32_t* rp = rowptr + (size_t)sl * (batch + 1);
+        const uint32_t lo = d.len ? rp[b] : 0, hi = d.len ? rp[b + 1] : 0;
+        const int64_t* ids = d.values;
+        const float* rows = d.grads;
+        const int64_t nrows = d.rows;
         float acc[VEC];
 #pragma unroll
         for (int q = 0; q < VEC; q++) acc[q] = 0.f;
-        uint32_t j = i;
-        for (; j < d.len && ex[j] == b; j++) {
-            const int64_t id = d.values[j];
-            if (id < 0 || id >= d.rows) {
-                if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
-                continue;
-            }
-            const float* row = d.grads + id * dim + c * VEC;
-            if (VEC == 4) {
-                const float4 v = *reinterpret_cast<const float4*>(row);
-                acc[0] += v.x;
-                acc[1] += v.y;
-                acc[2] += v.z;
-                acc[3] += v.w;
-            } else {
-                acc[0] += row[0];
-            }
-        }
-        const float div = combine_divisor(j - i, combiner);
-        float* out = d.var;
-        auto put = [&](int64_t r, const float* v) {
-            float* o = out + r * dim + c * VEC;
-            if (VEC == 4)
-                *reinterpret_cast<float4*>(o) = make_float4(v[0], v[1], v[2], v[3]);
-            else
-                o[0] = v[0];
-        };
-        float zero[VEC];
+        bool bad_id = false;
+        // windows of COMBINE_WINDOW lookups: ids first, then their rows, all loads independent;
+        // the additions run in lookup order
+        for (uint32_t j0 = lo; j0 < hi; j0 += COMBINE_WINDOW) {
+            int64_t wid[COMBINE_WINDOW];
 #pragma unroll
-        for (int q = 0; q < VEC; q++) {
-            zero[q] = 0.f;
-            acc[q] = acc[q] / div;
+            for (int q = 0; q < COMBINE_WINDOW; q++) wid[q] = (j0 + q < hi) ? ids[j0 + q] : -1;
+            float wr[COMBINE_WINDOW][VEC];
+#pragma unroll
+            for (int q = 0; q < COMBINE_WINDOW; q++) {
+                const bool in = j0 + q < hi;
+                const bool ok = in && wid[q] >= 0 && wid[q] < nrows;
+                if (in && !ok) bad_id = true;
+                const float* row = rows + (ok ? wid[q] : 0) * dim + c * VEC;
+                if (VEC == 4) {
+                    const float4 v = ok ? *reinterpret_cast<const float4*>(row) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    wr[q][0] = v.x;
+                    wr[q][1 % VEC] = v.y;
+                    wr[q][2 % VEC] = v.z;
+                    wr[q][3 % VEC] = v.w;
+                } else {
+                    wr[q][0] = ok ? row[0] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < COMBINE_WINDOW; q++)
+                if (j0 + q < hi)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] += wr[q][v];
         }
-        put(b, acc);
-        for (int64_t r = prev + 1; r < b; r++) put(r, zero);
-        if (j == d.len)
-            for (int64_t r = b + 1; r < batch; r++) put(r, zero);
+        if (bad_id && c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
+        const float div = combine_divisor(hi - lo, combiner);
+        float* o = d.var + b * dim + c * VEC;
+        if (VEC == 4)
+            *reinterpret_cast<float4*>(o) = make_float4(acc[0] / div, acc[1 % VEC] / div, acc[2 % VEC] / div, acc[3 % VEC] / div);
+        else
+            o[0] = acc[0] / div;
     }
 }
 
@@ -105,30 +128,37 @@ __global__ __launch_bounds__(256) void k_zero_f32(float* __restrict__ out, int64
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = 0.f;
 }
 
-// Backward, step 1: sort keys (distinct index of every lookup) and values (its position);
-// with a mean / sqrtn combiner also the number of lookups of the lookup's example.
+// Backward, step 1: sort keys (distinct index of every lookup) and values: the lookup's
+// example in the high word, the number of lookups of that example in the low word -- all the
+// reduction needs to know about the lookup, so that it reads them in sorted order instead of
+// chasing positions.  The first lookup of an example writes the values of all its lookups.
 __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     const uint32_t* __restrict__ u_of_gi, int64_t batch, int combiner,
-                                                     uint32_t* __restrict__ keys, uint32_t* __restrict__ vals,
-                                                     uint32_t* __restrict__ nlook, DevStatus* status) {
+                                                     const uint32_t* __restrict__ u_of_gi, int64_t batch,
+                                                     uint32_t* __restrict__ keys, uint64_t* __restrict__ vals,
+                                                     DevStatus* status, uint32_t* long_count) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *long_count = 0;  // list of the frequent signs, filled by k_reduce_pooled
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         keys[gi] = u_of_gi[gi] & ~FIRST_BIT;
-        vals[gi] = gi;
         const int sl = find_slot(lb, N, gi);
         const SlotDesc& d = descs[sl];
         const int64_t* ex = example_of(d);
         const uint32_t i = gi - lb[sl];
         const int64_t b = ex[i];
         const int64_t prev = i > 0 ? ex[i - 1] : -1;
-        if (b < 0 || b >= batch || prev > b) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-        if (combiner == COMBINE_SUM || prev == b) continue;
+        if (b < 0 || b >= batch || prev > b) {
+            atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+            vals[gi] = ~0ull;  // no share
+            continue;
+        }
+        if (prev == b) continue;
         uint32_t j = i;
         while (j < d.len && ex[j] == b) j++;
-        for (uint32_t q = i; q < j; q++) nlook[lb[sl] + q] = j - i;  // the example's first lookup tells the others
+        const uint64_t v = ((uint64_t)b << 32) | (uint64_t)(j - i);
+        for (uint32_t q = i; q < j; q++) vals[lb[sl] + q] = v;
     }
 }
 
@@ -143,17 +173,39 @@ __global__ __launch_bounds__(256) void k_segment_starts(const uint32_t* __restri
     }
 }
 
-// Step 3: one group of `chunks` threads per distinct index sums its lookups' share of the
-// pooled gradient rows, in position order.
+// The share of a lookup in the gradient of its distinct sign: its example's pooled row times
+// 1 / d(lookups of the example), chunk c.
+template <int VEC>
+__device__ __forceinline__ void add_lookup_share(const float* __restrict__ pooled, uint64_t v, int dim, int c,
+                                                 int combiner, float (&acc)[VEC]) {
+    if (v == ~0ull) return;  // flagged by k_lookup_keys
+    const uint32_t b = (uint32_t)(v >> 32);
+    const float scale = combiner == COMBINE_SUM ? 1.f : 1.f / combine_divisor((uint32_t)v, combiner);
+    const float* row = pooled + (uint64_t)b * dim + c * VEC;
+    if (VEC == 4) {
+        const float4 g = *reinterpret_cast<const float4*>(row);
+        acc[0] += g.x * scale;
+        acc[1] += g.y * scale;
+        acc[2] += g.z * scale;
+        acc[3] += g.w * scale;
+    } else {
+        acc[0] += row[0] * scale;
+    }
+}
+
+// Step 3: one group of `chunks` threads per distinct index sums its lookups' shares of the
+// pooled gradient rows, in position order.  A distinct index with long_min lookups or more (a
+// frequent sign) is only noted in long_list: one workgroup each sums those (k_reduce_long).
 template <int VEC>
 __global__ __launch_bounds__(256) void k_reduce_pooled(const SlotDesc* __restrict__ descs,
-                                                       const uint32_t* __restrict__ lbase, int N, int dim,
-                                                       int64_t batch, int combiner, const DevStatus* status,
+                                                       const uint32_t* __restrict__ ubase, int N, int dim,
+                                                       int combiner, const DevStatus* status,
                                                        const uint32_t* __restrict__ seg_off,
-                                                       const uint32_t* __restrict__ svals,
-                                                       const uint32_t* __restrict__ nlook, float* __restrict__ flat) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
-    load_lbase(lb, lbase, N);
+                                                       const uint64_t* __restrict__ svals, float* __restrict__ flat,
+                                                       uint32_t long_min, uint32_t* __restrict__ long_list,
+                                                       uint32_t* long_count) {
+    __shared__ uint32_t ub[MAX_SLOTS + 1];
+    load_lbase(ub, ubase, N);
     const int chunks = dim / VEC;
     const int64_t total = (int64_t)status->n_unique * chunks;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -161,35 +213,79 @@ __global__ __launch_bounds__(256) void k_reduce_pooled(const SlotDesc* __restric
         const uint32_t u = (uint32_t)(t / chunks);
         const int c = (int)(t - (int64_t)u * chunks);
         const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
+        if (hi - lo >= long_min) {
+            if (c == 0) long_list[atomicAdd(long_count, 1u)] = u;
+            continue;
+        }
         float acc[VEC];
 #pragma unroll
         for (int q = 0; q < VEC; q++) acc[q] = 0.f;
-        if (lo < hi) {
-            const int sl = find_slot(lb, N, svals[lo]);  // all lookups of a distinct index lie in one slot
-            const SlotDesc& d = descs[sl];
-            const int64_t* ex = example_of(d);
-            for (uint32_t j = lo; j < hi; j++) {
-                const uint32_t gi = svals[j];
-                const int64_t b = ex[gi - lb[sl]];
-                if (b < 0 || b >= batch) continue;  // flagged by k_lookup_keys
-                const float scale = combiner == COMBINE_SUM ? 1.f : 1.f / combine_divisor(nlook[gi], combiner);
-                const float* row = d.grads + b * dim + c * VEC;
-                if (VEC == 4) {
-                    const float4 v = *reinterpret_cast<const float4*>(row);
-                    acc[0] += v.x * scale;
-                    acc[1] += v.y * scale;
-                    acc[2] += v.z * scale;
-                    acc[3] += v.w * scale;
-                } else {
-                    acc[0] += row[0] * scale;
-                }
-            }
+        const float* pooled = descs[find_slot(ub, N, u)].grads;  // the slot whose window of distinct indices holds u
+        for (uint32_t j0 = lo; j0 < hi; j0 += COMBINE_WINDOW) {  // values of a window first, then their rows
+            uint64_t wv[COMBINE_WINDOW];
+#pragma unroll
+            for (int q = 0; q < COMBINE_WINDOW; q++) wv[q] = (j0 + q < hi) ? svals[j0 + q] : ~0ull;
+#pragma unroll
+            for (int q = 0; q < COMBINE_WINDOW; q++) add_lookup_share<VEC>(pooled, wv[q], dim, c, combiner, acc);
         }
         float* o = flat + (uint64_t)u * dim + c * VEC;
         if (VEC == 4)
             *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
         else
             o[0] = acc[0];
+    }
+}
+
+// One workgroup per frequent distinct index: its 256 / chunks thread groups each sum every
+// (256 / chunks)-th lookup in position order, then the partial sums are added in group order.
+// The order of the additions is fixed, so the result does not vary from run to run.
+constexpr int LONG_PART_FLOATS = 1024;  // 256 threads x 4 floats
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_reduce_long(const SlotDesc* __restrict__ descs,
+                                                     const uint32_t* __restrict__ ubase, int N, int dim, int combiner,
+                                                     const uint32_t* __restrict__ seg_off,
+                                                     const uint64_t* __restrict__ svals, float* __restrict__ flat,
+                                                     const uint32_t* __restrict__ long_list,
+                                                     const uint32_t* long_count) {
+    __shared__ float part[LONG_PART_FLOATS];
+    const int chunks = dim / VEC;
+    const int groups = 256 / chunks;
+    const int q = threadIdx.x / chunks, c = threadIdx.x - q * chunks;
+    const uint32_t n_long = *long_count;
+    for (uint32_t k = blockIdx.x; k < n_long; k += gridDim.x) {
+        const uint32_t u = long_list[k];
+        const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
+        const float* pooled = descs[find_slot(ubase, N, u)].grads;
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[v] = 0.f;
+        if (q < groups) {
+            for (uint32_t j0 = lo + q; j0 < hi; j0 += COMBINE_WINDOW * groups) {  // values of a window first, then their rows
+                uint64_t wv[COMBINE_WINDOW];
+#pragma unroll
+                for (int w = 0; w < COMBINE_WINDOW; w++) wv[w] = (j0 + w * groups < hi) ? svals[j0 + w * groups] : ~0ull;
+#pragma unroll
+                for (int w = 0; w < COMBINE_WINDOW; w++) add_lookup_share<VEC>(pooled, wv[w], dim, c, combiner, acc);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; v++) part[threadIdx.x * VEC + v] = acc[v];
+        __syncthreads();
+        if (q == 0) {
+            float sum[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; v++) sum[v] = 0.f;
+            for (int g = 0; g < groups; g++)
+#pragma unroll
+                for (int v = 0; v < VEC; v++) sum[v] += part[(g * chunks + c) * VEC + v];
+            float* o = flat + (uint64_t)u * dim + c * VEC;
+            if (VEC == 4)
+                *reinterpret_cast<float4*>(o) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+            else
+                o[0] = sum[0];
+        }
+        __syncthreads();
     }
 }
 

@@ -11,8 +11,8 @@ namespace tn {
 
 // sort_pairs.hip
 int sort_pairs_temp_bytes(size_t n, int key_bits, size_t* bytes);
-int sort_pairs_u32(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out, const uint32_t* vals_in,
-                   uint32_t* vals_out, size_t n, int key_bits, hipStream_t st);
+int sort_pairs_u32_u64(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
+                       const uint64_t* vals_in, uint64_t* vals_out, size_t n, int key_bits, hipStream_t st);
 
 namespace {
 
@@ -571,6 +571,7 @@ void launch_grouping(const Plan& p, const Scratch& w, const PushSrc& src, int64_
 }
 
 constexpr int MASK_SLOTS = 128;
+constexpr uint32_t LONG_SEGMENT = 64;  // lookups of one distinct sign from which a workgroup sums them
 
 
 // The same result for the distinct signs of an op with at most 128 slots, from slot masks.
@@ -1184,34 +1185,47 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         size_t temp_bytes = 0;
         TN_TRY(sort_pairs_temp_bytes(L, bits, &temp_bytes));
         Carver c{nullptr};
-        auto carve = [&](Carver& cv, uint32_t*& keys, uint32_t*& vals, uint32_t*& skeys, uint32_t*& svals,
-                         uint32_t*& nlook, uint32_t*& seg_off, float*& flat, char*& temp) {
+        uint32_t *long_list, *long_count, *keys, *skeys, *seg_off;
+        uint64_t *vals, *svals;
+        float* flat;
+        char* temp;
+        auto carve = [&](Carver& cv) {
+            long_count = cv.take<uint32_t>(1);
+            long_list = cv.take<uint32_t>(L / LONG_SEGMENT + 1);
             keys = cv.take<uint32_t>(L);
-            vals = cv.take<uint32_t>(L);
             skeys = cv.take<uint32_t>(L);
-            svals = cv.take<uint32_t>(L);
-            nlook = cv.take<uint32_t>(L);
+            vals = cv.take<uint64_t>(L);
+            svals = cv.take<uint64_t>(L);
             seg_off = cv.take<uint32_t>(L + 1);
             flat = cv.take<float>(L * (size_t)grad_dim);
             temp = cv.take<char>(temp_bytes);
         };
-        uint32_t *keys, *vals, *skeys, *svals, *nlook, *seg_off;
-        float* flat;
-        char* temp;
-        carve(c, keys, vals, skeys, svals, nlook, seg_off, flat, temp);
+        carve(c);
         TN_TRY(t->pooled_ws.ensure(align_up(c.off, 256)));
         Carver c2{(char*)t->pooled_ws.p};
-        carve(c2, keys, vals, skeys, svals, nlook, seg_off, flat, temp);
-        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, batch,
-                  combiner, keys, vals, nlook, ds);
-        TN_TRY(sort_pairs_u32(temp, temp_bytes, keys, skeys, vals, svals, L, bits, st));
+        carve(c2);
+        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, batch, keys,
+                  vals, ds, long_count);
+        TN_TRY(sort_pairs_u32_u64(temp, temp_bytes, keys, skeys, vals, svals, L, bits, st));
         TN_LAUNCH(k_segment_starts, dim3(lblocks), dim3(256), st, skeys, (uint32_t)L, ds, seg_off);
-        if (vec)
-            TN_LAUNCH((k_reduce_pooled<4>), dim3(launch_grid((int64_t)L * (grad_dim / 4), 256, GRID_CAP * 4)), dim3(256),
-                      st, p.descs, p.lbase, N, grad_dim, batch, combiner, ds, seg_off, svals, nlook, flat);
-        else
-            TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * grad_dim, 256, GRID_CAP * 4)), dim3(256), st,
-                      p.descs, p.lbase, N, grad_dim, batch, combiner, ds, seg_off, svals, nlook, flat);
+        // signs with LONG_SEGMENT lookups or more get a workgroup each instead of one thread group
+        const int chunks = vec ? grad_dim / 4 : grad_dim;
+        const uint32_t long_min = chunks <= 256 ? LONG_SEGMENT : 0xFFFFFFFFu;
+        const int long_blocks = launch_grid((int64_t)L / LONG_SEGMENT + 1, 1, GRID_CAP);
+        if (vec) {
+            TN_LAUNCH((k_reduce_pooled<4>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
+                      p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
+                      long_count);
+            TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim, combiner,
+                      seg_off, svals, flat, long_list, long_count);
+        } else {
+            TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
+                      p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
+                      long_count);
+            if (long_min != 0xFFFFFFFFu)
+                TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim,
+                          combiner, seg_off, svals, flat, long_list, long_count);
+        }
         src.flat = flat;
         return TN_OK;
     };
@@ -1322,14 +1336,13 @@ int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* cons
         harvest(t);
     }
     t->last_stream = st;
-    for (int s = 0; s < N; s++)
-        if (value_lens[s] == 0)  // no lookups: every example of the slot gets zeros
-            TN_LAUNCH(k_zero_f32, dim3(launch_grid(batch * dim, 256, GRID_CAP)), dim3(256), st, out[s], batch * dim);
-    if (L > 0) {
+    {
         const size_t db = (size_t)N * sizeof(SlotDesc), lb = (size_t)(N + 1) * sizeof(uint32_t);
-        TN_TRY(t->comb_buf.ensure(align_up(db, 256) + lb));
+        const size_t rp = (size_t)N * (size_t)(batch + 1) * sizeof(uint32_t);
+        TN_TRY(t->comb_buf.ensure(align_up(db, 256) + align_up(lb, 256) + rp));
         SlotDesc* ddescs = (SlotDesc*)t->comb_buf.p;
         uint32_t* dlbase = (uint32_t*)((char*)t->comb_buf.p + align_up(db, 256));
+        uint32_t* rowptr = (uint32_t*)((char*)dlbase + align_up(lb, 256));
         if (t->stage_pending) {
             TN_HIP(hipEventSynchronize(t->stage_ev));
             t->stage_pending = false;
@@ -1341,12 +1354,16 @@ int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* cons
                   dlbase, (uint32_t)(lb / 4), t->dstatus, (int)STATUS_NEW_PLAN, (uint32_t*)nullptr, 0u);
         TN_HIP(hipEventRecord(t->stage_ev, st));
         t->stage_pending = true;
+        // where the lookups of every example start, then one thread group per (slot, example)
+        if (L > 0)
+            TN_LAUNCH(k_example_rowptr, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, ddescs, dlbase, N,
+                      (uint32_t)L, batch, rowptr, t->dstatus);
         if (vec)
-            TN_LAUNCH((k_combine_fwd<4>), dim3(launch_grid((int64_t)L * (dim / 4), 256, GRID_CAP * 4)), dim3(256), st,
-                      ddescs, dlbase, N, (uint32_t)L, dim, batch, combiner, t->dstatus);
+            TN_LAUNCH((k_combine_fwd<4>), dim3(launch_grid((int64_t)N * batch * (dim / 4), 256, GRID_CAP * 4)), dim3(256),
+                      st, ddescs, N, dim, batch, combiner, rowptr, t->dstatus);
         else
-            TN_LAUNCH((k_combine_fwd<1>), dim3(launch_grid((int64_t)L * dim, 256, GRID_CAP * 4)), dim3(256), st, ddescs,
-                      dlbase, N, (uint32_t)L, dim, batch, combiner, t->dstatus);
+            TN_LAUNCH((k_combine_fwd<1>), dim3(launch_grid((int64_t)N * batch * dim, 256, GRID_CAP * 4)), dim3(256), st,
+                      ddescs, N, dim, batch, combiner, rowptr, t->dstatus);
     }
     TN_HIP(hipGetLastError());
     TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
