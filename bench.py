@@ -192,6 +192,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
     ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
+    ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -410,6 +411,29 @@ def main():
                     "in ms_per_step only",
         }
         log("combiner step: %.3f ms/step; %s" % (cms, out["combiner_step"]["kernels_ms_per_step"]))
+
+    # ---- side measurement: ShowDecay, one streaming pass over the whole table -------
+    if not args.no_decay:
+        cap = tn.core.sparse_table_capacity(h)
+        keys_now = tn.core.sparse_table_key_count(h)
+        tn.core.show_decay(h, 1)
+        torch.cuda.synchronize()
+        d0 = torch.cuda.Event(enable_timing=True)
+        d1 = torch.cuda.Event(enable_timing=True)
+        d0.record()
+        for _ in range(3):
+            tn.core.show_decay(h, 1)
+        d1.record()
+        torch.cuda.synchronize()
+        dms = d0.elapsed_time(d1) / 3
+        # every slot's key is read; a resident row's state (16 B for AdaGrad) is read and written
+        dbytes_decay = 8 * cap + 32 * keys_now
+        out["show_decay"] = {
+            "slots": cap, "resident_keys": keys_now, "ms": dms,
+            "algorithmic_GBps": dbytes_decay / (dms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": dbytes_decay / (dms * 1e-3) / HBM_PEAK,
+        }
+        log("show_decay over %d slots: %.2f ms" % (cap, dms))
 
     # ---- dense Adam side measurement (cfg5's flat array) --------------------------
     if not args.no_dense:

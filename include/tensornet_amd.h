@@ -263,6 +263,25 @@ int tn_sparse_table_push_pooled_op(uint32_t table_handle, int N, const int64_t* 
                                    const float* const* pooled_grads, int64_t batch, int grad_dim, int combiner,
                                    const int64_t* const* feature_labels, void* stream);
 
+/*
+ * SparseTable::ShowDecay (core/ps/table/sparse_table.h:59, sparse_table.cc:139,
+ * bound to Python as tn.core.show_decay, core/main/py_wrapper.cc:259-262): every
+ * resident row ages by delta_days -- AdaGrad: show and click times
+ * show_decay_rate, no_show_days += delta_days (ada_grad_kernel.cc:191-195);
+ * Ftrl: show times show_decay_rate (ftrl_kernel.cc:124); Adam: nothing
+ * (adam_kernel.h:67).  One streaming pass over the table, enqueued on `stream`.
+ */
+int tn_sparse_table_show_decay(uint32_t handle, int delta_days, void* stream);
+
+/*
+ * Value::DeleteByShow (ada_grad_kernel.cc:197-204, ftrl_kernel.cc:126,
+ * adam_kernel.h:69), the feature-elimination test the reference applies to every
+ * row when it saves a table (optimizer_kernel.h:332,345): out[i] (device) = 1 if
+ * the row of signs[i] (device) would be left out, 0 if it is kept or absent.
+ * Returns after the stream work has completed.
+ */
+int tn_sparse_table_delete_by_show(uint32_t handle, const uint64_t* signs, int64_t n, uint8_t* out, void* stream);
+
 /* Wait for the table's enqueued work and return (and clear) its latched error. */
 int tn_sparse_table_sync(uint32_t handle);
 

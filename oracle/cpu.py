@@ -38,6 +38,10 @@ def load():
     lib.orc_table_state_floats.argtypes = [P]
     lib.orc_table_key_count.restype = C.c_uint64
     lib.orc_table_key_count.argtypes = [P]
+    lib.orc_table_show_decay.restype = None
+    lib.orc_table_show_decay.argtypes = [P, C.c_int]
+    lib.orc_table_delete_by_show.restype = None
+    lib.orc_table_delete_by_show.argtypes = [P, P, C.c_int64, P]
     lib.orc_table_set_rows.argtypes = [P, P, P, P, C.c_int64]
     lib.orc_table_get_rows.argtypes = [P, P, C.c_int64, P, P, P]
     lib.orc_table_pull.argtypes = [P, P, C.c_int64, C.c_int, P]
@@ -98,7 +102,13 @@ def _params(kind, **kw):
             kw.get("lambda2", 1.0),
             kw.get("initial_scale", 1.0),
         ]
-    return np.asarray(vals + [0.0] * (8 - len(vals)), dtype=np.float32)
+    tail = [
+        kw.get("show_decay_rate", 0.98),
+        kw.get("show_threshold", 0.0),
+        float(kw.get("no_show_days", 1000)),
+        float(kw.get("elimination_logic", 0)),
+    ]
+    return np.asarray(vals + [0.0] * (8 - len(vals)) + tail, dtype=np.float32)
 
 
 def pull_remap(values):
@@ -139,6 +149,15 @@ class Table(object):
 
     def key_count(self):
         return int(load().orc_table_key_count(self._h))
+
+    def show_decay(self, delta_days):
+        load().orc_table_show_decay(self._h, int(delta_days))
+
+    def delete_by_show(self, signs):
+        signs = np.ascontiguousarray(signs, dtype=np.uint64)
+        out = np.zeros(len(signs), dtype=np.uint8)
+        load().orc_table_delete_by_show(self._h, _p(signs), len(signs), _p(out))
+        return out.astype(bool)
 
     def set_rows(self, signs, w, state=None):
         signs = np.ascontiguousarray(signs, dtype=np.uint64)

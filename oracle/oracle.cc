@@ -297,6 +297,34 @@ public:
         return missing;
     }
 
+    // SparseOptimizerKernel::ShowDecay -> SparseKernelBlock::ShowDecay (optimizer_kernel.h:422-427,549-553):
+    // every resident row; AdaGrad ada_grad_kernel.cc:191-195, Ftrl ftrl_kernel.cc:124, Adam adam_kernel.h:67 (no-op)
+    void ShowDecay(int delta_days) {
+        for (auto& b : blocks) {
+            for (auto& kv : b->values) {
+                Row* r = kv.second;
+                if (opt.kind == K_ADAGRAD) {
+                    r->show *= opt.show_decay_rate;
+                    r->click *= opt.show_decay_rate;
+                    r->no_show_days += delta_days;
+                } else if (opt.kind == K_FTRL) {
+                    r->show *= opt.show_decay_rate;
+                }
+            }
+        }
+    }
+
+    // Value::DeleteByShow: would the row be left out of a saved table (optimizer_kernel.h:332,345)?
+    // AdaGrad ada_grad_kernel.cc:197-204, Ftrl ftrl_kernel.cc:126, Adam adam_kernel.h:69
+    bool DeleteByShow(const Row* r) const {
+        if (opt.kind == K_ADAGRAD) {
+            if (opt.elimination_logic == 1) return r->show < opt.show_threshold && r->no_show_days > opt.no_show_days;
+            return r->show < opt.show_threshold || r->no_show_days > opt.no_show_days;
+        }
+        if (opt.kind == K_FTRL) return r->show < opt.show_threshold;
+        return false;
+    }
+
     Opt opt;
     int D, wdim, payload;
     std::minstd_rand rng;  // std::default_random_engine in libstdc++
@@ -487,6 +515,11 @@ void FillOpt(Opt& o, int kind, const float* p, int use_cvm, int zero_init) {
         o.lambda2 = p[3];
         o.initial_scale = p[4];
     }
+    // common tail of the parameter array
+    o.show_decay_rate = p[8];
+    o.show_threshold = p[9];
+    o.no_show_days = (int)p[10];
+    o.elimination_logic = (int)p[11];
 }
 
 }  // namespace
@@ -497,6 +530,7 @@ extern "C" {
 // params: AdaGrad {lr, initial_g2sum, initial_scale, epsilon, grad_decay_rate, mom_decay_rate}
 //         Adam    {lr, beta1, beta2, epsilon, initial_scale}
 //         Ftrl    {lr, beta, lambda1, lambda2, initial_scale}
+//         all kinds, at [8..11]: {show_decay_rate, show_threshold, no_show_days, elimination_logic}
 // buckets: initial bucket count per hash block (the reference uses 15485863).
 void* orc_table_create(int kind, const float* params, int dim, int use_cvm, int zero_init, uint64_t seed,
                        uint64_t buckets) {
@@ -508,6 +542,15 @@ void orc_table_destroy(void* t) { delete static_cast<Table*>(t); }
 int orc_table_weight_floats(void* t) { return static_cast<Table*>(t)->wdim; }
 int orc_table_state_floats(void* t) { return static_cast<Table*>(t)->StateFloats(); }
 uint64_t orc_table_key_count(void* t) { return static_cast<Table*>(t)->KeyCount(); }
+void orc_table_show_decay(void* t, int delta_days) { static_cast<Table*>(t)->ShowDecay(delta_days); }
+// out[i] = 1 if signs[i] is resident and Value::DeleteByShow holds for its row
+void orc_table_delete_by_show(void* tp, const uint64_t* signs, int64_t n, uint8_t* out) {
+    Table* t = static_cast<Table*>(tp);
+    for (int64_t i = 0; i < n; ++i) {
+        Row* r = t->Find(signs[i]);
+        out[i] = (r && t->DeleteByShow(r)) ? 1 : 0;
+    }
+}
 
 // Snapshot injection through the row pointer (what the reference allows via
 // the mutable float* of SparseOptimizerKernelBase::GetWeight, optimizer_kernel.h:84).

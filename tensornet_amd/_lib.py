@@ -113,6 +113,8 @@ SIGNATURES = {
                                              C.c_int, _PP, _P]),
     "tn_sparse_table_push_pooled_op": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _PP, _PP, C.c_int64, C.c_int,
                                                  C.c_int, _PP, _P]),
+    "tn_sparse_table_show_decay": (C.c_int, [C.c_uint32, C.c_int, _P]),
+    "tn_sparse_table_delete_by_show": (C.c_int, [C.c_uint32, _P, C.c_int64, _P, _P]),
     "tn_sparse_table_sync": (C.c_int, [C.c_uint32]),
     "tn_sparse_table_last_unique_counts": (C.c_int, [C.c_uint32, C.c_int, _I64P]),
     "tn_sparse_table_set_async": (C.c_int, [C.c_uint32, C.c_int]),

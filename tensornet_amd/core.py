@@ -105,6 +105,15 @@ def create_dense_table(opt):
     return h.value
 
 
+def show_decay(table_handle, delta_days):
+    """tn.core.show_decay (core/main/py_wrapper.cc:259-262): every resident row of the sparse
+    table ages by delta_days (SparseTable::ShowDecay)."""
+    import torch
+
+    _lib.check(_lib.load().tn_sparse_table_show_decay(
+        table_handle, int(delta_days), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+
 def reserve_sparse_table(table_handle, max_keys):
     """Sizes the HBM hash table for max_keys resident signs (no counterpart in
     the reference, whose host hash maps grow by themselves)."""

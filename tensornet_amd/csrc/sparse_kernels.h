@@ -322,6 +322,59 @@ __global__ __launch_bounds__(256) void k_init_rows(Store s, OptDev o, uint64_t s
     }
 }
 
+// ------------------------------------------------- show decay / elimination
+struct DecayConf {
+    int kind;
+    float rate;            // show_decay_rate
+    float show_threshold;
+    int no_show_days;
+    int elimination_logic;
+};
+
+// SparseTable::ShowDecay (core/ps/table/sparse_table.cc:139 -> optimizer_kernel.h:422-427,549-553):
+// one pass over every slot of the table; resident rows get
+//   AdaGrad  show *= rate; click *= rate; no_show_days += delta_days   (ada_grad_kernel.cc:191-195)
+//   Ftrl     show *= rate                                              (ftrl_kernel.cc:124)
+//   Adam     nothing                                                   (adam_kernel.h:67)
+__global__ __launch_bounds__(256) void k_show_decay(Store s, DecayConf c, int delta_days) {
+    const uint64_t n = s.cap + 1;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const bool resident = i < s.cap ? s.keys[i] != EMPTY_KEY : *s.special != 0;
+        if (!resident) continue;
+        float* st = s.st + i * s.sstride;
+        if (c.kind == OPT_ADAGRAD) {
+            st[1] *= c.rate;
+            st[2] *= c.rate;
+            st[3] = __int_as_float(__float_as_int(st[3]) + delta_days);
+        } else if (c.kind == OPT_FTRL) {
+            st[2 * s.D] *= c.rate;
+        }
+    }
+}
+
+// Value::DeleteByShow for the rows of given signs: out[i] = 1 if the row would be left out of a
+// saved table (optimizer_kernel.h:332,345; ada_grad_kernel.cc:197-204, ftrl_kernel.cc:126,
+// adam_kernel.h:69), 0 otherwise and for absent signs.
+__global__ __launch_bounds__(256) void k_delete_by_show(Store s, DecayConf c, const uint32_t* __restrict__ rows,
+                                                        int64_t n, uint8_t* __restrict__ out) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint32_t row = rows[i];
+        bool del = false;
+        if (row != NO_ROW) {
+            const float* st = s.st + (uint64_t)row * s.sstride;
+            if (c.kind == OPT_ADAGRAD) {
+                const bool low = st[1] < c.show_threshold, old = __float_as_int(st[3]) > c.no_show_days;
+                del = c.elimination_logic == 1 ? (low && old) : (low || old);
+            } else if (c.kind == OPT_FTRL) {
+                del = st[2 * s.D] < c.show_threshold;
+            }
+        }
+        out[i] = del ? 1 : 0;
+    }
+}
+
 // ------------------------------------------------------------------ gathers
 // out[i, :] = w[rows[i], 0:wdim]   (SparseTable::Pull's append, sparse_table.cc:64)
 template <int VEC>

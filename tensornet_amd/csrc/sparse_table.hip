@@ -1005,6 +1005,65 @@ int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t 
     return TN_OK;
 }
 
+namespace {
+DecayConf make_decayconf(const SparseTable* t) {
+    const OptConf& c = *t->opt;
+    DecayConf d{};
+    d.kind = c.kind;
+    d.rate = c.show_decay_rate;
+    d.show_threshold = c.show_threshold;
+    d.no_show_days = c.no_show_days;
+    d.elimination_logic = c.elimination_logic;
+    return d;
+}
+}  // namespace
+
+int tn_sparse_table_show_decay(uint32_t handle, int delta_days, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_show_decay: bad table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    if (t->push_pending || t->pull_pending) {
+        if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    t->last_stream = st;
+    if (t->opt->kind == OPT_ADAM) return TN_OK;  // adam_kernel.h:67
+    const Store& s = t->store;
+    TN_LAUNCH(k_show_decay, dim3(launch_grid((int64_t)s.cap + 1, 256, GRID_CAP * 8)), dim3(256), st, s, make_decayconf(t),
+              delta_days);
+    TN_HIP(hipGetLastError());
+    return TN_OK;
+}
+
+int tn_sparse_table_delete_by_show(uint32_t handle, const uint64_t* signs, int64_t n, uint8_t* out, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_delete_by_show: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && (!signs || !out))) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_delete_by_show: NULL buffer");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    t->last_stream = st;
+    if (n == 0) return TN_OK;
+    if (n > 0x7FFFFFF0LL) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_delete_by_show: more than 2^31 rows per call");
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    TN_TRY(t->ws.ensure(align_up((size_t)n * sizeof(uint32_t), 256)));
+    uint32_t* rows = (uint32_t*)t->ws.p;
+    const Store& s = t->store;
+    const int blocks = launch_grid(n, 256, GRID_CAP * 4);
+    TN_LAUNCH((k_probe<false>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows,
+              (uint32_t*)nullptr, t->dstatus, 0u, make_optdev(t), t->seed);
+    TN_LAUNCH(k_delete_by_show, dim3(blocks), dim3(256), st, s, make_decayconf(t), rows, n, out);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipStreamSynchronize(st));
+    return TN_OK;
+}
+
 // --------------------------------------------------------------- op level
 int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
                             float* const* vars, const int64_t* var_rows, int var_dim, int64_t* const* mapped_values,

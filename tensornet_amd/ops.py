@@ -332,6 +332,16 @@ def table_export_rows(table_handle, signs):
     return w, st, found
 
 
+def table_delete_by_show(table_handle, signs):
+    """Value::DeleteByShow for the rows of `signs` (uint8 tensor: 1 = the row would be left out of
+    a saved table, 0 = kept or absent)."""
+    _require(signs, torch.int64, "signs")
+    out = torch.empty((signs.numel(),), dtype=torch.uint8, device=signs.device)
+    _lib.check(_lib.load().tn_sparse_table_delete_by_show(table_handle, signs.data_ptr(), signs.numel(),
+                                                          out.data_ptr(), _stream()))
+    return out
+
+
 def dense_table_get_weight(table_handle, device="cuda"):
     total = C.c_int64()
     _lib.check(_lib.load().tn_dense_table_total_elements(table_handle, C.byref(total)))
