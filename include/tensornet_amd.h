@@ -282,6 +282,34 @@ int tn_sparse_table_show_decay(uint32_t handle, int delta_days, void* stream);
  */
 int tn_sparse_table_delete_by_show(uint32_t handle, const uint64_t* signs, int64_t n, uint8_t* out, void* stream);
 
+/*
+ * SparseTable::Save / Load (core/ps/table/sparse_table.h:55-57, sparse_table.cc:84-137; Python
+ * tn.core.save_sparse_table / load_sparse_table, core/main/py_wrapper.cc:211-220) in the
+ * reference's on-disk formats: eight gzip files
+ * <filepath>/sparse_table/<name or handle>/rank_0/block_<i>.gz, a row in file
+ * (sign >> 32 | sign << 32) % 8, mode "txt" (default of the reference) or "bin"
+ * (optimizer_kernel.h:324-420,462-538; value formats ada_grad_kernel.cc:131-189,
+ * adam_kernel.cc:127-167, ftrl_kernel.cc:82-122).  Rows for which DeleteByShow holds are not
+ * saved.  Load derives prefix, suffix and mode from the first file name as the reference does
+ * (a name without _bin / _txt suffix is read as text) and adds the rows to the table.
+ * Both work on the default stream and return when done.
+ */
+int tn_sparse_table_save(uint32_t handle, const char* filepath, const char* mode);
+int tn_sparse_table_load(uint32_t handle, const char* filepath, const char* mode);
+
+/*
+ * Building blocks of the two above (no counterpart in the reference, whose table lives in host
+ * memory).  export_range: every resident row among the table slots
+ * [first_slot, first_slot + n_slots), compacted into signs / w [.., weight_floats] /
+ * state [.., state_floats] (device, room for n_slots rows) in no particular order;
+ * skip_eliminated leaves out rows for which DeleteByShow holds; *count (host) = rows written.
+ * name / optimizer: what the table was created with (optimizer kind 0 AdaGrad, 1 Adam, 2 Ftrl).
+ */
+int tn_sparse_table_export_range(uint32_t handle, uint64_t first_slot, uint64_t n_slots, int skip_eliminated,
+                                 uint64_t* signs, float* w, float* state, uint64_t* count, void* stream);
+int tn_sparse_table_name(uint32_t handle, char* name, int cap);
+int tn_sparse_table_optimizer(uint32_t handle, int* kind, int* use_cvm);
+
 /* Wait for the table's enqueued work and return (and clear) its latched error. */
 int tn_sparse_table_sync(uint32_t handle);
 

@@ -38,6 +38,10 @@ def load():
     lib.orc_table_state_floats.argtypes = [P]
     lib.orc_table_key_count.restype = C.c_uint64
     lib.orc_table_key_count.argtypes = [P]
+    lib.orc_table_serialize_block.restype = C.c_int64
+    lib.orc_table_serialize_block.argtypes = [P, C.c_int, C.c_int, P, C.c_int64]
+    lib.orc_table_deserialize_block.restype = C.c_int64
+    lib.orc_table_deserialize_block.argtypes = [P, C.c_int, P, C.c_int64]
     lib.orc_table_show_decay.restype = None
     lib.orc_table_show_decay.argtypes = [P, C.c_int]
     lib.orc_table_delete_by_show.restype = None
@@ -149,6 +153,44 @@ class Table(object):
 
     def key_count(self):
         return int(load().orc_table_key_count(self._h))
+
+    def serialize_block(self, block, mode="txt"):
+        """Uncompressed checkpoint stream of hash block 0..7, as bytes."""
+        lib = load()
+        n = lib.orc_table_serialize_block(self._h, block, int(mode == "bin"), None, 0)
+        buf = np.zeros(max(1, n), dtype=np.uint8)
+        lib.orc_table_serialize_block(self._h, block, int(mode == "bin"), _p(buf), n)
+        return buf[:n].tobytes()
+
+    def deserialize_block(self, data, mode="txt"):
+        buf = np.frombuffer(data, dtype=np.uint8)
+        n = load().orc_table_deserialize_block(self._h, int(mode == "bin"), _p(np.ascontiguousarray(buf)), len(buf))
+        if n < 0:
+            raise ValueError("checkpoint stream was written with another optimizer or dim")
+        return int(n)
+
+    def save(self, filepath, ident, mode="txt"):
+        """SparseTable::Save (core/ps/table/sparse_table.cc:84-108): eight gzip files
+        <filepath>/sparse_table/<ident>/rank_0/block_<i>.gz."""
+        import gzip
+
+        d = os.path.join(filepath, "sparse_table", str(ident), "rank_0")
+        os.makedirs(d, exist_ok=True)
+        for b in range(8):
+            with gzip.open(os.path.join(d, "block_%d.gz" % b), "wb") as f:
+                f.write(self.serialize_block(b, mode))
+
+    def load(self, filepath, ident, mode="txt", prefix="block_", suffix=""):
+        """SparseTable::Load (sparse_table.cc:110-137); the caller names prefix / suffix / mode,
+        which the reference derives from the first file name (optimizer_kernel.h:496-520)."""
+        import gzip
+
+        d = os.path.join(filepath, "sparse_table", str(ident), "rank_0")
+        n = 0
+        for b in range(8):
+            with gzip.open(os.path.join(d, "%s%d%s.gz" % (prefix, b, suffix)), "rb") as f:
+                n += self.deserialize_block(f.read(), mode)
+        return n
 
     def show_decay(self, delta_days):
         load().orc_table_show_decay(self._h, int(delta_days))

@@ -39,10 +39,13 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <limits>
 #include <map>
 #include <memory>
 #include <new>
 #include <random>
+#include <sstream>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -325,6 +328,177 @@ public:
         return false;
     }
 
+    // ---- checkpoint streams of one hash block: SparseKernelBlock's operator<< / operator>>
+    // (optimizer_kernel.h:324-420) with the value formats of ada_grad_kernel.cc:131-189,
+    // adam_kernel.cc:127-167, ftrl_kernel.cc:82-122, followed by the std::endl that
+    // SparseOptimizerKernel::Serialized appends (optimizer_kernel.h:484).  Rows for which
+    // DeleteByShow holds are left out.
+    const char* Name() const { return opt.kind == K_ADAGRAD ? "AdaGrad" : opt.kind == K_ADAM ? "Adam" : "Ftrl"; }
+
+    void SerializeRowTxt(std::ostream& os, const Row* r) const {
+        const float* w = r->data;
+        if (opt.kind == K_ADAGRAD) {
+            os << D << "\t";
+            for (int i = 0; i < D; i++) os << w[i] << "\t";
+            os << r->g2sum << "\t";
+            os << r->show << "\t";
+            os << r->no_show_days << "\t";
+            if (opt.use_cvm) os << r->click;
+        } else {
+            const float* a = r->data + D;
+            const float* b = r->data + 2 * D;
+            for (int i = 0; i < D; i++) {
+                os << w[i] << "\t";
+                os << a[i] << "\t";
+                os << b[i] << "\t";
+            }
+            os << r->show;
+        }
+    }
+
+    void SerializeRowBin(std::ostream& os, const Row* r) const {
+        os.write(reinterpret_cast<const char*>(r->data), D * sizeof(float));
+        if (opt.kind == K_ADAGRAD) {
+            os.write(reinterpret_cast<const char*>(&r->g2sum), sizeof(float));
+            os.write(reinterpret_cast<const char*>(&r->show), sizeof(float));
+            os.write(reinterpret_cast<const char*>(&r->no_show_days), sizeof(int));
+            if (opt.use_cvm) os.write(reinterpret_cast<const char*>(&r->click), sizeof(float));
+        } else {
+            os.write(reinterpret_cast<const char*>(r->data + D), D * sizeof(float));
+            os.write(reinterpret_cast<const char*>(r->data + 2 * D), D * sizeof(float));
+            os.write(reinterpret_cast<const char*>(&r->show), sizeof(float));
+        }
+    }
+
+    std::string SerializeBlock(int block, bool bin) const {
+        std::ostringstream os;
+        const Block& b = *blocks[block];
+        if (bin) {
+            os.write(reinterpret_cast<const char*>(&D), sizeof(D));
+            for (const auto& kv : b.values) {
+                if (DeleteByShow(kv.second)) continue;
+                os.write(reinterpret_cast<const char*>(&kv.first), sizeof(kv.first));
+                SerializeRowBin(os, kv.second);
+            }
+        } else {
+            os << "opt_name:" << Name() << std::endl;
+            os << "dim:" << D << std::endl;
+            for (const auto& kv : b.values) {
+                if (DeleteByShow(kv.second)) continue;
+                os << kv.first << "\t";
+                SerializeRowTxt(os, kv.second);
+                os << std::endl;
+            }
+        }
+        os << std::endl;
+        return os.str();
+    }
+
+    void CvmColumns(Row* r) {
+        if (!opt.use_cvm) return;
+        float log_show = logf(r->show + 1);
+        float log_click = logf(r->click + 1);
+        r->data[D] = r->show;
+        r->data[D + 1] = (log_click - log_show);
+    }
+
+    // a freshly allocated value (the reference allocates a new one per record and lets the
+    // stream overwrite what the format holds)
+    Row* FreshRow(uint64_t sign) {
+        Row* r = GetOrCreate(sign);
+        Construct(r);
+        return r;
+    }
+
+    void DeSerializeRowTxt(std::istream& is, Row* r, bool old_compat) {
+        float* w = r->data;
+        if (opt.kind == K_ADAGRAD) {
+            int dim_in_file;
+            is >> dim_in_file;
+            for (int i = 0; i < D; i++) is >> w[i];
+            is >> r->g2sum;
+            is >> r->show;
+            if (!old_compat) {
+                is >> r->no_show_days;
+                if (opt.use_cvm) {
+                    is >> r->click;
+                    CvmColumns(r);
+                }
+            }
+        } else {
+            float* a = r->data + D;
+            float* b = r->data + 2 * D;
+            for (int i = 0; i < D; i++) {
+                is >> w[i];
+                is >> a[i];
+                is >> b[i];
+            }
+            is >> r->show;
+        }
+    }
+
+    // returns the number of rows read, -1 on an optimizer / dim mismatch
+    int64_t DeSerializeBlock(const std::string& data, bool bin) {
+        std::istringstream is(data);
+        int64_t n = 0;
+        if (bin) {
+            int dim = 0;
+            is.read(reinterpret_cast<char*>(&dim), sizeof(dim));
+            if (dim != D) return -1;
+            uint64_t sign = 0;
+            while (is.read(reinterpret_cast<char*>(&sign), sizeof(sign))) {
+                Row* r = FreshRow(sign);
+                is.read(reinterpret_cast<char*>(r->data), D * sizeof(float));
+                if (opt.kind == K_ADAGRAD) {
+                    is.read(reinterpret_cast<char*>(&r->g2sum), sizeof(float));
+                    is.read(reinterpret_cast<char*>(&r->show), sizeof(float));
+                    is.read(reinterpret_cast<char*>(&r->no_show_days), sizeof(int));
+                    if (opt.use_cvm) {
+                        is.read(reinterpret_cast<char*>(&r->click), sizeof(float));
+                        CvmColumns(r);
+                    }
+                } else {
+                    is.read(reinterpret_cast<char*>(r->data + D), D * sizeof(float));
+                    is.read(reinterpret_cast<char*>(r->data + 2 * D), D * sizeof(float));
+                    is.read(reinterpret_cast<char*>(&r->show), sizeof(float));
+                }
+                n++;
+            }
+            return n;
+        }
+        std::string opt_name;
+        is.ignore(std::numeric_limits<std::streamsize>::max(), ':') >> opt_name;
+        if (opt_name != Name()) return -1;
+        int dim = 0;
+        is.ignore(std::numeric_limits<std::streamsize>::max(), ':') >> dim;
+        if (dim != D) return -1;
+        // AdaGrad::NeedOldCompat (optimizer.h:94-115): the first row decides whether the file predates
+        // the no_show_days column; that row is then parsed from the sampled line
+        bool old_compat = false;
+        std::string sample;
+        if (opt.kind == K_ADAGRAD) {
+            std::string line, cell;
+            std::getline(is, line);
+            std::getline(is, line);
+            std::istringstream iss(line);
+            int columns = 0;
+            while (std::getline(iss, cell, '\t')) ++columns;
+            old_compat = columns == D + 4;
+            sample = line;
+        }
+        std::istringstream sample_is(sample);
+        uint64_t sign = 0;
+        while (sample_is >> sign) {
+            DeSerializeRowTxt(sample_is, FreshRow(sign), old_compat);
+            n++;
+        }
+        while (is >> sign) {
+            DeSerializeRowTxt(is, FreshRow(sign), old_compat);
+            n++;
+        }
+        return n;
+    }
+
     Opt opt;
     int D, wdim, payload;
     std::minstd_rand rng;  // std::default_random_engine in libstdc++
@@ -543,6 +717,16 @@ int orc_table_weight_floats(void* t) { return static_cast<Table*>(t)->wdim; }
 int orc_table_state_floats(void* t) { return static_cast<Table*>(t)->StateFloats(); }
 uint64_t orc_table_key_count(void* t) { return static_cast<Table*>(t)->KeyCount(); }
 void orc_table_show_decay(void* t, int delta_days) { static_cast<Table*>(t)->ShowDecay(delta_days); }
+// Checkpoint stream of hash block `block` (uncompressed).  Returns its size; copies it if cap suffices.
+int64_t orc_table_serialize_block(void* tp, int block, int bin, uint8_t* out, int64_t cap) {
+    const std::string s = static_cast<Table*>(tp)->SerializeBlock(block, bin != 0);
+    if ((int64_t)s.size() <= cap && out) std::memcpy(out, s.data(), s.size());
+    return (int64_t)s.size();
+}
+// Reads such a stream back; returns the rows read, -1 on a mismatch of optimizer or dim.
+int64_t orc_table_deserialize_block(void* tp, int bin, const uint8_t* data, int64_t n) {
+    return static_cast<Table*>(tp)->DeSerializeBlock(std::string(reinterpret_cast<const char*>(data), (size_t)n), bin != 0);
+}
 // out[i] = 1 if signs[i] is resident and Value::DeleteByShow holds for its row
 void orc_table_delete_by_show(void* tp, const uint64_t* signs, int64_t n, uint8_t* out) {
     Table* t = static_cast<Table*>(tp);

@@ -115,6 +115,12 @@ SIGNATURES = {
                                                  C.c_int, _PP, _P]),
     "tn_sparse_table_show_decay": (C.c_int, [C.c_uint32, C.c_int, _P]),
     "tn_sparse_table_delete_by_show": (C.c_int, [C.c_uint32, _P, C.c_int64, _P, _P]),
+    "tn_sparse_table_save": (C.c_int, [C.c_uint32, C.c_char_p, C.c_char_p]),
+    "tn_sparse_table_load": (C.c_int, [C.c_uint32, C.c_char_p, C.c_char_p]),
+    "tn_sparse_table_export_range": (C.c_int, [C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, _P, _P, _P,
+                                               C.POINTER(C.c_uint64), _P]),
+    "tn_sparse_table_name": (C.c_int, [C.c_uint32, C.c_char_p, C.c_int]),
+    "tn_sparse_table_optimizer": (C.c_int, [C.c_uint32, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "tn_sparse_table_sync": (C.c_int, [C.c_uint32]),
     "tn_sparse_table_last_unique_counts": (C.c_int, [C.c_uint32, C.c_int, _I64P]),
     "tn_sparse_table_set_async": (C.c_int, [C.c_uint32, C.c_int]),

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtensornet_amd.so")
-SOURCES = ["core.hip", "dense_table.hip", "sparse_table.hip", "sort_pairs.hip"]
+SOURCES = ["core.hip", "dense_table.hip", "sparse_table.hip", "sort_pairs.hip", "checkpoint.hip"]
 HEADERS = ["tn_common.h", "sparse_kernels.h"]
 
 FLAGS = [
@@ -39,7 +39,7 @@ HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "host_mirror_test")
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc] + FLAGS + ["-I", os.path.join(ROOT, "include"), "-I", CSRC]
-    cmd += [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES] + ["-lz", "-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

@@ -105,6 +105,17 @@ def create_dense_table(opt):
     return h.value
 
 
+def save_sparse_table(table_handle, filepath, mode="txt"):
+    """tn.core.save_sparse_table (core/main/py_wrapper.cc:211-215): the table in the reference's
+    checkpoint format under <filepath>/sparse_table/<name or handle>/rank_0/."""
+    _lib.check(_lib.load().tn_sparse_table_save(table_handle, str(filepath).encode(), str(mode).encode()))
+
+
+def load_sparse_table(table_handle, filepath, mode="txt"):
+    """tn.core.load_sparse_table (core/main/py_wrapper.cc:216-220)."""
+    _lib.check(_lib.load().tn_sparse_table_load(table_handle, str(filepath).encode(), str(mode).encode()))
+
+
 def show_decay(table_handle, delta_days):
     """tn.core.show_decay (core/main/py_wrapper.cc:259-262): every resident row of the sparse
     table ages by delta_days (SparseTable::ShowDecay)."""

@@ -375,6 +375,50 @@ __global__ __launch_bounds__(256) void k_delete_by_show(Store s, DecayConf c, co
     }
 }
 
+// Every resident row among the slots [first, first + n_slots) of the table (slot `cap` is
+// the row of the sign 0xFFFF...F), compacted into signs / w / state in no particular order;
+// with skip_eliminated rows for which DeleteByShow holds are left out (what a saved table
+// holds, optimizer_kernel.h:332,345).  *count = rows written.
+__global__ __launch_bounds__(256) void k_export_range(Store s, DecayConf c, uint64_t first, uint64_t n_slots,
+                                                      int skip_eliminated, uint64_t* __restrict__ signs,
+                                                      float* __restrict__ w, float* __restrict__ state,
+                                                      uint32_t* count) {
+    const int sf = (c.kind == OPT_ADAGRAD) ? 4 : 2 * s.D + 2;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t rounds = (n_slots + stride - 1) / stride;  // whole wavefronts take part in every round
+    for (uint64_t r = 0; r < rounds; r++) {
+        const uint64_t k = r * stride + (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        const uint64_t i = first + k;
+        bool take = false;
+        uint64_t sign = EMPTY_KEY;
+        if (k < n_slots && i <= s.cap) {
+            if (i < s.cap) {
+                sign = s.keys[i];
+                take = sign != EMPTY_KEY;
+            } else {
+                take = *s.special != 0;
+            }
+            if (take && skip_eliminated) {
+                const float* st = s.st + i * s.sstride;
+                if (c.kind == OPT_ADAGRAD) {
+                    const bool low = st[1] < c.show_threshold, old = __float_as_int(st[3]) > c.no_show_days;
+                    take = !(c.elimination_logic == 1 ? (low && old) : (low || old));
+                } else if (c.kind == OPT_FTRL) {
+                    take = !(st[2 * s.D] < c.show_threshold);
+                }
+            }
+        }
+        const uint32_t at = wave_alloc(take, count);
+        if (take) {
+            signs[at] = sign;
+            const float* sw = s.w + i * s.wstride;
+            const float* ss = s.st + i * s.sstride;
+            for (int q = 0; q < s.wdim; q++) w[(uint64_t)at * s.wdim + q] = sw[q];
+            for (int q = 0; q < sf; q++) state[(uint64_t)at * sf + q] = ss[q];
+        }
+    }
+}
+
 // ------------------------------------------------------------------ gathers
 // out[i, :] = w[rows[i], 0:wdim]   (SparseTable::Pull's append, sparse_table.cc:64)
 template <int VEC>

@@ -1018,6 +1018,51 @@ DecayConf make_decayconf(const SparseTable* t) {
 }
 }  // namespace
 
+int tn_sparse_table_export_range(uint32_t handle, uint64_t first_slot, uint64_t n_slots, int skip_eliminated,
+                                 uint64_t* signs, float* w, float* state, uint64_t* count, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_export_range: bad table handle " + std::to_string(handle));
+    if (!count || (n_slots > 0 && (!signs || !w || !state)))
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_export_range: NULL buffer");
+    if (n_slots > 0x7FFFFFF0ull) return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_export_range: more than 2^31 slots per call");
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    TN_TRY(ensure_allocated(t, st));
+    if (t->push_pending || t->pull_pending) {
+        if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    t->last_stream = st;
+    *count = 0;
+    const Store& s = t->store;
+    if (n_slots == 0 || first_slot > s.cap) return TN_OK;
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, t->dstatus, 0u, 0u);
+    TN_LAUNCH(k_export_range, dim3(launch_grid((int64_t)n_slots, 256, GRID_CAP * 4)), dim3(256), st, s, make_decayconf(t),
+              first_slot, n_slots, skip_eliminated, signs, w, state, &t->dstatus->n_new);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, t->dstatus, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    TN_HIP(hipStreamSynchronize(st));
+    *count = t->hpull->st.n_new;
+    return TN_OK;
+}
+
+int tn_sparse_table_name(uint32_t handle, char* name, int cap) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_name: bad table handle " + std::to_string(handle));
+    if (!name || cap <= 0) return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_name: NULL buffer");
+    std::snprintf(name, (size_t)cap, "%s", t->name.c_str());
+    return TN_OK;
+}
+
+int tn_sparse_table_optimizer(uint32_t handle, int* kind, int* use_cvm) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_optimizer: bad table handle " + std::to_string(handle));
+    if (kind) *kind = t->opt->kind;
+    if (use_cvm) *use_cvm = t->use_cvm ? 1 : 0;
+    return TN_OK;
+}
+
 int tn_sparse_table_show_decay(uint32_t handle, int delta_days, void* stream) {
     SparseTable* t = get_table(handle);
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_show_decay: bad table handle " + std::to_string(handle));
