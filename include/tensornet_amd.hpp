@@ -155,6 +155,17 @@ public:
         tn_sparse_table_key_count(handle_, &n);
         return n;
     }
+    // SparseTable::Save / Load (sparse_table.h:55-57): the reference's checkpoint files.
+    int Save(const std::string& filepath, const std::string& mode = "txt") {
+        return tn_sparse_table_save(handle_, filepath.c_str(), mode.c_str());
+    }
+    int Load(const std::string& filepath, const std::string& mode = "txt") {
+        return tn_sparse_table_load(handle_, filepath.c_str(), mode.c_str());
+    }
+    // SparseTable::ShowDecay (sparse_table.h:59)
+    int ShowDecay(int delta_days, void* stream = nullptr) const {
+        return tn_sparse_table_show_decay(handle_, delta_days, stream);
+    }
     // HBM sizing (no counterpart in the reference, whose host maps grow by themselves).
     int Reserve(uint64_t max_keys) { return tn_sparse_table_reserve(handle_, max_keys); }
     int Sync() { return tn_sparse_table_sync(handle_); }

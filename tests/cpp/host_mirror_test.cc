@@ -7,7 +7,9 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <string>
 #include <vector>
 
 #include "tensornet_amd.hpp"
@@ -114,6 +116,19 @@ static void gpu_checks() {
     // U_s must stay below the rows of the variable (sparse_table_ops.cc:136)
     std::vector<ops::PullSlot> tight = {{dv0, 3, var0, 2, m0}};
     EXPECT(ops::SparseTablePull((uint32_t)t->GetHandle(), tight, D) == TN_ERR_VAR_CAPACITY);
+
+    // SparseTable::ShowDecay / Save / Load: a second table of the same name reads the files back
+    EXPECT(t->ShowDecay(1) == TN_OK);
+    const char* tmp = std::getenv("TMPDIR");
+    const std::string ckpt = std::string(tmp ? tmp : "/tmp") + "/tn_host_mirror_ckpt";
+    EXPECT(t->Save(ckpt, "txt") == TN_OK);
+    SparseTable* t2 = CreateSparseTable(opt, "gpu", D, 1, 0, "");
+    EXPECT(t2 && t2 != t && t2->Load(ckpt, "txt") == TN_OK);
+    EXPECT(t2->KeyCount() == t->KeyCount());
+    EXPECT(t2->Pull(dsigns, 4, D, dout) == TN_OK);
+    std::vector<float> back(4 * D);
+    (void)hipMemcpy(back.data(), dout, back.size() * sizeof(float), hipMemcpyDeviceToHost);
+    for (int i = 0; i < D; i++) EXPECT(std::fabs(back[i] - w11) < 1e-5f);  // text keeps six digits
 
     // dense Adam, first step from zero moments: w -= lr * g / (|g| + eps')
     Adam* adam = new Adam();
