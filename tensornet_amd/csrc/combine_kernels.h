@@ -64,6 +64,7 @@ template <int VEC>
 __global__ __launch_bounds__(256) void k_combine_fwd(const SlotDesc* __restrict__ descs, int N, int dim, int64_t batch,
                                                      int combiner, const uint32_t* __restrict__ rowptr,
                                                      DevStatus* status) {
+    if (status->err) return;  // bad example ids: the row pointers are not to be trusted
     const int chunks = dim / VEC;
     const int64_t per_slot = batch * chunks;
     const int64_t total = (int64_t)N * per_slot;
@@ -151,7 +152,8 @@ __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict_
         const int64_t prev = i > 0 ? ex[i - 1] : -1;
         if (b < 0 || b >= batch || prev > b) {
             atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-            vals[gi] = ~0ull;  // no share
+            status->abort = 1;  // values of later lookups may never be written: nothing downstream may run
+            vals[gi] = ~0ull;
             continue;
         }
         if (prev == b) continue;
@@ -165,6 +167,7 @@ __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict_
 // Step 2 (after the sort): where the lookups of every distinct index start.
 __global__ __launch_bounds__(256) void k_segment_starts(const uint32_t* __restrict__ skeys, uint32_t L,
                                                         const DevStatus* status, uint32_t* __restrict__ seg_off) {
+    if (status->abort) return;
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < L; i += stride) {
         const uint32_t k = skeys[i];
@@ -204,6 +207,7 @@ __global__ __launch_bounds__(256) void k_reduce_pooled(const SlotDesc* __restric
                                                        const uint64_t* __restrict__ svals, float* __restrict__ flat,
                                                        uint32_t long_min, uint32_t* __restrict__ long_list,
                                                        uint32_t* long_count) {
+    if (status->abort) return;
     __shared__ uint32_t ub[MAX_SLOTS + 1];
     load_lbase(ub, ubase, N);
     const int chunks = dim / VEC;
@@ -247,7 +251,8 @@ __global__ __launch_bounds__(256) void k_reduce_long(const SlotDesc* __restrict_
                                                      const uint32_t* __restrict__ seg_off,
                                                      const uint64_t* __restrict__ svals, float* __restrict__ flat,
                                                      const uint32_t* __restrict__ long_list,
-                                                     const uint32_t* long_count) {
+                                                     const uint32_t* long_count, const DevStatus* status) {
+    if (status->abort) return;
     __shared__ float part[LONG_PART_FLOATS];
     const int chunks = dim / VEC;
     const int groups = 256 / chunks;

@@ -124,6 +124,7 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
         status->gcap = gcap;
         status->n_members = 0;
         status->mismatch = 0;
+        status->abort = 0;
         status->n_big = 0;
     }
 }
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ h
     if (tid == 0 && status_mode != STATUS_KEEP) {
         status->err = 0;
         status->mismatch = 0;
+        status->abort = 0;
         if (status_mode == STATUS_NEW_PLAN) {
             status->n_unique = 0;
             status->n_single = 0;
@@ -1225,7 +1227,8 @@ template <int KIND, int LPG>
 __global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc src, DevStatus* status,
                                                       const uint32_t* __restrict__ grp_row,
                                                       const Member* __restrict__ list) {
-    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
     const uint32_t n_single = status->n_single;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;
@@ -1306,7 +1309,8 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                                                    const uint32_t* __restrict__ grp_cnt,
                                                    const Member* __restrict__ list, uint32_t big_k,
                                                    uint32_t ids_cap) {
-    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
     const uint32_t n_multi = status->n_multi;
     const int D = s.D;
     const int sub = threadIdx.x % LPG;                       // my float4 inside the row
@@ -1437,7 +1441,8 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
     const int D = s.D;
     const int Dp = D + 1;  // padded staging row: lanes walking down a column hit different banks
     const int lane = threadIdx.x;
-    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
     const uint32_t n_big = status->n_big;
     const int per_chunk = (gbuf_floats / Dp) < 64 ? (gbuf_floats / Dp) : 64;
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
@@ -1574,7 +1579,8 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
                                                       const uint32_t* __restrict__ grp_cnt,
                                                       const Member* __restrict__ list, uint32_t big_k,
                                                       uint32_t ids_cap) {
-    if (status->mismatch) return;  // a push launched on a plan that turned out not to be its batch's: the host redoes it
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
     const uint32_t n_single = status->n_single, n_multi = status->n_multi;
     const int D = s.D;
     const uint32_t stride = gridDim.x * blockDim.x;

@@ -1321,14 +1321,14 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
                       p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
                       long_count);
             TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim, combiner,
-                      seg_off, svals, flat, long_list, long_count);
+                      seg_off, svals, flat, long_list, long_count, ds);
         } else {
             TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
                       p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
                       long_count);
             if (long_min != 0xFFFFFFFFu)
                 TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim,
-                          combiner, seg_off, svals, flat, long_list, long_count);
+                          combiner, seg_off, svals, flat, long_list, long_count, ds);
         }
         src.flat = flat;
         return TN_OK;

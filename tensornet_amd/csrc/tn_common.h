@@ -88,7 +88,8 @@ struct DevStatus {
     uint32_t n_members;  // records in groups with several records (their lists fill the member array from the top)
     uint32_t mismatch;   // a push found other signs than the plan was built from
     uint32_t n_big;      // groups with many records (handled one wavefront each)
-    uint32_t pad[3];
+    uint32_t abort;      // the call's inputs are unusable (flagged in err): later kernels of the call do nothing
+    uint32_t pad[2];
 };
 
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {

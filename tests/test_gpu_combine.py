@@ -94,6 +94,29 @@ def test_combine_rejects_bad_example_ids_and_ids(tn, oracle):
     assert float(out[0].abs().sum()) == 0.0
 
 
+def test_pooled_push_with_unsorted_example_ids_changes_nothing(tn, oracle):
+    """Example ids that are not sorted (or lie outside the batch) cannot be reduced: the push is
+    reported as failed at the next synchronising call and leaves every row as it was."""
+    rng = np.random.default_rng(4)
+    batch, slots, vocab, dim = 100, 3, 300, 8
+    pair = Pair(tn, oracle, "AdaGrad", dim, ADAGRAD_HP)
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    values, examples = ragged_slots(rng, slots, batch, vocab, 3.0)
+    pair.pull_op(values)
+    pooled = [dev(rng.standard_normal((batch, dim)).astype(np.float32)) for _ in range(slots)]
+    labels = [dev(np.zeros(len(v), np.int64)) for v in values]
+    for spoil in ("unsorted", "out of range"):
+        bad = [e.copy() for e in examples]
+        if spoil == "unsorted":
+            bad[1][[0, -1]] = bad[1][[-1, 0]]
+        else:
+            bad[0][-1] = batch
+        tn.ops.sparse_table_push_pooled([dev(v) for v in values], [dev(e) for e in bad], pooled, labels, pair.h, "mean")
+        with pytest.raises(TensorNetError):
+            tn.ops.sparse_table_sync(pair.h)
+        pair.assert_rows_match(base, exact=True)
+
+
 def test_full_size_pooled_push_equals_push_of_reduced_gradients(tn, oracle):
     """cfg3-sized batch (16384 x 100 slots, ~5 M lookups): a pooled push must leave the table in
     the state a plain push leaves it in when the per-distinct-sign gradients are reduced by torch
