@@ -547,7 +547,7 @@ def test_remap_falls_back_when_a_bucket_overflows(tn, oracle):
     D = 8
     rng = np.random.default_rng(77)
     n_slot = 40000
-    nb = (n_slot + 1535) // 1536  # buckets of the slot
+    nb = (n_slot + 767) // 768  # buckets of the slot (768 lookups each on average)
     cand = rng.integers(0, 1 << 63, 400000, dtype=np.uint64)
     x = cand.copy()
     x ^= x >> np.uint64(33)
@@ -566,6 +566,37 @@ def test_remap_falls_back_when_a_bucket_overflows(tn, oracle):
     pair.populate(all_signs(values))
     counts = check_pull(pair, values)
     assert counts.tolist() == [len(np.unique(slot0)), len(np.unique(slot1))]
+    grads = synth.make_grads(counts, D, 0.01)
+    pair.push_op(values, grads, [np.ones(len(v), np.int64) for v in values])
+    pair.assert_rows_match(all_signs(values))
+
+
+def test_grouping_falls_back_when_a_second_level_bucket_overflows(tn, oracle):
+    """The distinct records of all slots are grouped in buckets chosen by the sign's hash (room
+    for 1536 records each); 2500 distinct signs crafted into one such bucket make the call fall
+    back to the global-table path, with the reference's results."""
+    D = 8
+    rng = np.random.default_rng(78)
+    slots, per_slot = 64, 1000
+    nb2 = (slots * per_slot + 1023) // 1024
+    cand = rng.integers(0, 1 << 63, 600000, dtype=np.uint64)
+    x = cand.copy()
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xFF51AFD7ED558CCD)
+    x ^= x >> np.uint64(33)
+    x *= np.uint64(0xC4CEB9FE1A85EC53)
+    x ^= x >> np.uint64(33)
+    bucket = ((x >> np.uint64(32)) * np.uint64(nb2)) >> np.uint64(32)
+    crowd = cand[bucket == 0][:2560]
+    assert len(crowd) == 2560
+    filler = cand[bucket != 0]
+    values = []
+    for s in range(slots):
+        mine = np.concatenate([crowd[s * 40:(s + 1) * 40], filler[s * 900:s * 900 + 960]])
+        values.append(rng.permutation(mine).view(np.int64))
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=300000)
+    pair.populate(all_signs(values))
+    counts = check_pull(pair, values)
     grads = synth.make_grads(counts, D, 0.01)
     pair.push_op(values, grads, [np.ones(len(v), np.int64) for v in values])
     pair.assert_rows_match(all_signs(values))
