@@ -600,3 +600,24 @@ def test_grouping_falls_back_when_a_second_level_bucket_overflows(tn, oracle):
     grads = synth.make_grads(counts, D, 0.01)
     pair.push_op(values, grads, [np.ones(len(v), np.int64) for v in values])
     pair.assert_rows_match(all_signs(values))
+
+
+def test_cfg3_full_batch_against_the_oracle(tn, oracle):
+    """One whole cfg3 batch (16384 x 100 slots, ~5 M lookups, ~2 M distinct per slot, ~1.1 M
+    distinct signs) through pull and push on both sides: every mapped id and pulled row bit for
+    bit, every updated row within the tolerance (and nearly all of them bit for bit).  The
+    resident set is the batch's own signs (the oracle cannot hold 5e8 rows)."""
+    cfg = synth.CONFIGS["cfg3"]
+    D = cfg["dim"]
+    values = synth.make_batch(cfg, 2)
+    signs = all_signs(values)
+    pair = Pair(tn, oracle, "AdaGrad", D, cfg["hyper"], reserve=3 * 10 ** 6)
+    pair.populate(signs)
+    counts = check_pull(pair, values)
+    assert sum(len(v) for v in values) > 4.9e6 and int(counts.sum()) > 1.9e6
+    grads = synth.make_grads(counts, D, cfg["grad_sigma"], seed=9)
+    rng = np.random.default_rng(9)
+    labels = [(rng.random(len(v)) < 0.05).astype(np.int64) for v in values]
+    pair.push_op(values, grads, labels)
+    assert pair.assert_rows_match(signs) > 0.99
+    check_pull(pair, values)
