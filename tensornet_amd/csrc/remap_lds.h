@@ -365,6 +365,16 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
     }
 }
 
+// Rank of the first occurrence at position gi = number of first occurrences before it: the
+// count up to its 64-lookup word (wordpre, written by k_lds_assign) plus the flags below it
+// in the word.  Both arrays are small enough to stay in L2 (L / 8 and L / 16 bytes), so a
+// rank costs two cache hits instead of a random read of a 4-byte-per-lookup array.
+__device__ __forceinline__ uint32_t rank_of(const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ wordpre,
+                                            uint32_t gi) {
+    const uint64_t word = reinterpret_cast<const uint64_t*>(flag8)[gi >> 6];
+    return wordpre[gi >> 6] + (uint32_t)__popcll(word & ((1ull << (gi & 63)) - 1ull));
+}
+
 // Tile counts of first occurrences; a lookup is one iff first_of[gi] == gi.
 __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const uint32_t* __restrict__ first_of,
                                                              uint8_t* __restrict__ flag8,
@@ -384,14 +394,14 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const u
     if (threadIdx.x == 0) tilesum[blockIdx.x] = total;
 }
 
-// Ranks of the first occurrences (rank_at[gi]) and, with LISTS, the distinct
+// Ranks of the first occurrences (per 64-lookup word: wordpre, see rank_of) and, with LISTS, the distinct
 // lists and show counts.  Each thread owns 8 consecutive lookups; all loads are
 // issued before any dependent store.
 template <bool LISTS>
 __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L,
     const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff, const uint32_t* __restrict__ cnt_at,
-    uint32_t* __restrict__ rank_at, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
+    uint32_t* __restrict__ wordpre, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
     uint32_t* __restrict__ uniq_slot, uint32_t* __restrict__ ushow) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t red[4];
@@ -401,6 +411,7 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     if (base < L) bits = flag8[base / REMAP_ITEMS];
     uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256<uint32_t>(__popc(bits), red, nullptr);
     if (base >= L) return;
+    if ((base & 63u) == 0) wordpre[base >> 6] = u;  // first occurrences before this 64-lookup word
     int sls[REMAP_ITEMS];
     uint64_t vals[REMAP_ITEMS];
     uint32_t cnts[REMAP_ITEMS];
@@ -430,7 +441,6 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
             for (int e = sl - 1; e >= 0 && lb[e] == gi; e--) ubase[e] = u;
         }
         if (bits & (1u << j)) {
-            rank_at[gi] = u;
             if (LISTS) {
                 uniq_sign[u] = vals[j];
                 uniq_slot[u] = (uint32_t)sl;
@@ -446,14 +456,15 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
                                                     const uint32_t* __restrict__ lbase,
                                                     const uint32_t* __restrict__ ubase, int N, uint32_t L,
                                                     const uint32_t* __restrict__ first_of,
-                                                    const uint32_t* __restrict__ rank_at,
+                                                    const uint8_t* __restrict__ flag8,
+                                                    const uint32_t* __restrict__ wordpre,
                                                     uint32_t* __restrict__ u_of_gi) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const uint32_t f = first_of[gi];
-        const uint32_t u = rank_at[f];
+        const uint32_t u = rank_of(flag8, wordpre, f);
         u_of_gi[gi] = u | (f == gi ? FIRST_BIT : 0u);
         const int sl = find_slot(lb, N, gi);
         descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
@@ -626,7 +637,8 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
 __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
-                                                    const uint32_t* __restrict__ rank_at, uint32_t ids_cap,
+                                                    const uint8_t* __restrict__ flag8,
+                                                    const uint32_t* __restrict__ wordpre, uint32_t ids_cap,
                                                     uint32_t big_k, uint64_t* __restrict__ grp_sign,
                                                     uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
@@ -648,7 +660,7 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
         }
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++)
-            if (j * 256 + threadIdx.x < n) us[j] = rank_at[rs[j].gi];
+            if (j * 256 + threadIdx.x < n) us[j] = rank_of(flag8, wordpre, rs[j].gi);
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
             if (j * 256 + threadIdx.x >= n) continue;

@@ -370,7 +370,7 @@ struct Scratch {
     uint32_t* pgi;
     uint32_t* first_of;
     uint32_t* cnt_at;
-    uint32_t* rank_at;
+    uint32_t* wordpre;  // first occurrences before every 64-lookup word
     // grouping through LDS (second-level buckets)
     uint32_t nb2;
     uint32_t* cursor2;
@@ -441,7 +441,7 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.pgi = c.take<uint32_t>(L);
         w.first_of = c.take<uint32_t>(L);
         w.cnt_at = c.take<uint32_t>(L);
-        w.rank_at = c.take<uint32_t>(L);
+        w.wordpre = c.take<uint32_t>(L / 64 + 2);
         w.dt = nullptr;
         w.dt_entries = 0;
         w.tidx = nullptr;
@@ -628,11 +628,11 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
         if (lds_groups)
             TN_LAUNCH((k_lds_assign<false>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
         else
             TN_LAUNCH((k_lds_assign<true>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.rank_at, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
-        TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.rank_at,
+                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+        TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.flag8, w.wordpre,
                   p.u_of_gi);
     } else {
         TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st,
@@ -650,7 +650,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
-        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.rank_at, L,
+        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.flag8, w.wordpre, L,
                   big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u);
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
