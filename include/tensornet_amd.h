@@ -353,6 +353,19 @@ int tn_dense_table_set_weight(uint32_t handle, const float* w, void* stream);
 /* Optimizer state read-back for tests: Adam m,v ; AdaGrad d2sum,g2sum,m (device, total floats each; NULL skips). */
 int tn_dense_table_get_state(uint32_t handle, float* s0, float* s1, float* s2, void* stream);
 
+/*
+ * DenseTable::Save / Load (core/ps/table/dense_table.cc:103-157; py_wrapper.cc:221-230):
+ * one text file <filepath>/dense_table/<handle>/<self_shard_id> holding the total, the
+ * shard count and, per block of ceil(total / 8) elements, the optimizer's name, the
+ * block length, Adam's beta powers and one line of w and state per element, printed as
+ * operator<< prints a float (6 significant digits).  Save of a table that was never
+ * initialised writes nothing.  Load initialises the table to the file's total (an
+ * initialised table of another size: TN_ERR_ALREADY_INIT) and refuses a file of another
+ * optimizer or shard count.  Synchronous, host code.
+ */
+int tn_dense_table_save(uint32_t handle, const char* filepath);
+int tn_dense_table_load(uint32_t handle, const char* filepath);
+
 /* --------------------------------------------------------------- profiling */
 /*
  * Measurement hooks with no counterpart in the reference (which instruments

@@ -233,6 +233,9 @@ public:
         int64_t lens[1] = {total};
         return tn_dense_table_push_pull(handle_, 1, vars, grads, lens, lr, stream);
     }
+    // DenseTable::Save / Load (dense_table.cc:103-157): text file <filepath>/dense_table/<handle>/0.
+    int Save(const std::string& filepath) const { return tn_dense_table_save(handle_, filepath.c_str()); }
+    int Load(const std::string& filepath) { return tn_dense_table_load(handle_, filepath.c_str()); }
     uint32_t GetHandle() const { return handle_; }
     int TotalElements() const {
         int64_t t = 0;

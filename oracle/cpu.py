@@ -64,6 +64,10 @@ def load():
     lib.orc_dense_apply.argtypes = [P, P, C.c_float]
     lib.orc_dense_num_blocks.argtypes = [P]
     lib.orc_dense_get_state.argtypes = [P, C.c_int, P]
+    lib.orc_dense_serialize.restype = C.c_int64
+    lib.orc_dense_serialize.argtypes = [P, C.c_int, P, C.c_int64]
+    lib.orc_dense_deserialize.argtypes = [P, C.c_int, P, C.c_int64]
+    lib.orc_dense_get_powers.argtypes = [P, C.c_int, P]
     _lib = lib
     return lib
 
@@ -290,3 +294,34 @@ class Dense(object):
         out = np.zeros(self.total, dtype=np.float32)
         load().orc_dense_get_state(self._h, which, _p(out))
         return out
+
+    def beta_powers(self, block=0):
+        out = np.zeros(2, dtype=np.float32)
+        load().orc_dense_get_powers(self._h, block, _p(out))
+        return float(out[0]), float(out[1])
+
+    def serialize(self, rank_num=1):
+        """Text of the checkpoint file DenseTable::Save writes (core/ps/table/dense_table.cc:103-128)."""
+        lib = load()
+        n = lib.orc_dense_serialize(self._h, rank_num, None, 0)
+        buf = np.zeros(max(1, n), dtype=np.uint8)
+        lib.orc_dense_serialize(self._h, rank_num, _p(buf), n)
+        return buf[:n].tobytes()
+
+    def deserialize(self, data, shard_num=1):
+        """DenseTable::Load (dense_table.cc:130-157) into a table of the file's total."""
+        buf = np.ascontiguousarray(np.frombuffer(data, dtype=np.uint8))
+        rc = load().orc_dense_deserialize(self._h, shard_num, _p(buf), len(buf))
+        if rc != 0:
+            raise ValueError({-1: "total elements", -2: "shard count", -3: "optimizer", -4: "block length"}[rc]
+                             + " of the checkpoint differs from the table's")
+
+    def save(self, filepath, handle, shard=0):
+        d = os.path.join(filepath, "dense_table", str(handle))
+        os.makedirs(d, exist_ok=True)
+        with open(os.path.join(d, str(shard)), "wb") as f:
+            f.write(self.serialize())
+
+    def load(self, filepath, handle, shard=0):
+        with open(os.path.join(filepath, "dense_table", str(handle), str(shard)), "rb") as f:
+            self.deserialize(f.read())

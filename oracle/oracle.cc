@@ -631,6 +631,63 @@ struct Dense {
         }
     }
 
+    const char* Name() const { return opt.kind == K_ADAGRAD ? "AdaGrad" : "Adam"; }
+
+    // DenseTable::Save (core/ps/table/dense_table.cc:103-128) down to the value streams:
+    // table header, then DenseOptimizerKernel::Serialized (optimizer_kernel.h:224-229) =
+    // per block "opt_name:" + value + endl (block stream, :139-146) + endl, the value being
+    // DenseAdamValue's (adam_kernel.cc:57-69) or DenseAdaGradValue's (ada_grad_kernel.cc:50-60).
+    std::string Serialize(int rank_num) const {
+        std::ostringstream os;
+        os << "total_elements:" << (int)total << std::endl;
+        os << "rank_num:" << rank_num << std::endl;
+        for (const DenseBlock& b : blocks) {
+            os << "opt_name:" << Name() << std::endl;
+            int array_size = (int)b.w.size();
+            os << "array_size:" << array_size << std::endl;
+            if (opt.kind == K_ADAM) {
+                os << "beta1_power:" << b.beta1_power << std::endl;
+                os << "beta2_power:" << b.beta2_power << std::endl;
+                for (int i = 0; i < array_size; i++) os << b.w[i] << "\t" << b.a[i] << "\t" << b.b[i] << std::endl;
+            } else {
+                for (int i = 0; i < array_size; i++)
+                    os << b.w[i] << "\t" << b.a[i] << "\t" << b.b[i] << "\t" << b.c[i] << std::endl;
+            }
+            os << std::endl;  // block stream: os << value << endl
+            os << std::endl;  // Serialized: os << block << endl
+        }
+        return os.str();
+    }
+
+    // DenseTable::Load (dense_table.cc:130-157) on a table created with the file's total;
+    // returns 0, or -1 total / -2 rank_num / -3 optimizer / -4 block length mismatch (the
+    // reference's CHECKs).  Value streams: adam_kernel.cc:71-87, ada_grad_kernel.cc:62-76.
+    int DeSerialize(const std::string& data, int shard_num) {
+        std::istringstream is(data);
+        const auto skip = std::numeric_limits<std::streamsize>::max();
+        int total_elements = 0, rank_num = 0;
+        is.ignore(skip, ':') >> total_elements;
+        is.ignore(skip, ':') >> rank_num;
+        if (shard_num != rank_num) return -2;
+        if (total_elements != (int)total) return -1;
+        for (DenseBlock& b : blocks) {
+            std::string name;
+            is.ignore(skip, ':') >> name;
+            if (name != Name()) return -3;
+            int array_size = 0;
+            is.ignore(skip, ':') >> array_size;
+            if (array_size != (int)b.w.size()) return -4;
+            if (opt.kind == K_ADAM) {
+                is.ignore(skip, ':') >> b.beta1_power;
+                is.ignore(skip, ':') >> b.beta2_power;
+                for (int i = 0; i < array_size; i++) is >> b.w[i] >> b.a[i] >> b.b[i];
+            } else {
+                for (int i = 0; i < array_size; i++) is >> b.w[i] >> b.a[i] >> b.b[i] >> b.c[i];
+            }
+        }
+        return 0;
+    }
+
     // DenseAdamValue::Apply, adam_kernel.cc:46-55.  Eigen evaluates each
     // expression elementwise in float; double scalars are narrowed to float first.
     void ApplyAdam(DenseBlock& b, const float* g, float lr) {
@@ -850,6 +907,20 @@ void orc_dense_destroy(void* d) { delete static_cast<Dense*>(d); }
 void orc_dense_set_weight(void* d, const float* w) { static_cast<Dense*>(d)->SetWeight(w); }
 void orc_dense_get_weight(void* d, float* w) { static_cast<Dense*>(d)->GetWeight(w); }
 void orc_dense_apply(void* d, const float* grad, float lr) { static_cast<Dense*>(d)->Apply(grad, lr); }
+// The text of the table's checkpoint file.  Returns its size; copies it if cap suffices.
+int64_t orc_dense_serialize(void* dp, int rank_num, uint8_t* out, int64_t cap) {
+    const std::string s = static_cast<Dense*>(dp)->Serialize(rank_num);
+    if ((int64_t)s.size() <= cap && out) std::memcpy(out, s.data(), s.size());
+    return (int64_t)s.size();
+}
+int orc_dense_deserialize(void* dp, int shard_num, const uint8_t* data, int64_t n) {
+    return static_cast<Dense*>(dp)->DeSerialize(std::string(reinterpret_cast<const char*>(data), (size_t)n), shard_num);
+}
+void orc_dense_get_powers(void* dp, int block, float* out) {
+    const DenseBlock& b = static_cast<Dense*>(dp)->blocks[(size_t)block];
+    out[0] = b.beta1_power;
+    out[1] = b.beta2_power;
+}
 int orc_dense_num_blocks(void* d) { return (int)static_cast<Dense*>(d)->blocks.size(); }
 // which: 0 = first state array (Adam m / AdaGrad d2sum), 1 = second (v / g2sum), 2 = third (AdaGrad m)
 void orc_dense_get_state(void* dp, int which, float* out) {

@@ -131,6 +131,8 @@ SIGNATURES = {
     "tn_dense_table_get_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_set_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_get_state": (C.c_int, [C.c_uint32, _P, _P, _P, _P]),
+    "tn_dense_table_save": (C.c_int, [C.c_uint32, C.c_char_p]),
+    "tn_dense_table_load": (C.c_int, [C.c_uint32, C.c_char_p]),
     "tn_profile_enable": (C.c_int, [C.c_int]),
     "tn_profile_reset": (C.c_int, []),
     "tn_profile_summary": (C.c_int, [C.c_char_p, C.c_size_t]),

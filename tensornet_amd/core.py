@@ -116,6 +116,17 @@ def load_sparse_table(table_handle, filepath, mode="txt"):
     _lib.check(_lib.load().tn_sparse_table_load(table_handle, str(filepath).encode(), str(mode).encode()))
 
 
+def save_dense_table(table_handle, filepath):
+    """tn.core.save_dense_table (core/main/py_wrapper.cc:221-225): the dense table as the
+    reference's text file <filepath>/dense_table/<handle>/0."""
+    _lib.check(_lib.load().tn_dense_table_save(table_handle, str(filepath).encode()))
+
+
+def load_dense_table(table_handle, filepath):
+    """tn.core.load_dense_table (core/main/py_wrapper.cc:226-230)."""
+    _lib.check(_lib.load().tn_dense_table_load(table_handle, str(filepath).encode()))
+
+
 def show_decay(table_handle, delta_days):
     """tn.core.show_decay (core/main/py_wrapper.cc:259-262): every resident row of the sparse
     table ages by delta_days (SparseTable::ShowDecay)."""

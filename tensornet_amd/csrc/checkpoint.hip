@@ -461,10 +461,154 @@ int load_table(uint32_t handle, const char* filepath, const char* mode) {
     return ld.flush();
 }
 
+// ------------------------------------------------------------------ dense table
+// DenseTable::Save / Load (core/ps/table/dense_table.cc:103-157): one plain text file
+//   <filepath>/dense_table/<handle>/<self_shard_id>
+//   "total_elements:<n>\n" "rank_num:<shards>\n", then per block of ceil(n / 8) elements
+//   (DenseOptimizerKernel, optimizer_kernel.h:174-188,224-235; block stream :139-160)
+//   "opt_name:<Name>\n" "array_size:<len>\n" [Adam: "beta1_power:<f>\n" "beta2_power:<f>\n"]
+//   one element per line, tab separated: Adam w m v (adam_kernel.cc:57-87), AdaGrad
+//   w d2sum g2sum m (ada_grad_kernel.cc:50-76), then two empty lines.
+constexpr int kDenseBlocks = 8;                 // DENSE_KERNEL_BLOCK_NUM
+constexpr int64_t kDenseChunk = 1 << 20;        // elements formatted / parsed per round
+
+std::string dense_file(uint32_t handle, const char* filepath, const DenseMeta& m) {
+    return std::string(filepath) + "/dense_table/" + std::to_string(handle) + "/" + std::to_string(m.self_shard_id);
+}
+
+int save_dense(uint32_t handle, const char* filepath) {
+    if (!filepath) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: NULL path");
+    DenseMeta m;
+    TN_TRY(dense_meta(handle, m));
+    if (!m.initialized) return TN_OK;  // no kernel for this shard yet: nothing is written (dense_table.cc:106-109)
+    const std::string file = dense_file(handle, filepath, m);
+    TN_TRY(make_dirs(file.substr(0, file.rfind('/'))));
+    FILE* f = std::fopen(file.c_str(), "wb");
+    if (!f) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: cannot write " + file);
+    const int arrays = m.kind == OPT_ADAM ? 3 : 4;
+    std::vector<float> host[4];
+    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, m.total));
+    float* arr[4] = {host[0].data(), host[1].data(), host[2].data(), arrays == 4 ? host[3].data() : nullptr};
+    std::string out = "total_elements:" + std::to_string(m.total) + "\nrank_num:" + std::to_string(m.shard_num) + "\n";
+    const int64_t per_block = (m.total + kDenseBlocks - 1) / kDenseBlocks;
+    int rc = TN_OK;
+    for (int64_t b0 = 0; b0 < m.total && rc == TN_OK; b0 += per_block) {
+        const int64_t len = std::min(per_block, m.total - b0);
+        out += std::string("opt_name:") + opt_name(m.kind) + "\narray_size:" + std::to_string(len) + "\n";
+        if (m.kind == OPT_ADAM) {
+            out += "beta1_power:";
+            put_float(out, m.beta1_power);
+            out += "\nbeta2_power:";
+            put_float(out, m.beta2_power);
+            out += '\n';
+        }
+        for (int64_t c0 = 0; c0 < len && rc == TN_OK; c0 += kDenseChunk) {
+            const int64_t n = std::min(kDenseChunk, len - c0);
+            rc = dense_copy_range(handle, b0 + c0, n, arr, true);
+            for (int64_t i = 0; i < n && rc == TN_OK; i++) {
+                for (int a = 0; a < arrays; a++) {
+                    put_float(out, host[a][(size_t)i]);
+                    out += a + 1 < arrays ? '\t' : '\n';
+                }
+            }
+            if (std::fwrite(out.data(), 1, out.size(), f) != out.size())
+                rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: write failed on " + file);
+            out.clear();
+        }
+        out += "\n\n";
+    }
+    if (rc == TN_OK && std::fwrite(out.data(), 1, out.size(), f) != out.size())
+        rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: write failed on " + file);
+    if (std::fclose(f) != 0 && rc == TN_OK) rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: close failed on " + file);
+    return rc;
+}
+
+// "<anything>:<token>" as `is.ignore(max, ':') >> x` reads it
+bool after_colon(Tokens& tk, std::string& token) {
+    while (tk.p < tk.end && *tk.p != ':') tk.p++;
+    if (tk.p >= tk.end) return false;
+    tk.p++;
+    const char *b, *e;
+    if (!tk.next(b, e)) return false;
+    token.assign(b, e);
+    return true;
+}
+
+int load_dense(uint32_t handle, const char* filepath) {
+    if (!filepath) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_load: NULL path");
+    DenseMeta m;
+    TN_TRY(dense_meta(handle, m));
+    const std::string file = dense_file(handle, filepath, m);
+    FILE* f = std::fopen(file.c_str(), "rb");
+    if (!f) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_load: cannot read " + file);
+    std::string data;
+    {
+        std::vector<char> buf(1 << 22);
+        size_t got;
+        while ((got = std::fread(buf.data(), 1, buf.size(), f)) > 0) data.append(buf.data(), got);
+        std::fclose(f);
+    }
+    const std::string bad = "tn_dense_table_load: malformed file " + file;
+    Tokens tk{data.data(), data.data() + data.size()};
+    std::string tok;
+    if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+    const int64_t total = std::strtoll(tok.c_str(), nullptr, 10);
+    if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+    const int rank_num = std::atoi(tok.c_str());
+    if (rank_num != m.shard_num)  // CHECK_EQ(shard_num_, rank_num), dense_table.cc:140
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_load: file written by " + std::to_string(rank_num) +
+                                                 " shards, table has " + std::to_string(m.shard_num));
+    TN_TRY(dense_ensure_init(handle, total));  // CHECK_EQ(0, Init(total_elements_)), :142
+    const int arrays = m.kind == OPT_ADAM ? 3 : 4;
+    std::vector<float> host[4];
+    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, total));
+    float* arr[4] = {host[0].data(), host[1].data(), host[2].data(), arrays == 4 ? host[3].data() : nullptr};
+    const int64_t per_block = (total + kDenseBlocks - 1) / kDenseBlocks;
+    bool have_powers = false;
+    float b1p = 1.f, b2p = 1.f;
+    for (int64_t b0 = 0; b0 < total; b0 += per_block) {
+        const int64_t len = std::min(per_block, total - b0);
+        if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+        if (tok != opt_name(m.kind))  // optimizer_kernel.h:153-155
+            return fail(TN_ERR_INVALID_ARGUMENT, "last trained model with optimizer is:" + tok +
+                                                     " but current model use:" + opt_name(m.kind) + " instead");
+        if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+        if (std::strtoll(tok.c_str(), nullptr, 10) != len)  // CHECK_EQ(array_size, w_.size())
+            return fail(TN_ERR_DIM_MISMATCH, "tn_dense_table_load: block of " + tok + " elements, table expects " +
+                                                 std::to_string(len));
+        if (m.kind == OPT_ADAM) {
+            float p1, p2;
+            if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+            p1 = std::strtof(tok.c_str(), nullptr);
+            if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+            p2 = std::strtof(tok.c_str(), nullptr);
+            // every block steps on every push, so all blocks of one file hold the same powers
+            if (have_powers && (p1 != b1p || p2 != b2p))
+                return fail(TN_ERR_UNSUPPORTED, "tn_dense_table_load: blocks with different beta powers in " + file);
+            b1p = p1;
+            b2p = p2;
+            have_powers = true;
+        }
+        for (int64_t c0 = 0; c0 < len; c0 += kDenseChunk) {
+            const int64_t n = std::min(kDenseChunk, len - c0);
+            for (int64_t i = 0; i < n; i++)
+                for (int a = 0; a < arrays; a++)
+                    if (!tk.f32(host[a][(size_t)i])) return fail(TN_ERR_INVALID_ARGUMENT, bad);
+            TN_TRY(dense_copy_range(handle, b0 + c0, n, arr, false));
+        }
+    }
+    if (have_powers) TN_TRY(dense_set_powers(handle, b1p, b2p));
+    return TN_OK;
+}
+
 }  // namespace
 }  // namespace tn
 
 extern "C" {
+
+int tn_dense_table_save(uint32_t handle, const char* filepath) { return tn::save_dense(handle, filepath); }
+
+int tn_dense_table_load(uint32_t handle, const char* filepath) { return tn::load_dense(handle, filepath); }
 
 int tn_sparse_table_save(uint32_t handle, const char* filepath, const char* mode) {
     return tn::save_table(handle, filepath, mode);

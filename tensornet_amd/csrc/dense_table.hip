@@ -125,6 +125,46 @@ int launch_grid(int64_t work_items, int threads, int max_blocks) {
     return (int)b;
 }
 
+int dense_meta(uint32_t handle, DenseMeta& m) {
+    DenseTable* t = get_dense(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad dense table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    m.kind = t->opt->kind;
+    m.shard_num = t->shard_num;
+    m.self_shard_id = t->self_shard_id;
+    m.initialized = t->initialized;
+    m.total = t->total;
+    m.beta1_power = t->beta1_power;
+    m.beta2_power = t->beta2_power;
+    return TN_OK;
+}
+
+int dense_set_powers(uint32_t handle, float beta1_power, float beta2_power) {
+    DenseTable* t = get_dense(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad dense table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->beta1_power = beta1_power;
+    t->beta2_power = beta2_power;
+    return TN_OK;
+}
+
+int dense_copy_range(uint32_t handle, int64_t off, int64_t n, float* const arr[4], bool to_host) {
+    DenseTable* t = get_dense(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad dense table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (!t->initialized) return fail(TN_ERR_NOT_INIT, "dense table not initialised");
+    if (off < 0 || n < 0 || off + n > t->total) return fail(TN_ERR_INVALID_ARGUMENT, "dense table range out of bounds");
+    float* dev[4] = {t->w, t->s0, t->s1, t->s2};
+    for (int a = 0; a < 4; a++) {
+        if (!dev[a] || !arr[a] || n == 0) continue;
+        if (to_host)
+            TN_HIP(hipMemcpy(arr[a], dev[a] + off, (size_t)n * sizeof(float), hipMemcpyDeviceToHost));
+        else
+            TN_HIP(hipMemcpy(dev[a] + off, arr[a], (size_t)n * sizeof(float), hipMemcpyHostToDevice));
+    }
+    return TN_OK;
+}
+
 }  // namespace tn
 
 using namespace tn;
@@ -180,6 +220,19 @@ static int dense_alloc(DenseTable* t, int64_t total, hipStream_t st) {
     t->initialized = true;
     return TN_OK;
 }
+
+}  // extern "C"
+
+int tn::dense_ensure_init(uint32_t handle, int64_t total) {
+    DenseTable* t = get_dense(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad dense table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    TN_TRY(dense_alloc(t, total, nullptr));
+    TN_HIP(hipStreamSynchronize(nullptr));
+    return TN_OK;
+}
+
+extern "C" {
 
 int tn_dense_table_init(uint32_t handle, int N, const float* const* vars, const int64_t* var_lens, void* stream) {
     DenseTable* t = get_dense(handle);

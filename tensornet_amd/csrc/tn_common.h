@@ -123,6 +123,23 @@ struct DevBuf {
 
 int launch_grid(int64_t work_items, int threads, int max_blocks);
 
+// Host-side access to a dense table for the checkpoint code (defined beside the table).
+struct DenseMeta {
+    int kind;  // OPT_ADAM / OPT_ADAGRAD
+    int shard_num, self_shard_id;
+    bool initialized;
+    int64_t total;
+    float beta1_power, beta2_power;
+};
+int dense_meta(uint32_t handle, DenseMeta& m);
+// DenseTable::Init(total): allocates on first use, a different size afterwards is an error.
+int dense_ensure_init(uint32_t handle, int64_t total);
+int dense_set_powers(uint32_t handle, float beta1_power, float beta2_power);
+// Copies elements [off, off + n) between the table's arrays and host arrays: arr[0] = w,
+// arr[1..3] = the optimizer's state arrays in the order its value prints them (Adam m, v;
+// AdaGrad d2sum, g2sum, m); arrays the optimizer lacks are skipped.
+int dense_copy_range(uint32_t handle, int64_t off, int64_t n, float* const arr[4], bool to_host);
+
 // ---------------------------------------------------------------- profiling
 // When enabled (tn_profile_enable) every kernel launch is bracketed by a pair
 // of HIP events on the stream it is launched on; tn_profile_summary adds the

@@ -141,6 +141,26 @@ static void gpu_checks() {
     (void)hipDeviceSynchronize();
     (void)hipMemcpy(w.data(), dw, w.size() * sizeof(float), hipMemcpyDeviceToHost);
     for (int i = 0; i < 1000; i++) EXPECT(std::fabs(w[i] - 0.9f) < 1e-5f);
+
+    // DenseTable::Save / Load: the file initialises a second table, and a second step on the
+    // copy equals a second step on the original (weights, moments and beta powers came along)
+    EXPECT(d->Save(ckpt) == TN_OK);
+    DenseTable* d2 = CreateDenseTable(adam, 1, 0);
+    const std::string from = ckpt + "/dense_table/" + std::to_string(d->GetHandle()) + "/0";
+    const std::string to_dir = ckpt + "/dense_table/" + std::to_string(d2->GetHandle());
+    EXPECT(d2->Load(ckpt) != TN_OK);  // no file for this handle yet
+    EXPECT(std::system(("mkdir -p " + to_dir + " && cp " + from + " " + to_dir + "/0").c_str()) == 0);
+    EXPECT(d2->Load(ckpt) == TN_OK);
+    EXPECT(d2->TotalElements() == 1000);
+    float* dw2 = nullptr;
+    (void)hipMalloc((void**)&dw2, 1000 * sizeof(float));
+    EXPECT(d->PushPull(dg, 0.1f, dw, 1000) == TN_OK);
+    EXPECT(d2->PushPull(dg, 0.1f, dw2, 1000) == TN_OK);
+    (void)hipDeviceSynchronize();
+    std::vector<float> w2(1000);
+    (void)hipMemcpy(w.data(), dw, w.size() * sizeof(float), hipMemcpyDeviceToHost);
+    (void)hipMemcpy(w2.data(), dw2, w2.size() * sizeof(float), hipMemcpyDeviceToHost);
+    for (int i = 0; i < 1000; i++) EXPECT(std::fabs(w[i] - w2[i]) < 1e-5f);
 }
 
 int main(int argc, char** argv) {
