@@ -321,7 +321,10 @@ int tn_sparse_table_last_unique_counts(uint32_t handle, int N, int64_t* counts);
 int tn_sparse_table_set_async(uint32_t handle, int async_pull);
 
 /* ------------------------------------------------------------- dense table */
-/* CreateDenseTable (core/ps/table/dense_table.cc:180-186); Adam or AdaGrad. */
+/* CreateDenseTable (core/ps/table/dense_table.cc:180-186); Adam or AdaGrad.  With shard_num > 1
+ * the table is worker self_shard_id's share: after Init it owns the contiguous range
+ * [id * ceil(total / shard_num), ...) of the concatenated parameters (DenseTable::Init,
+ * dense_table.cc:46-66); the other ranges live on other workers. */
 int tn_dense_table_create(tn_opt_t opt, int shard_num, int self_shard_id, uint32_t* handle);
 
 /*
@@ -346,17 +349,21 @@ int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const f
 /* DenseTable::TotalElements (core/ps/table/dense_table.h:44). */
 int tn_dense_table_total_elements(uint32_t handle, int64_t* total);
 
+/* DenseOptimizerKernelBase::OffsetBegin / OffsetEnd (optimizer_kernel.h:55-57): the range of
+ * the table this shard holds; [0, total) with one shard, empty for a shard past the end. */
+int tn_dense_table_range(uint32_t handle, int64_t* begin, int64_t* end);
+
 /* DenseOptimizerKernelBase::GetWeight / SetWeight (optimizer_kernel.h:63-65)
- * over the whole single-worker range; device pointers of total floats. */
+ * over the shard's range; device pointers of end - begin floats. */
 int tn_dense_table_get_weight(uint32_t handle, float* w, void* stream);
 int tn_dense_table_set_weight(uint32_t handle, const float* w, void* stream);
-/* Optimizer state read-back for tests: Adam m,v ; AdaGrad d2sum,g2sum,m (device, total floats each; NULL skips). */
+/* Optimizer state read-back for tests: Adam m,v ; AdaGrad d2sum,g2sum,m (device, end - begin floats each; NULL skips). */
 int tn_dense_table_get_state(uint32_t handle, float* s0, float* s1, float* s2, void* stream);
 
 /*
  * DenseTable::Save / Load (core/ps/table/dense_table.cc:103-157; py_wrapper.cc:221-230):
  * one text file <filepath>/dense_table/<handle>/<self_shard_id> holding the total, the
- * shard count and, per block of ceil(total / 8) elements, the optimizer's name, the
+ * shard count and, per block of ceil(range / 8) elements of the shard's range, the optimizer's name, the
  * block length, Adam's beta powers and one line of w and state per element, printed as
  * operator<< prints a float (6 significant digits).  Save of a table that was never
  * initialised writes nothing.  Load initialises the table to the file's total (an

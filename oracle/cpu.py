@@ -65,8 +65,8 @@ def load():
     lib.orc_dense_num_blocks.argtypes = [P]
     lib.orc_dense_get_state.argtypes = [P, C.c_int, P]
     lib.orc_dense_serialize.restype = C.c_int64
-    lib.orc_dense_serialize.argtypes = [P, C.c_int, P, C.c_int64]
-    lib.orc_dense_deserialize.argtypes = [P, C.c_int, P, C.c_int64]
+    lib.orc_dense_serialize.argtypes = [P, C.c_int, C.c_int, P, C.c_int64]
+    lib.orc_dense_deserialize.argtypes = [P, C.c_int, C.c_int, P, C.c_int64]
     lib.orc_dense_get_powers.argtypes = [P, C.c_int, P]
     _lib = lib
     return lib
@@ -300,18 +300,22 @@ class Dense(object):
         load().orc_dense_get_powers(self._h, block, _p(out))
         return float(out[0]), float(out[1])
 
-    def serialize(self, rank_num=1):
-        """Text of the checkpoint file DenseTable::Save writes (core/ps/table/dense_table.cc:103-128)."""
+    def serialize(self, rank_num=1, table_total=None):
+        """Text of the checkpoint file DenseTable::Save writes (core/ps/table/dense_table.cc:103-128).
+        With several shards this object is one shard's kernel (its range of the table) and
+        table_total the size of the whole table."""
         lib = load()
-        n = lib.orc_dense_serialize(self._h, rank_num, None, 0)
+        tt = self.total if table_total is None else int(table_total)
+        n = lib.orc_dense_serialize(self._h, rank_num, tt, None, 0)
         buf = np.zeros(max(1, n), dtype=np.uint8)
-        lib.orc_dense_serialize(self._h, rank_num, _p(buf), n)
+        lib.orc_dense_serialize(self._h, rank_num, tt, _p(buf), n)
         return buf[:n].tobytes()
 
-    def deserialize(self, data, shard_num=1):
+    def deserialize(self, data, shard_num=1, table_total=None):
         """DenseTable::Load (dense_table.cc:130-157) into a table of the file's total."""
         buf = np.ascontiguousarray(np.frombuffer(data, dtype=np.uint8))
-        rc = load().orc_dense_deserialize(self._h, shard_num, _p(buf), len(buf))
+        tt = self.total if table_total is None else int(table_total)
+        rc = load().orc_dense_deserialize(self._h, shard_num, tt, _p(buf), len(buf))
         if rc != 0:
             raise ValueError({-1: "total elements", -2: "shard count", -3: "optimizer", -4: "block length"}[rc]
                              + " of the checkpoint differs from the table's")

@@ -637,9 +637,11 @@ struct Dense {
     // table header, then DenseOptimizerKernel::Serialized (optimizer_kernel.h:224-229) =
     // per block "opt_name:" + value + endl (block stream, :139-146) + endl, the value being
     // DenseAdamValue's (adam_kernel.cc:57-69) or DenseAdaGradValue's (ada_grad_kernel.cc:50-60).
-    std::string Serialize(int rank_num) const {
+    // `total` here is the length of one shard's kernel; table_total is what the table of
+    // all shards holds (equal with one shard).
+    std::string Serialize(int rank_num, int table_total) const {
         std::ostringstream os;
-        os << "total_elements:" << (int)total << std::endl;
+        os << "total_elements:" << table_total << std::endl;
         os << "rank_num:" << rank_num << std::endl;
         for (const DenseBlock& b : blocks) {
             os << "opt_name:" << Name() << std::endl;
@@ -662,14 +664,14 @@ struct Dense {
     // DenseTable::Load (dense_table.cc:130-157) on a table created with the file's total;
     // returns 0, or -1 total / -2 rank_num / -3 optimizer / -4 block length mismatch (the
     // reference's CHECKs).  Value streams: adam_kernel.cc:71-87, ada_grad_kernel.cc:62-76.
-    int DeSerialize(const std::string& data, int shard_num) {
+    int DeSerialize(const std::string& data, int shard_num, int table_total) {
         std::istringstream is(data);
         const auto skip = std::numeric_limits<std::streamsize>::max();
         int total_elements = 0, rank_num = 0;
         is.ignore(skip, ':') >> total_elements;
         is.ignore(skip, ':') >> rank_num;
         if (shard_num != rank_num) return -2;
-        if (total_elements != (int)total) return -1;
+        if (total_elements != table_total) return -1;
         for (DenseBlock& b : blocks) {
             std::string name;
             is.ignore(skip, ':') >> name;
@@ -908,13 +910,14 @@ void orc_dense_set_weight(void* d, const float* w) { static_cast<Dense*>(d)->Set
 void orc_dense_get_weight(void* d, float* w) { static_cast<Dense*>(d)->GetWeight(w); }
 void orc_dense_apply(void* d, const float* grad, float lr) { static_cast<Dense*>(d)->Apply(grad, lr); }
 // The text of the table's checkpoint file.  Returns its size; copies it if cap suffices.
-int64_t orc_dense_serialize(void* dp, int rank_num, uint8_t* out, int64_t cap) {
-    const std::string s = static_cast<Dense*>(dp)->Serialize(rank_num);
+int64_t orc_dense_serialize(void* dp, int rank_num, int table_total, uint8_t* out, int64_t cap) {
+    const std::string s = static_cast<Dense*>(dp)->Serialize(rank_num, table_total);
     if ((int64_t)s.size() <= cap && out) std::memcpy(out, s.data(), s.size());
     return (int64_t)s.size();
 }
-int orc_dense_deserialize(void* dp, int shard_num, const uint8_t* data, int64_t n) {
-    return static_cast<Dense*>(dp)->DeSerialize(std::string(reinterpret_cast<const char*>(data), (size_t)n), shard_num);
+int orc_dense_deserialize(void* dp, int shard_num, int table_total, const uint8_t* data, int64_t n) {
+    return static_cast<Dense*>(dp)->DeSerialize(std::string(reinterpret_cast<const char*>(data), (size_t)n), shard_num,
+                                                table_total);
 }
 void orc_dense_get_powers(void* dp, int block, float* out) {
     const DenseBlock& b = static_cast<Dense*>(dp)->blocks[(size_t)block];

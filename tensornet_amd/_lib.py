@@ -128,6 +128,7 @@ SIGNATURES = {
     "tn_dense_table_init": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _P]),
     "tn_dense_table_push_pull": (C.c_int, [C.c_uint32, C.c_int, _PP, _PP, _I64P, C.c_float, _P]),
     "tn_dense_table_total_elements": (C.c_int, [C.c_uint32, _I64P]),
+    "tn_dense_table_range": (C.c_int, [C.c_uint32, _I64P, _I64P]),
     "tn_dense_table_get_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_set_weight": (C.c_int, [C.c_uint32, _P, _P]),
     "tn_dense_table_get_state": (C.c_int, [C.c_uint32, _P, _P, _P, _P]),

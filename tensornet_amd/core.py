@@ -98,10 +98,11 @@ def create_sparse_table(opt, name, dimension, use_cvm=False, embedding_group="")
     return h.value
 
 
-def create_dense_table(opt):
-    """py_wrapper.cc:182-191 -> CreateDenseTable (dense_table.cc:180-186)."""
+def create_dense_table(opt, shard_num=1, self_shard_id=0):
+    """py_wrapper.cc:182-191 -> CreateDenseTable (dense_table.cc:180-186).  The reference takes
+    the shard count and id from its cluster (RankNum, Rank); one worker is the default here."""
     h = C.c_uint32()
-    _lib.check(_lib.load().tn_dense_table_create(opt.handle, 1, 0, C.byref(h)))
+    _lib.check(_lib.load().tn_dense_table_create(opt.handle, int(shard_num), int(self_shard_id), C.byref(h)))
     return h.value
 
 

@@ -463,8 +463,8 @@ int load_table(uint32_t handle, const char* filepath, const char* mode) {
 
 // ------------------------------------------------------------------ dense table
 // DenseTable::Save / Load (core/ps/table/dense_table.cc:103-157): one plain text file
-//   <filepath>/dense_table/<handle>/<self_shard_id>
-//   "total_elements:<n>\n" "rank_num:<shards>\n", then per block of ceil(n / 8) elements
+//   <filepath>/dense_table/<handle>/<self_shard_id>     (the shard's own range of the table)
+//   "total_elements:<n>\n" "rank_num:<shards>\n", then per block of ceil(range / 8) elements
 //   (DenseOptimizerKernel, optimizer_kernel.h:174-188,224-235; block stream :139-160)
 //   "opt_name:<Name>\n" "array_size:<len>\n" [Adam: "beta1_power:<f>\n" "beta2_power:<f>\n"]
 //   one element per line, tab separated: Adam w m v (adam_kernel.cc:57-87), AdaGrad
@@ -480,20 +480,20 @@ int save_dense(uint32_t handle, const char* filepath) {
     if (!filepath) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: NULL path");
     DenseMeta m;
     TN_TRY(dense_meta(handle, m));
-    if (!m.initialized) return TN_OK;  // no kernel for this shard yet: nothing is written (dense_table.cc:106-109)
+    if (!m.initialized || m.length == 0) return TN_OK;  // no kernel for this shard: nothing is written (dense_table.cc:106-109)
     const std::string file = dense_file(handle, filepath, m);
     TN_TRY(make_dirs(file.substr(0, file.rfind('/'))));
     FILE* f = std::fopen(file.c_str(), "wb");
     if (!f) return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_save: cannot write " + file);
     const int arrays = m.kind == OPT_ADAM ? 3 : 4;
     std::vector<float> host[4];
-    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, m.total));
+    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, m.length));
     float* arr[4] = {host[0].data(), host[1].data(), host[2].data(), arrays == 4 ? host[3].data() : nullptr};
     std::string out = "total_elements:" + std::to_string(m.total) + "\nrank_num:" + std::to_string(m.shard_num) + "\n";
-    const int64_t per_block = (m.total + kDenseBlocks - 1) / kDenseBlocks;
+    const int64_t per_block = (m.length + kDenseBlocks - 1) / kDenseBlocks;
     int rc = TN_OK;
-    for (int64_t b0 = 0; b0 < m.total && rc == TN_OK; b0 += per_block) {
-        const int64_t len = std::min(per_block, m.total - b0);
+    for (int64_t b0 = 0; b0 < m.length && rc == TN_OK; b0 += per_block) {
+        const int64_t len = std::min(per_block, m.length - b0);
         out += std::string("opt_name:") + opt_name(m.kind) + "\narray_size:" + std::to_string(len) + "\n";
         if (m.kind == OPT_ADAM) {
             out += "beta1_power:";
@@ -559,15 +559,17 @@ int load_dense(uint32_t handle, const char* filepath) {
         return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_load: file written by " + std::to_string(rank_num) +
                                                  " shards, table has " + std::to_string(m.shard_num));
     TN_TRY(dense_ensure_init(handle, total));  // CHECK_EQ(0, Init(total_elements_)), :142
+    TN_TRY(dense_meta(handle, m));
+    const int64_t length = m.length;  // this shard's range; without a kernel nothing more is read (:144-147)
     const int arrays = m.kind == OPT_ADAM ? 3 : 4;
     std::vector<float> host[4];
-    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, total));
+    for (int a = 0; a < arrays; a++) host[a].resize((size_t)std::min<int64_t>(kDenseChunk, std::max<int64_t>(length, 1)));
     float* arr[4] = {host[0].data(), host[1].data(), host[2].data(), arrays == 4 ? host[3].data() : nullptr};
-    const int64_t per_block = (total + kDenseBlocks - 1) / kDenseBlocks;
+    const int64_t per_block = (length + kDenseBlocks - 1) / kDenseBlocks;
     bool have_powers = false;
     float b1p = 1.f, b2p = 1.f;
-    for (int64_t b0 = 0; b0 < total; b0 += per_block) {
-        const int64_t len = std::min(per_block, total - b0);
+    for (int64_t b0 = 0; b0 < length; b0 += per_block) {
+        const int64_t len = std::min(per_block, length - b0);
         if (!after_colon(tk, tok)) return fail(TN_ERR_INVALID_ARGUMENT, bad);
         if (tok != opt_name(m.kind))  // optimizer_kernel.h:153-155
             return fail(TN_ERR_INVALID_ARGUMENT, "last trained model with optimizer is:" + tok +

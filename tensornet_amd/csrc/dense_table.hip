@@ -8,8 +8,14 @@
 // is bound by HBM bandwidth.  One thread handles one float4 of each array.
 // The reference's 8 blocks all step together on a single worker, so their
 // beta powers are identical and one pair is kept on the host.
+//
+// With shard_num > 1 the table is one worker's share: it holds the contiguous
+// range [begin, end) of the concatenated parameters (ceil(total / shard_num)
+// per shard), applies that slice of the gradients and writes that slice of
+// the variables; the other ranges belong to other workers.
 #include "tn_common.h"
 
+#include <algorithm>
 #include <cmath>
 
 namespace tn {
@@ -22,7 +28,8 @@ struct DenseTable {
     uint32_t handle = 0;
     int device = 0;
     bool initialized = false;
-    int64_t total = 0;
+    int64_t total = 0;           // elements of the whole table (all shards)
+    int64_t begin = 0, end = 0;  // this shard's range of it (dense_table.cc:46-66); arrays hold end - begin
     float* w = nullptr;
     float* s0 = nullptr;  // Adam m      / AdaGrad d2sum
     float* s1 = nullptr;  // Adam v      / AdaGrad g2sum
@@ -134,6 +141,7 @@ int dense_meta(uint32_t handle, DenseMeta& m) {
     m.self_shard_id = t->self_shard_id;
     m.initialized = t->initialized;
     m.total = t->total;
+    m.length = t->end - t->begin;
     m.beta1_power = t->beta1_power;
     m.beta2_power = t->beta2_power;
     return TN_OK;
@@ -153,7 +161,7 @@ int dense_copy_range(uint32_t handle, int64_t off, int64_t n, float* const arr[4
     if (!t) return fail(TN_ERR_BAD_HANDLE, "bad dense table handle " + std::to_string(handle));
     std::lock_guard<std::mutex> lk(t->mu);
     if (!t->initialized) return fail(TN_ERR_NOT_INIT, "dense table not initialised");
-    if (off < 0 || n < 0 || off + n > t->total) return fail(TN_ERR_INVALID_ARGUMENT, "dense table range out of bounds");
+    if (off < 0 || n < 0 || off + n > t->end - t->begin) return fail(TN_ERR_INVALID_ARGUMENT, "dense table range out of bounds");
     float* dev[4] = {t->w, t->s0, t->s1, t->s2};
     for (int a = 0; a < 4; a++) {
         if (!dev[a] || !arr[a] || n == 0) continue;
@@ -177,8 +185,9 @@ int tn_dense_table_create(tn_opt_t opt, int shard_num, int self_shard_id, uint32
     if (!conf) return fail(TN_ERR_BAD_HANDLE, "tn_dense_table_create: unknown optimizer handle");
     if (conf->kind == OPT_FTRL)
         return fail(TN_ERR_UNSUPPORTED, "tn_dense_table_create: dense Ftrl is an empty stub in the reference");
-    if (shard_num != 1 || self_shard_id != 0)
-        return fail(TN_ERR_UNSUPPORTED, "tn_dense_table_create: one worker only (shard_num 1, self_shard_id 0)");
+    if (shard_num < 1 || self_shard_id < 0 || self_shard_id >= shard_num)
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_dense_table_create: shard " + std::to_string(self_shard_id) + " of " +
+                                                 std::to_string(shard_num));
     DenseTable* t = new DenseTable();
     t->opt = conf;
     t->shard_num = shard_num;
@@ -201,19 +210,27 @@ static int dense_alloc(DenseTable* t, int64_t total, hipStream_t st) {
     if (total <= 0) return fail(TN_ERR_INVALID_ARGUMENT, "dense table init: total elements must be positive");
     if (total > 0x7fffffffLL)
         return fail(TN_ERR_INVALID_ARGUMENT, "dense table init: total elements exceed int (dense_table.cc:37)");
-    size_t bytes = (size_t)total * sizeof(float);
-    TN_HIP(hipMalloc((void**)&t->w, bytes));
-    TN_HIP(hipMalloc((void**)&t->s0, bytes));
-    TN_HIP(hipMalloc((void**)&t->s1, bytes));
-    int blocks = launch_grid(total, 256, 8192);
-    TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->w, total, 0.f);
-    TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s0, total, 0.f);
-    if (t->opt->kind == OPT_ADAGRAD) {
-        TN_HIP(hipMalloc((void**)&t->s2, bytes));
-        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, total, t->opt->initial_g2sum);
-        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s2, total, 0.f);
-    } else {
-        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, total, 0.f);
+    // DenseTable::Init, dense_table.cc:46-66: ceil(total / shards) elements per shard, the last
+    // one shorter; a shard that starts past the end gets no kernel
+    const int64_t every = (total + t->shard_num - 1) / t->shard_num;
+    t->begin = std::min<int64_t>((int64_t)t->self_shard_id * every, total);
+    t->end = std::min<int64_t>(t->begin + every, total);
+    const int64_t len = t->end - t->begin;
+    if (len > 0) {
+        size_t bytes = (size_t)len * sizeof(float);
+        TN_HIP(hipMalloc((void**)&t->w, bytes));
+        TN_HIP(hipMalloc((void**)&t->s0, bytes));
+        TN_HIP(hipMalloc((void**)&t->s1, bytes));
+        int blocks = launch_grid(len, 256, 8192);
+        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->w, len, 0.f);
+        TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s0, len, 0.f);
+        if (t->opt->kind == OPT_ADAGRAD) {
+            TN_HIP(hipMalloc((void**)&t->s2, bytes));
+            TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, len, t->opt->initial_g2sum);
+            TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s2, len, 0.f);
+        } else {
+            TN_LAUNCH(k_fill_f32, dim3(blocks), dim3(256), st, t->s1, len, 0.f);
+        }
     }
     TN_HIP(hipGetLastError());
     t->total = total;
@@ -249,9 +266,10 @@ int tn_dense_table_init(uint32_t handle, int N, const float* const* vars, const 
     TN_TRY(dense_alloc(t, total, st));
     int64_t off = 0;
     for (int i = 0; i < N; i++) {
-        if (var_lens[i] > 0)
-            TN_HIP(hipMemcpyAsync(t->w + off, vars[i], (size_t)var_lens[i] * sizeof(float), hipMemcpyDeviceToDevice,
-                                  st));
+        const int64_t lo = std::max(off, t->begin), hi = std::min(off + var_lens[i], t->end);
+        if (lo < hi)
+            TN_HIP(hipMemcpyAsync(t->w + (lo - t->begin), vars[i] + (lo - off), (size_t)(hi - lo) * sizeof(float),
+                                  hipMemcpyDeviceToDevice, st));
         off += var_lens[i];
     }
     TN_HIP(hipStreamSynchronize(st));
@@ -294,12 +312,16 @@ int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const f
         ga.c = (float)(1.0 - (double)o.mom_decay_rate);
         ga.eps = o.epsilon;
     }
-    int64_t off = 0;
+    int64_t var_off = 0;
     for (int i = 0; i < N; i++) {
-        int64_t n = lens[i];
-        if (n == 0) continue;
-        float* out = vars ? vars[i] : nullptr;
-        const float* g = grads[i];
+        // the part of variable i inside this shard's range
+        const int64_t lo = std::max(var_off, t->begin), hi = std::min(var_off + lens[i], t->end);
+        const int64_t skip = lo - var_off;
+        var_off += lens[i];
+        if (lo >= hi) continue;
+        const int64_t n = hi - lo, off = lo - t->begin;
+        float* out = (vars && vars[i]) ? vars[i] + skip : nullptr;
+        const float* g = grads[i] + skip;
         if (o.kind == OPT_ADAM) {
             bool vec = (off % 4 == 0) && aligned16(g) && (!out || aligned16(out));
             int64_t n4 = vec ? n / 4 : 0;
@@ -316,7 +338,6 @@ int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const f
             int blocks = launch_grid(n, 256, 1 << 20);
             TN_LAUNCH(k_dense_adagrad_s, dim3(blocks), dim3(256), st, g, t->w + off, t->s0 + off, t->s1 + off, t->s2 + off, out, n, ga);
         }
-        off += n;
     }
     TN_HIP(hipGetLastError());
     return TN_OK;
@@ -329,12 +350,24 @@ int tn_dense_table_total_elements(uint32_t handle, int64_t* total) {
     return TN_OK;
 }
 
+int tn_dense_table_range(uint32_t handle, int64_t* begin, int64_t* end) {
+    DenseTable* t = get_dense(handle);
+    if (!t || !begin || !end) return fail(TN_ERR_BAD_HANDLE, "tn_dense_table_range: bad handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (!t->initialized) return fail(TN_ERR_NOT_INIT, "tn_dense_table_range: dense table not initialised");
+    *begin = t->begin;
+    *end = t->end;
+    return TN_OK;
+}
+
 int tn_dense_table_get_weight(uint32_t handle, float* w, void* stream) {
     DenseTable* t = get_dense(handle);
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_dense_table_get_weight: bad handle");
     std::lock_guard<std::mutex> lk(t->mu);
     if (!t->initialized) return fail(TN_ERR_NOT_INIT, "tn_dense_table_get_weight: dense table not initialised");
-    TN_HIP(hipMemcpyAsync(w, t->w, (size_t)t->total * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    if (t->end > t->begin)
+        TN_HIP(hipMemcpyAsync(w, t->w, (size_t)(t->end - t->begin) * sizeof(float), hipMemcpyDeviceToDevice,
+                              (hipStream_t)stream));
     return TN_OK;
 }
 
@@ -343,7 +376,9 @@ int tn_dense_table_set_weight(uint32_t handle, const float* w, void* stream) {
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_dense_table_set_weight: bad handle");
     std::lock_guard<std::mutex> lk(t->mu);
     if (!t->initialized) return fail(TN_ERR_NOT_INIT, "tn_dense_table_set_weight: dense table not initialised");
-    TN_HIP(hipMemcpyAsync(t->w, w, (size_t)t->total * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    if (t->end > t->begin)
+        TN_HIP(hipMemcpyAsync(t->w, w, (size_t)(t->end - t->begin) * sizeof(float), hipMemcpyDeviceToDevice,
+                              (hipStream_t)stream));
     return TN_OK;
 }
 
@@ -352,8 +387,9 @@ int tn_dense_table_get_state(uint32_t handle, float* s0, float* s1, float* s2, v
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_dense_table_get_state: bad handle");
     std::lock_guard<std::mutex> lk(t->mu);
     if (!t->initialized) return fail(TN_ERR_NOT_INIT, "tn_dense_table_get_state: dense table not initialised");
-    size_t bytes = (size_t)t->total * sizeof(float);
+    size_t bytes = (size_t)(t->end - t->begin) * sizeof(float);
     hipStream_t st = (hipStream_t)stream;
+    if (bytes == 0) return TN_OK;
     if (s0) TN_HIP(hipMemcpyAsync(s0, t->s0, bytes, hipMemcpyDeviceToDevice, st));
     if (s1) TN_HIP(hipMemcpyAsync(s1, t->s1, bytes, hipMemcpyDeviceToDevice, st));
     if (s2 && t->s2) TN_HIP(hipMemcpyAsync(s2, t->s2, bytes, hipMemcpyDeviceToDevice, st));

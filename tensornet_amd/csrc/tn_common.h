@@ -128,14 +128,15 @@ struct DenseMeta {
     int kind;  // OPT_ADAM / OPT_ADAGRAD
     int shard_num, self_shard_id;
     bool initialized;
-    int64_t total;
+    int64_t total;   // elements of the whole table
+    int64_t length;  // elements of this shard's range
     float beta1_power, beta2_power;
 };
 int dense_meta(uint32_t handle, DenseMeta& m);
 // DenseTable::Init(total): allocates on first use, a different size afterwards is an error.
 int dense_ensure_init(uint32_t handle, int64_t total);
 int dense_set_powers(uint32_t handle, float beta1_power, float beta2_power);
-// Copies elements [off, off + n) between the table's arrays and host arrays: arr[0] = w,
+// Copies elements [off, off + n) of the shard's range between the table's arrays and host arrays: arr[0] = w,
 // arr[1..3] = the optimizer's state arrays in the order its value prints them (Adam m, v;
 // AdaGrad d2sum, g2sum, m); arrays the optimizer lacks are skipped.
 int dense_copy_range(uint32_t handle, int64_t off, int64_t n, float* const arr[4], bool to_host);

@@ -342,18 +342,23 @@ def table_delete_by_show(table_handle, signs):
     return out
 
 
+def dense_table_range(table_handle):
+    """(begin, end) of the table's elements this shard holds (optimizer_kernel.h:55-57)."""
+    b, e = C.c_int64(), C.c_int64()
+    _lib.check(_lib.load().tn_dense_table_range(table_handle, C.byref(b), C.byref(e)))
+    return b.value, e.value
+
+
 def dense_table_get_weight(table_handle, device="cuda"):
-    total = C.c_int64()
-    _lib.check(_lib.load().tn_dense_table_total_elements(table_handle, C.byref(total)))
-    w = torch.empty((total.value,), dtype=torch.float32, device=device)
+    b, e = dense_table_range(table_handle)
+    w = torch.empty((e - b,), dtype=torch.float32, device=device)
     _lib.check(_lib.load().tn_dense_table_get_weight(table_handle, w.data_ptr(), _stream()))
     return w
 
 
 def dense_table_get_state(table_handle, n_states=2, device="cuda"):
-    total = C.c_int64()
-    _lib.check(_lib.load().tn_dense_table_total_elements(table_handle, C.byref(total)))
-    outs = [torch.empty((total.value,), dtype=torch.float32, device=device) for _ in range(n_states)]
+    b, e = dense_table_range(table_handle)
+    outs = [torch.empty((e - b,), dtype=torch.float32, device=device) for _ in range(n_states)]
     ptrs = [o.data_ptr() for o in outs] + [None] * (3 - n_states)
     _lib.check(_lib.load().tn_dense_table_get_state(table_handle, ptrs[0], ptrs[1], ptrs[2], _stream()))
     return outs

@@ -77,6 +77,8 @@ def test_dense_errors(tn):
     assert e.value.code == 3
     with pytest.raises(tn.TensorNetError):
         tn.core.create_dense_table(tn.core.Ftrl())
+    with pytest.raises(tn.TensorNetError):
+        tn.core.create_dense_table(tn.core.Adam(), 2, 2)  # shard id outside the shard count
 
 
 def test_dense_full_size_properties(tn):

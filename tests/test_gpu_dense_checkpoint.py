@@ -128,3 +128,62 @@ def test_dense_checkpoint_errors(tn, oracle, tmp_path):
     put(cut, text[: len(text) // 2])
     with pytest.raises(tn.TensorNetError, match="malformed"):
         tn.core.load_dense_table(cut, tmp_path)
+
+
+@pytest.mark.parametrize("kind", ["adam", "adagrad"])
+@pytest.mark.parametrize("total,shards", [(1003, 3), (10, 4), (5, 8)])
+def test_shards_of_one_table(tn, oracle, kind, total, shards, tmp_path):
+    """A table cut into shards (DenseTable::Init, dense_table.cc:46-66): every shard updates
+    its own range of the variables, all shards together equal the unsharded oracle table,
+    and each writes its own checkpoint file."""
+    rng = np.random.default_rng(total * shards)
+    every = -(-total // shards)
+    w0 = rng.uniform(-0.05, 0.05, total).astype(np.float32)
+    sizes = [total // 3, total - total // 3]  # two variables; the shard borders cut through them
+    cuts = [(0, sizes[0]), (sizes[0], total)]
+    _, (okind, hp) = make(tn, oracle, kind)
+    whole = oracle.Dense(okind, total, **hp)
+    whole.set_weight(w0)
+    tables, ranges = [], []
+    for r in range(shards):
+        opt = tn.core.Adam(learning_rate=1e-3, **hp) if kind == "adam" else tn.core.AdaGrad(**hp)
+        h = tn.core.create_dense_table(opt, shards, r)
+        tn.ops.dense_table_init([dev(w0[a:b]) for a, b in cuts], h)
+        b, e = tn.ops.dense_table_range(h)
+        assert (b, e) == (min(r * every, total), min((r + 1) * every, total))
+        tables.append(h)
+        ranges.append((b, e))
+    merged = w0.copy()
+    for step in range(3):
+        g = (rng.standard_normal(total) * 1e-2).astype(np.float32)
+        whole.apply(g, 0.01)
+        for h, (b, e) in zip(tables, ranges):
+            vars_ = [torch.full((n,), 7.0, device="cuda") for n in sizes]
+            tn.ops.dense_table_push_pull(vars_, [dev(g[a:c]) for a, c in cuts], 0.01, h)
+            got = torch.cat(vars_).cpu().numpy()
+            outside = np.ones(total, bool)
+            outside[b:e] = False
+            assert (got[outside] == 7.0).all()  # other shards' ranges are not this worker's to write
+            merged[b:e] = got[b:e]
+    np.testing.assert_allclose(merged, whole.get_weight(), rtol=RTOL, atol=ATOL)
+    for r, (h, (b, e)) in enumerate(zip(tables, ranges)):
+        np.testing.assert_array_equal(tn.ops.dense_table_get_weight(h).cpu().numpy(), merged[b:e])
+        tn.core.save_dense_table(h, tmp_path)
+        path = os.path.join(str(tmp_path), "dense_table", str(h), str(r))
+        if e == b:
+            assert not os.path.exists(path)  # a shard past the end has no kernel and writes nothing
+            continue
+        text = open(path).read()
+        assert text.startswith("total_elements:%d\nrank_num:%d\n" % (total, shards))
+        part = oracle.Dense(okind, e - b, **hp)
+        part.deserialize(text.encode(), shard_num=shards, table_total=total)
+        np.testing.assert_array_equal(part.get_weight(), np.array([float("%g" % x) for x in merged[b:e]], np.float32))
+        # a fresh shard table takes the file back
+        opt = tn.core.Adam(learning_rate=1e-3, **hp) if kind == "adam" else tn.core.AdaGrad(**hp)
+        h2 = tn.core.create_dense_table(opt, shards, r)
+        os.makedirs(os.path.join(str(tmp_path), "dense_table", str(h2)), exist_ok=True)
+        with open(os.path.join(str(tmp_path), "dense_table", str(h2), str(r)), "w") as f:
+            f.write(text)
+        tn.core.load_dense_table(h2, tmp_path)
+        assert tn.ops.dense_table_range(h2) == (b, e)
+        np.testing.assert_array_equal(tn.ops.dense_table_get_weight(h2).cpu().numpy(), part.get_weight())

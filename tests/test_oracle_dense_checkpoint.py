@@ -66,3 +66,12 @@ def test_mismatches_are_refused():
         oracle.Dense(oracle.ADAGRAD, 16).deserialize(text)
     with pytest.raises(ValueError, match="shard"):
         oracle.Dense(oracle.ADAM, 16).deserialize(text, shard_num=2)
+
+
+def test_shard_file_header_names_the_whole_table():
+    # shard 1 of 3 over 10 elements holds [4, 8): ceil(10 / 3) = 4 per shard (dense_table.cc:46-60)
+    d = oracle.Dense(oracle.ADAGRAD, 4)
+    text = d.serialize(rank_num=3, table_total=10).decode()
+    assert text.startswith("total_elements:10\nrank_num:3\nopt_name:AdaGrad\narray_size:1\n")
+    assert text.count("array_size:1\n") == 4  # ceil(4 / 8) = 1 element per block
+    oracle.Dense(oracle.ADAGRAD, 4).deserialize(text.encode(), shard_num=3, table_total=10)
