@@ -102,8 +102,7 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
         "k_probe": 8 * G + 4 * G,              # one stored-key compare per distinct sign, row number out
         "k_gather_vars": U * (2 * row + 4),    # row read + variable row write
         # push
-        "k_verify_values": 16 * L,             # the op's signs against the pull's copy
-        "k_count_click": 8 * L,                # labels
+        "k_verify_values": 24 * L,             # the op's signs against the pull's copy, labels
         "k_reset_counts": 8 * U,
         "k_apply_single": apply_bytes(shape["G1"], shape["G1"]),
         "k_apply_vec": apply_bytes(shape["Rm"], shape["Gm"]),

@@ -694,23 +694,6 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
     }
 }
 
-// Push on a plan whose member lists already hold the show counts: the click
-// sums are cleared (k_reset_counts) and the non-zero labels added
-// (sparse_table_ops.cc:283-296).
-__global__ __launch_bounds__(256) void k_count_click(const SlotDesc* __restrict__ descs,
-                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     const uint32_t* __restrict__ u_of_gi,
-                                                     const uint2* __restrict__ where_u, Member* list) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
-    load_lbase(lb, lbase, N);
-    const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        const int sl = find_slot(lb, N, gi);
-        const int label = (int)descs[sl].labels[gi - lb[sl]];
-        if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
-    }
-}
-
 }  // namespace tn
 
 #endif  // TN_REMAP_LDS_H_

@@ -763,22 +763,27 @@ __global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict
     }
 }
 
-// Push: are the signs of this call the ones the plan was built from?  With
-// list != nullptr the same pass starts the click sums of the plan's member
-// lists at zero (the show counts of the pull stay), as k_reset_counts would.
+// Push: are the signs of this call the ones the plan was built from?  With CLICKS the same
+// pass adds the non-zero labels to the click sums of the plan's member lists, which start
+// at zero (sparse_table_ops.cc:283-296; on a mismatch the plan is discarded anyway).
+template <bool CLICKS>
 __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                        const uint64_t* __restrict__ vals_copy, DevStatus* status,
-                                                       Member* __restrict__ list) {
+                                                       const uint32_t* __restrict__ u_of_gi,
+                                                       const uint2* __restrict__ where_u, Member* list) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
-    const uint32_t n_single = status->n_single, n_members = status->n_members;
     bool bad = false;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
         const int sl = find_slot(lb, N, gi);
-        bad |= (uint64_t)descs[sl].values[gi - lb[sl]] != vals_copy[gi];
-        if (list && gi < n_single + n_members) list[group_id(gi, n_single, n_members, L)].click = 0;
+        const SlotDesc& d = descs[sl];
+        bad |= (uint64_t)d.values[gi - lb[sl]] != vals_copy[gi];
+        if (CLICKS) {
+            const int label = (int)d.labels[gi - lb[sl]];
+            if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
+        }
     }
     if (bad) atomicOr(&status->mismatch, 1u);
 }

@@ -60,6 +60,7 @@ struct SparseTable {
     DevBuf pooled_ws;               // scratch of a push of pooled gradients (sort buffers, reduced rows)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipEvent_t fork_ev = nullptr, join_ev = nullptr;
+    bool plan_clicks_dirty = false;  // a push has added clicks to the member lists of the current plan
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
     bool pull_pending = false;
@@ -1185,6 +1186,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         t->pending_rows.assign(var_rows, var_rows + N);
         // a push of the same batch may reuse the analysis
         t->plan_valid = true;
+        t->plan_clicks_dirty = false;  // a new plan's click sums start at zero
         t->plan_has_show = use_lds;
         t->plan_N = N;
         t->plan_lens.assign(value_lens, value_lens + N);
@@ -1261,20 +1263,11 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     DevStatus* ds = t->dplan;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
     const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
-    // show / click counts of the batch into the member lists of plan p
-    auto launch_counts = [&](bool has_show) -> int {
-        if (has_show) {
-            if (with_click) {
-                TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
-                TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
-                          p.where_u, p.list);
-            }
-        } else {
-            TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
-            TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)),
-                      dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.where_u, p.list,
-                      with_click ? 1 : 0);
-        }
+    // show / click counts of the batch into the member lists of a plan that has none
+    auto launch_counts = [&]() -> int {
+        TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
+        TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256),
+                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.where_u, p.list, with_click ? 1 : 0);
         return TN_OK;
     };
     // Where the apply kernels find the gradient of a record.  Pooled gradients are first reduced
@@ -1336,20 +1329,27 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_REUSE_PLAN));
-        const bool clicks = t->plan_has_show && with_click;  // the verify pass also clears the click sums
-        TN_LAUNCH(k_verify_values, dim3(launch_grid(L, 256, GRID_CAP * 2)), dim3(256), st, p.descs, p.lbase, N,
-                  (uint32_t)L, p.vals_copy, ds, clicks ? p.list : (Member*)nullptr);
+        // On a plan with show counts the verify pass also sums the clicks; they start at zero
+        // after the pull, a further push on the same plan clears them first.
+        const bool clicks = t->plan_has_show && with_click;
+        const int vblocks = launch_grid(L, 256, GRID_CAP * 2);
+        if (clicks) {
+            if (t->plan_clicks_dirty)
+                TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
+            t->plan_clicks_dirty = true;
+            TN_LAUNCH((k_verify_values<true>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.vals_copy,
+                      ds, p.u_of_gi, p.where_u, p.list);
+        } else {
+            TN_LAUNCH((k_verify_values<false>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L,
+                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list);
+        }
         TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush),
                   (unsigned long long*)nullptr);
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // Counts and apply kernels are queued before the host knows the outcome: the counts only
         // touch the plan's member lists, which a mismatch discards anyway, and the apply kernels
         // return at once when the mismatch flag is set.  The device never waits for the host.
-        if (clicks)
-            TN_LAUNCH(k_count_click, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi,
-                      p.where_u, p.list);
-        else
-            TN_TRY(launch_counts(t->plan_has_show));
+        if (!t->plan_has_show) TN_TRY(launch_counts());
         TN_TRY(prepare_src());
         TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
         TN_HIP(hipEventSynchronize(t->verify_ev));
@@ -1365,7 +1365,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st));
-        TN_TRY(launch_counts(false));
+        TN_TRY(launch_counts());
         TN_TRY(prepare_src());
         TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
     }
