@@ -621,3 +621,21 @@ def test_cfg3_full_batch_against_the_oracle(tn, oracle):
     pair.push_op(values, grads, labels)
     assert pair.assert_rows_match(signs) > 0.99
     check_pull(pair, values)
+
+
+def test_two_pushes_on_one_pull_count_their_own_clicks(tn, oracle):
+    """A pull followed by two pushes of the same batch with different labels (the plan of the
+    pull serves both): every push adds its own click sums, not the sum of both."""
+    D = 8
+    rng = np.random.default_rng(77)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, use_cvm=True, reserve=200000)
+    vocab = 20000
+    pool = synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool.view(np.uint64))
+    values = [pool[rng.integers(0, vocab, 3000)] for _ in range(16)]  # 48000 lookups: the LDS path
+    counts = check_pull(pair, values, loose_col=D + 1)
+    for push in range(2):
+        grads = [(rng.standard_normal((int(u), D + 2)) * 0.01).astype(np.float32) for u in counts]
+        labels = [rng.integers(0, 3, len(v)).astype(np.int64) for v in values]
+        pair.push_op(values, grads, labels)
+        pair.assert_rows_match(all_signs(values))
