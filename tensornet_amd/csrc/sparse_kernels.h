@@ -193,7 +193,13 @@ __device__ __forceinline__ uint32_t group_id(uint32_t i, uint32_t n_single, uint
     return i < n_single ? i : ids_cap - n_multi + (i - n_single);
 }
 
-constexpr int PROBE_WIDTH = 4;
+constexpr int PROBE_WIDTH = 8;
+static_assert(PROBE_WIDTH == 8, "probe_slot reads a group as four 16-byte loads");
+
+// First slot of the aligned group of PROBE_WIDTH slots that holds the home slot of a sign.
+__device__ __forceinline__ uint64_t home_group(uint64_t sign, uint64_t cap) {
+    return slot_of(sign, cap) & ~(uint64_t)(PROBE_WIDTH - 1);
+}
 
 __device__ __forceinline__ void init_row(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row);
 
@@ -210,31 +216,29 @@ __device__ __forceinline__ uint32_t probe_slot(const Store& s, uint64_t sign, bo
         }
         return ld_relaxed(s.special) ? (uint32_t)s.cap : NO_ROW;
     }
-    // PROBE_WIDTH consecutive slots per round trip: their loads are issued together, so a
-    // probe sequence of a few slots costs one memory latency instead of one per slot.
-    uint64_t idx = slot_of(sign, s.cap);
+    // Linear probing in aligned groups of PROBE_WIDTH slots, starting at the group of the home
+    // slot (the capacity is a multiple of PROBE_WIDTH): a group is one 64-byte granule, read
+    // with four 16-byte loads in one round trip, and at a load of 0.75 few probes need a second
+    // group.  Unaligned windows straddle granule boundaries and were measured at half the rate.
+    uint64_t idx = home_group(sign, s.cap);
     for (uint64_t p = 0; p < s.cap; p += PROBE_WIDTH) {
-        uint64_t at[PROBE_WIDTH], k[PROBE_WIDTH];
+        // plain loads: a key never changes once set, and a stale free slot is settled by the compare-and-swap
+        const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + idx);
+        const ulonglong2 q0 = g[0], q1 = g[1], q2 = g[2], q3 = g[3];
+        const uint64_t k[PROBE_WIDTH] = {q0.x, q0.y, q1.x, q1.y, q2.x, q2.y, q3.x, q3.y};
 #pragma unroll
         for (int j = 0; j < PROBE_WIDTH; j++) {
-            at[j] = idx + j;
-            if (at[j] >= s.cap) at[j] -= s.cap;
-            // plain load: a key never changes once set, and a stale free slot is settled by the compare-and-swap
-            k[j] = s.keys[at[j]];
-        }
-#pragma unroll
-        for (int j = 0; j < PROBE_WIDTH; j++) {
-            if (k[j] == sign) return (uint32_t)at[j];
+            if (k[j] == sign) return (uint32_t)(idx + j);
             if (k[j] == EMPTY_KEY) {
                 if (!INSERT) return NO_ROW;
-                uint64_t old = atomicCAS(ull(&s.keys[at[j]]), EMPTY_KEY, sign);
+                uint64_t old = atomicCAS(ull(&s.keys[idx + j]), EMPTY_KEY, sign);
                 if (old == EMPTY_KEY || old == sign) {
                     is_new = old == EMPTY_KEY;
-                    return (uint32_t)at[j];
+                    return (uint32_t)(idx + j);
                 }
             }
         }
-        idx = at[PROBE_WIDTH - 1] + 1 == s.cap ? 0 : at[PROBE_WIDTH - 1] + 1;
+        idx = idx + PROBE_WIDTH >= s.cap ? 0 : idx + PROBE_WIDTH;
     }
     return NO_ROW;
 }
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(256) void k_rehash(Store from, Store to, DevStatus*
         } else {
             const uint64_t sign = from.keys[i];
             if (sign == EMPTY_KEY) continue;
-            uint64_t idx = slot_of(sign, to.cap);
+            uint64_t idx = home_group(sign, to.cap);  // the probe sequence of probe_slot
             dst = EMPTY_KEY;
             for (uint64_t p = 0; p < to.cap; ++p) {
                 uint64_t old = atomicCAS(ull(&to.keys[idx]), EMPTY_KEY, sign);

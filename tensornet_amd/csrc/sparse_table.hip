@@ -135,6 +135,7 @@ int state_floats(const SparseTable* t) { return (t->opt->kind == OPT_ADAGRAD) ? 
 int alloc_store(const SparseTable* t, uint64_t cap, Store& s, hipStream_t st) {
     layout(t, s);
     if (cap < 64) cap = 64;
+    cap = (cap + PROBE_WIDTH - 1) / PROBE_WIDTH * PROBE_WIDTH;  // probing goes by aligned groups of slots
     if (cap > MAX_SLOTS_PER_TABLE) return fail(TN_ERR_UNSUPPORTED, "sparse table: more than 2^32 slots");
     s.cap = cap;
     choose_strides(s, cap);
