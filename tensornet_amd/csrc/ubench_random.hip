@@ -1,7 +1,9 @@
 // Random-access ceilings of the device for the access patterns of the sparse table:
 // a stand-alone program (no library code) that times, on a table-sized allocation,
 //
-//   read64    64 bytes of a random 128-byte-pitch row, 4 lanes per row        (the gather)
+//   read64    64 bytes of a random 128-byte-pitch row, 4 lanes per row
+//   gather    the same rows in random order, each copied to the next 64 bytes of
+//             a dense array                                                   (k_gather_vars)
 //   rmw80     64 + 16 bytes of a random row read, updated and written back     (an update)
 //   apply     the same through an index array, with a 64-byte gradient row
 //             gathered from a second array                                     (k_apply_single)
@@ -71,6 +73,17 @@ __global__ __launch_bounds__(256) void k_rows(float* tab, uint64_t rows, uint64_
         }
     }
     if (acc == 1.2345f) sink[0] = acc;
+}
+
+// rows in random order (the order of the distinct indices of a batch), dense output
+__global__ __launch_bounds__(256) void k_gather(const float* __restrict__ tab, uint64_t rows, uint64_t n,
+                                                float* __restrict__ dense) {
+    const int sub = threadIdx.x & 3;
+    const uint64_t stride = (uint64_t)gridDim.x * 64;
+    for (uint64_t i = (uint64_t)blockIdx.x * 64 + (threadIdx.x >> 2); i < n; i += stride) {
+        const uint64_t r = __umul64hi(mix64(i + 1), rows);
+        reinterpret_cast<float4*>(dense + i * 16)[sub] = reinterpret_cast<const float4*>(tab + r * ROW_FLOATS)[sub];
+    }
 }
 
 __global__ void k_fill_index(uint32_t* rows_idx, uint32_t* grad_idx, uint64_t n, uint64_t rows) {
@@ -199,6 +212,7 @@ int main(int argc, char** argv) {
     for (uint64_t n : {1000000ull, 2000000ull}) {
         const int cover = (int)((n + 63) / 64);
         report("read64", n, tm.best_us([&] { hipLaunchKernelGGL(k_rows<false>, dim3(cover), dim3(256), 0, 0, tab, rows, n, sink); }));
+        report("gather", n, tm.best_us([&] { hipLaunchKernelGGL(k_gather, dim3(cover), dim3(256), 0, 0, tab, rows, n, grads); }));
         report("rmw80", n, tm.best_us([&] { hipLaunchKernelGGL(k_rows<true>, dim3(cover), dim3(256), 0, 0, tab, rows, n, sink); }));
         hipLaunchKernelGGL(k_fill_index, dim3(1024), dim3(256), 0, 0, rows_idx, grad_idx, n, rows);
         CK(hipDeviceSynchronize());
