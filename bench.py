@@ -68,7 +68,7 @@ def step_algorithmic_bytes(opt, dim, L, U):
 
 # Launched on the table's side stream, concurrently with kernels of the caller's stream (the
 # other apply kernels; the ranking kernels of the remap): not on the step's critical path.
-SIDE_STREAM_KERNELS = ("k_apply_big", "k_group_count", "k_group_offsets")
+SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_vec", "k_group_count", "k_group_offsets")
 BIG_GROUP = 16  # records from which a sign is applied by k_apply_big (sparse_table.hip)
 
 

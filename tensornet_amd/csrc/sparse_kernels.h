@@ -1421,16 +1421,33 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
     }
 }
 
+// Value of v in lane `src` (the same for the whole wavefront), by register read-out.
+__device__ __forceinline__ float lane_value(float v, int src) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+__device__ __forceinline__ double lane_value(double v, int src) {
+    const long long b = __double_as_longlong(v);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(b & 0xFFFFFFFFll), src);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(b >> 32), src);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
 constexpr int BIG_DIM_MAX = 128;    // largest dim k_apply_big stages in LDS
 constexpr int BIG_GBUF = 2176;      // floats of gradient staging per wavefront at most (dynamic LDS: big_gbuf_floats)
 
-// Staging for up to 64 records of dim D (rows padded by one float), capped at BIG_GBUF.
-inline int big_gbuf_floats(int D) { return 64 * (D + 1) < BIG_GBUF ? 64 * (D + 1) : BIG_GBUF; }
+// Staging for up to BIG_CHUNK records of dim D (rows padded by one float), capped at BIG_GBUF.  The
+// kernel is bound by the wavefronts a CU can hold (chains of dependent loads per sign), so the
+// LDS of a wavefront is kept small enough not to be what limits them.
+constexpr int BIG_CHUNK = 64;
+constexpr int BIG_LOADS = 8;  // gradient loads a lane issues before it waits for the first
+inline int big_gbuf_floats(int D) { return BIG_CHUNK * (D + 1) < BIG_GBUF ? BIG_CHUNK * (D + 1) : BIG_GBUF; }
+// dynamic LDS of k_apply_big: the staging and the row (weights and two state vectors)
+inline size_t big_lds_bytes(int D) { return (size_t)(big_gbuf_floats(D) + 3 * D) * sizeof(float); }
 
 // A sign with many records (it occurs in many slots) would make one lane
 // group chase a long chain of dependent loads.  Here one wavefront owns the
 // sign: the row lives in LDS and the (already ordered) records are taken up
-// to 64 at a time: all lanes resolve and fetch the gradients in parallel,
+// to BIG_CHUNK at a time: the lanes resolve and fetch the gradients in parallel,
 // then the records are applied strictly in order -- for AdaGrad the g2sum
 // chain by one lane, the square roots by one lane per record, the element
 // updates by one lane per element.
@@ -1441,22 +1458,26 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                                                   const uint32_t* __restrict__ grp_off,
                                                   const uint32_t* __restrict__ grp_cnt,
                                                   const Member* __restrict__ list, int gbuf_floats) {
-    __shared__ float rw[BIG_DIM_MAX], ra[BIG_DIM_MAX], rb[BIG_DIM_MAX];
-    extern __shared__ float gbuf[];  // gbuf_floats floats
-    __shared__ const float* gptr[64];
-    __shared__ int gshow[64], gclick[64], gok[64];
-    __shared__ double msq[64];
-    __shared__ float den[64];
+    extern __shared__ float gbuf[];  // gbuf_floats floats of staging, then the row: rw[D], ra[D], rb[D]
+    __shared__ const float* gptr[BIG_CHUNK];
+    __shared__ int gshow[BIG_CHUNK], gok[BIG_CHUNK];
+    __shared__ float den[BIG_CHUNK];
     const int D = s.D;
+    float* rw = gbuf + gbuf_floats;
+    float* ra = rw + D;
+    float* rb = ra + D;
     const int Dp = D + 1;  // padded staging row: lanes walking down a column hit different banks
     const int lane = threadIdx.x;
     // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
     if (status->mismatch | status->abort) return;
     const uint32_t n_big = status->n_big;
-    const int per_chunk = (gbuf_floats / Dp) < 64 ? (gbuf_floats / Dp) : 64;
+    const int per_chunk = (gbuf_floats / Dp) < BIG_CHUNK ? (gbuf_floats / Dp) : BIG_CHUNK;
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
     const bool pow2 = (D & (D - 1)) == 0;
     const double inv_d = 1.0 / (double)D;  // exact when D is a power of two
+    // D divides 64: the lanes tile (records, elements) as lane = record * D + element
+    const bool tiled = D <= 64 && 64 % D == 0;
+    const int li = tiled ? lane % D : 0, lm = tiled ? lane / D : 0, mstep = tiled ? 64 / D : 1;
     for (uint32_t bi = blockIdx.x; bi < n_big; bi += gridDim.x) {
         const uint32_t g = big_list[bi];
         const uint32_t row = grp_row[g];
@@ -1472,7 +1493,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                 rb[i] = sp[D + i];
             }
         }
-        // lane 0 carries the scalars of the row
+        // the scalars of the row, the same in every lane
         float g2sum = 0.f, show = 0.f, click = 0.f;
         int delta_show = 0;
         if (KIND == OPT_ADAGRAD) {
@@ -1486,45 +1507,94 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
         __syncthreads();
         for (uint32_t c0 = 0; c0 < k; c0 += per_chunk) {
             const int cn = (int)((k - c0) < (uint32_t)per_chunk ? (k - c0) : (uint32_t)per_chunk);
+            // lane m resolves record m of the chunk and keeps its counts
+            bool ok = false;
+            int sh = 0, ck = 0;
             if (lane < cn) {
                 const float* gp = nullptr;
-                int sh = 0, ck = 0;
-                const bool ok = src_record(src, list[off + c0 + lane], gp, sh, ck);
+                ok = src_record(src, list[off + c0 + lane], gp, sh, ck);
                 gptr[lane] = gp;
                 gshow[lane] = sh;
-                gclick[lane] = ck;
                 gok[lane] = ok ? 1 : 0;
             }
+            const unsigned long long okmask = __ballot(ok);  // the usable records, known to every lane
             __syncthreads();
-            for (int t = lane; t < cn * D; t += 64) {
-                const int m = t / D, i = t - m * D;
-                gbuf[m * Dp + i] = gok[m] ? gptr[m][i] : 0.f;
+            // gradients into the staging, BIG_LOADS loads of a lane in flight at a time
+            if (tiled) {  // lane = (record within a round, element): no division per element
+                for (int m0 = lm; m0 < cn; m0 += mstep * BIG_LOADS) {
+                    float v[BIG_LOADS];
+#pragma unroll
+                    for (int q = 0; q < BIG_LOADS; q++) {
+                        const int m = m0 + q * mstep;
+                        v[q] = (m < cn && ((okmask >> m) & 1ull)) ? gptr[m][li] : 0.f;
+                    }
+#pragma unroll
+                    for (int q = 0; q < BIG_LOADS; q++) {
+                        const int m = m0 + q * mstep;
+                        if (m < cn) gbuf[m * Dp + li] = v[q];
+                    }
+                }
+            } else {
+                for (int t0 = lane; t0 < cn * D; t0 += 64 * BIG_LOADS) {
+                    float v[BIG_LOADS];
+#pragma unroll
+                    for (int q = 0; q < BIG_LOADS; q++) {
+                        const int t = t0 + q * 64;
+                        v[q] = 0.f;
+                        if (t < cn * D) {
+                            const int m = t / D, i = t - m * D;
+                            if ((okmask >> m) & 1ull) v[q] = gptr[m][i];
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < BIG_LOADS; q++) {
+                        const int t = t0 + q * 64;
+                        if (t < cn * D) {
+                            const int m = t / D;
+                            gbuf[m * Dp + (t - m * D)] = v[q];
+                        }
+                    }
+                }
             }
             __syncthreads();
             if (KIND == OPT_ADAGRAD) {
-                if (lane < cn) {  // add_g2sum / dim of record `lane`: double sum of float products, element order
+                // add_g2sum / dim of record `lane`: double sum of float products in element order
+                double mq = 0.0;
+                if (lane < cn) {
                     const float* gr = gbuf + lane * Dp;
                     double tot = 0.0;
                     for (int i = 0; i < D; i++) tot += (double)(gr[i] * gr[i]);
-                    msq[lane] = pow2 ? tot * inv_d : tot / (double)D;
+                    mq = pow2 ? tot * inv_d : tot / (double)D;
                 }
+                // g2sum after every record (float += double, rounded each time), show and click in
+                // record order: every lane runs the same chain on values read out of the records'
+                // lanes, lane m keeps the g2sum its record meets
+                const float fsh = (float)sh, fck = (float)ck;
+                float myg2 = 0.f;
+                for (int m = 0; m < cn; m++) {
+                    if (!((okmask >> m) & 1ull)) continue;
+                    show += lane_value(fsh, m);
+                    click += lane_value(fck, m);
+                    g2sum = (float)((double)g2sum + lane_value(mq, m));
+                    if (lane == m) myg2 = g2sum;
+                }
+                if (lane < cn) den[lane] = o.eps + sqrtf(myg2);
                 __syncthreads();
-                if (lane == 0) {  // g2sum after every record (float += double, rounded each time)
-                    for (int m = 0; m < cn; m++) {
-                        if (!gok[m]) continue;
-                        show += (float)gshow[m];
-                        click += (float)gclick[m];
-                        g2sum = (float)((double)g2sum + msq[m]);
-                        den[m] = g2sum;
+                // the steps lr * g / den of all records and elements by all lanes (independent divisions),
+                // then per element the subtractions in record order
+                if (tiled) {
+                    for (int m = lm; m < cn; m += mstep) gbuf[m * Dp + li] = o.lr * gbuf[m * Dp + li] / den[m];
+                } else {
+                    for (int t = lane; t < cn * D; t += 64) {
+                        const int m = t / D, i = t - m * D;
+                        gbuf[m * Dp + i] = o.lr * gbuf[m * Dp + i] / den[m];
                     }
                 }
-                __syncthreads();
-                if (lane < cn) den[lane] = o.eps + sqrtf(den[lane]);
                 __syncthreads();
                 for (int i = lane; i < D; i += 64) {
                     float w = rw[i];
                     for (int m = 0; m < cn; m++)
-                        if (gok[m]) w -= o.lr * gbuf[m * Dp + i] / den[m];
+                        if ((okmask >> m) & 1ull) w -= gbuf[m * Dp + i];
                     rw[i] = w;
                 }
             } else {
@@ -1545,12 +1615,9 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                     rb[i] = b;
                 }
             }
-            for (int m = 0; m < cn; m++) {
-                if (gok[m])
-                    any = true;
-                else if (lane == 0)
-                    atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-            }
+            const unsigned long long chunk_mask = cn == 64 ? ~0ull : (1ull << cn) - 1ull;
+            if (okmask) any = true;
+            if (lane == 0 && okmask != chunk_mask) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
             __syncthreads();
         }
         if (any) {

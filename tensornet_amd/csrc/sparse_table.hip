@@ -667,9 +667,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     return TN_OK;
 }
 
-// The three kernels touch disjoint rows.  k_apply_big is latency-bound (few wavefronts, long
-// dependent chains) while the other two saturate the memory system, so it runs beside them on
-// the table's side stream, forked from and joined back into the caller's stream by events.
+// The three kernels touch disjoint rows.  k_apply_single saturates the memory system (it runs
+// at the device's rate for random row updates); k_apply_big and k_apply_vec are bound by
+// dependent chains and instruction issue, so they run one after the other on the table's side
+// stream beside it, forked from and joined back into the caller's stream by events.
 template <int KIND>
 int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
                       const Plan& p, int64_t n_upper, hipStream_t st) {
@@ -681,16 +682,15 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
         TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
         const int gfloats = big_gbuf_floats(s.D);
         TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
-                      gfloats * sizeof(float), t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
+                      big_lds_bytes(s.D), t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
                       p.list, gfloats);
-        TN_HIP(hipEventRecord(t->join_ev, t->side));
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
         TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
                   o, src, ds, p.grp_row, p.list);                                                                 \
-        TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256), st, s, \
-                  o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);                           \
+        TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256),    \
+                  with_big ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap); \
     } while (0)
     switch (lpg) {
         case 1: TN_LAUNCH_VEC(1); break;
@@ -704,7 +704,10 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
                       p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);
     }
 #undef TN_LAUNCH_VEC
-    if (with_big) TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
+    if (with_big) {
+        TN_HIP(hipEventRecord(t->join_ev, t->side));
+        TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
+    }
     return TN_OK;
 }
 
