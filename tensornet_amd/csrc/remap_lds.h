@@ -55,7 +55,8 @@ constexpr int GRP_TABLE = 2048;         // entries of its LDS hash table (> GRP_
 constexpr int GRP_THREADS = 512;        // threads of k_group_count
 constexpr int GRP_RECS = GRP_CAP / GRP_THREADS;  // records per thread of a second-level bucket's workgroup
 static_assert(GRP_CAP % GRP_THREADS == 0 && GRP_CAP % 256 == 0 && GRP_CAP < GRP_TABLE, "a bucket fits its table and the registers of one workgroup");
-constexpr int EMIT_RECS = GRP_CAP / 256;  // records per thread of k_group_emit (256 threads)
+constexpr int EMIT_THREADS = 512;
+constexpr int EMIT_RECS = GRP_CAP / EMIT_THREADS;  // records per thread of k_group_emit
 constexpr int GRP_ITEMS = (GRP_TABLE + 1 + GRP_THREADS - 1) / GRP_THREADS;
 constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
 
@@ -634,25 +635,41 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
 // ids and member places counted up from 0 (place == id), groups with several
 // get ids counted down from ids_cap - 1 and slices carved from the top of the
 // member array, in bucket order.
-__global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+//
+// A bucket's groups and members occupy contiguous ranges of those arrays, but its records
+// arrive in hash order: written record by record, every store is a transaction of its own
+// (several million per call, which is what the kernel's time was).  So the bucket's part of
+// the arrays is first put together in LDS and then copied out in order; only where_u, indexed
+// by the distinct index of the record, stays a scattered store.
+__global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
+                                                    const uint4* __restrict__ bcounts,
                                                     const uint8_t* __restrict__ flag8,
                                                     const uint32_t* __restrict__ wordpre, uint32_t ids_cap,
                                                     uint32_t big_k, uint64_t* __restrict__ grp_sign,
                                                     uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
                                                     uint2* __restrict__ where_u) {
+    // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
+    // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
+    __shared__ Member s_list[GRP_CAP];
+    __shared__ unsigned long long s_sign[GRP_CAP];
+    __shared__ uint32_t s_off[GRP_CAP], s_cnt[GRP_CAP];
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+        if (n == 0) continue;
         const size_t first = (size_t)c * GRP_CAP;
         const uint4 bb = bbase[c];
+        const uint4 bc = bcounts[c];
+        const uint32_t n1 = bc.x, nm = bc.y, nr = bc.z;  // groups of one record, of several, records of the latter
+        const uint32_t top = ids_cap - 1 - bb.z;         // member place of local member 0 of the several-record groups
         GroupRec rs[EMIT_RECS];
         uint2 as[EMIT_RECS];
         uint32_t us[EMIT_RECS];
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
-            const uint32_t i = j * 256 + threadIdx.x;
+            const uint32_t i = j * EMIT_THREADS + threadIdx.x;
             if (i < n) {
                 rs[j] = recs[first + i];
                 as[j] = aux[first + i];
@@ -660,37 +677,56 @@ __global__ __launch_bounds__(256) void k_group_emit(uint32_t nb2, const uint32_t
         }
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++)
-            if (j * 256 + threadIdx.x < n) us[j] = rank_of(flag8, wordpre, rs[j].gi);
+            if (j * EMIT_THREADS + threadIdx.x < n) us[j] = rank_of(flag8, wordpre, rs[j].gi);
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
-            if (j * 256 + threadIdx.x >= n) continue;
+            if (j * EMIT_THREADS + threadIdx.x >= n) continue;
             const GroupRec r = rs[j];
             const uint2 a = as[j];
             const uint32_t k = a.x >> 24, idx = a.x & 0xFFFu, bigidx = (a.x >> 12) & 0xFFFu;
             const uint32_t place = (a.y >> 16) & 0xFFu, sl = a.y >> 24;
-            uint32_t g, off;
-            if (k == 1) {
-                g = bb.x + idx;
-                off = g;
-            } else {
-                g = ids_cap - 1 - (bb.y + idx);
-                off = ids_cap - (bb.z + (a.y & 0xFFFFu) + k);
-            }
-            const uint32_t at = off + place;
             Member m;
             m.u = us[j];
             m.slot = sl;
             m.show = (int32_t)r.cnt;  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             m.click = 0;
-            list[at] = m;
-            where_u[m.u] = make_uint2(at, g);
-            if (place == 0) {
-                grp_sign[g] = r.sign;
-                grp_off[g] = off;
-                grp_cnt[g] = k;
-                if (is_big(k, big_k)) big_list[bb.w + bigidx] = g;
+            if (k == 1) {
+                const uint32_t g = bb.x + idx;
+                s_list[idx] = m;
+                s_sign[idx] = r.sign;
+                s_off[idx] = g;
+                s_cnt[idx] = 1;
+                where_u[m.u] = make_uint2(g, g);
+            } else {
+                const uint32_t g = ids_cap - 1 - (bb.y + idx);
+                const uint32_t before = a.y & 0xFFFFu;        // records of the bucket's earlier groups of this kind
+                const uint32_t t = before + k - 1 - place;    // local member: the group's last record first
+                s_list[n1 + t] = m;
+                where_u[m.u] = make_uint2(top - t, g);
+                if (place == 0) {
+                    s_sign[n1 + idx] = r.sign;
+                    s_off[n1 + idx] = top - (before + k - 1);
+                    s_cnt[n1 + idx] = k;
+                    if (is_big(k, big_k)) big_list[bb.w + bigidx] = g;
+                }
             }
         }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < n1; i += EMIT_THREADS) {
+            const uint32_t g = bb.x + i;
+            list[g] = s_list[i];
+            grp_sign[g] = s_sign[i];
+            grp_off[g] = s_off[i];
+            grp_cnt[g] = s_cnt[i];
+        }
+        for (uint32_t i = threadIdx.x; i < nr; i += EMIT_THREADS) list[top - i] = s_list[n1 + i];
+        for (uint32_t i = threadIdx.x; i < nm; i += EMIT_THREADS) {
+            const uint32_t g = ids_cap - 1 - (bb.y + i);
+            grp_sign[g] = s_sign[n1 + i];
+            grp_off[g] = s_off[n1 + i];
+            grp_cnt[g] = s_cnt[n1 + i];
+        }
+        __syncthreads();
     }
 }
 

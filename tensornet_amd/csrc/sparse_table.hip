@@ -652,7 +652,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
-        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(256), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.flag8, w.wordpre, L,
+        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.bcounts, w.flag8, w.wordpre, L,
                   big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u);
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
