@@ -491,11 +491,12 @@ def test_bound_ops_over_several_steps_without_waiting(tn, oracle):
     pair.assert_rows_match(base)
 
 
+@pytest.mark.parametrize("D", [8, 12, 64, 128])
 @pytest.mark.parametrize("opt,hyper", [("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP)])
-def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper):
+def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper, D):
     """SparseTable::Push applies records in array order however often a sign repeats:
-    a few records, a few hundred (one wavefront per sign) and more than fit in LDS."""
-    D = 8
+    a few records, a few hundred (one wavefront per sign) and more than fit in LDS; dims that
+    divide the wavefront, one that does not, and one whose rows fill the staging 16 at a time."""
     rng = np.random.default_rng(13)
     pair = Pair(tn, oracle, opt, D, hyper)
     base = pair.populate(synth.splitmix64(np.arange(1, 41, dtype=np.uint64)))
