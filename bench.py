@@ -33,24 +33,23 @@ def log(msg):
 # Counters cannot be read from inside this script; the figures are refreshed together with that summary.
 MEASURED_TRAFFIC = {
     "k_show_decay": 85652100000,
-    "k_gather_vars": 506100000,
-    "k_group_emit": 455100000,
-    "k_reduce_pooled": 393600000,
-    "k_combine_fwd": 356200000,
+    "k_gather_vars": 506000000,
+    "k_reduce_pooled": 393500000,
+    "k_combine_fwd": 356300000,
     "k_apply_single": 341500000,
-    "k_reduce_long": 236500000,
-    "k_lds_scatter": 205100000,
-    "k_lds_dedup": 203500000,
-    "k_lds_mapped": 139000000,
+    "k_reduce_long": 236700000,
+    "k_lds_scatter": 203800000,
+    "k_lds_dedup": 203400000,
+    "k_group_emit": 186500000,
+    "k_verify_values": 124600000,
     "k_lookup_keys": 123300000,
-    "k_apply_vec": 118400000,
-    "k_verify_values": 114600000,
+    "k_apply_vec": 118500000,
     "k_lds_hist": 101300000,
-    "k_apply_big": 88900000,
+    "k_apply_big": 89000000,
+    "k_lds_mapped": 87400000,
     "k_group_count": 49300000,
-    "k_count_click": 42400000,
     "k_lds_flags": 20700000,
-    "k_lds_assign": 20500000,
+    "k_lds_assign": 1200000,
 }
 
 
