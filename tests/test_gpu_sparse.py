@@ -640,3 +640,64 @@ def test_two_pushes_on_one_pull_count_their_own_clicks(tn, oracle):
         labels = [rng.integers(0, 3, len(v)).astype(np.int64) for v in values]
         pair.push_op(values, grads, labels)
         pair.assert_rows_match(all_signs(values))
+
+
+def test_two_tables_driven_from_two_host_threads(tn, oracle):
+    """Different tables may be hit concurrently (TF runs ComputeAsync from inter-op threads,
+    core/kernels/sparse_table_ops.cc:203-236): two host threads, each with its own stream and
+    table, run pull + push steps at the same time; afterwards the oracle replays both
+    sequences and must see the same mapped ids, pulled rows and final tables."""
+    import threading
+
+    specs = [("AdaGrad", 8, ADAGRAD_HP, 21), ("Adam", 16, ADAM_HP, 22)]
+    vocab, steps = 30000, 4
+    pool = synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)).view(np.int64)
+    pairs, plans = [], []
+    for opt, D, hp, seed in specs:
+        pair = Pair(tn, oracle, opt, D, hp, reserve=300000, zero_init=True)
+        pair.populate(pool[:20000].view(np.uint64))
+        rng = np.random.default_rng(seed)
+        batches = []
+        for _ in range(steps):
+            values = [pool[rng.integers(0, vocab, int(rng.integers(2000, 4000)))] for _ in range(16)]  # LDS path
+            labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+            batches.append((values, labels, int(rng.integers(1 << 30))))
+        pairs.append(pair)
+        plans.append(batches)
+    results = [[] for _ in pairs]
+    errors = []
+
+    def drive(k):
+        try:
+            pair = pairs[k]
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for values, labels, gseed in plans[k]:
+                    gvars = [torch.full((len(v) + 1, pair.wf), -7.0, device="cuda") for v in values]
+                    mapped = tn.ops.sparse_table_pull(gvars, [dev(v) for v in values], pair.h)
+                    counts = tn.ops.sparse_table_last_unique_counts(pair.h, len(values))
+                    grads = synth.make_grads(np.array(counts), pair.wf, 0.01, seed=gseed)
+                    tn.ops.sparse_table_push([dev(v) for v in values], [dev(g) for g in grads],
+                                             [dev(l) for l in labels], pair.h)
+                    tn.ops.sparse_table_sync(pair.h)
+                    results[k].append(([m.cpu().numpy() for m in mapped], [v.cpu().numpy() for v in gvars], counts,
+                                       grads))
+        except Exception as e:  # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=drive, args=(k,)) for k in range(len(pairs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for k, pair in enumerate(pairs):
+        for (values, labels, _), (gm, gv, counts, grads) in zip(plans[k], results[k]):
+            cvars = [np.full((len(v) + 1, pair.wf), -7.0, np.float32) for v in values]
+            rc, cm, ccounts = pair.o.pull_op(values, cvars)
+            assert rc == 0 and ccounts.tolist() == counts
+            for s in range(len(values)):
+                assert (gm[s] == cm[s]).all()
+                assert (gv[s].view(np.int32) == cvars[s].view(np.int32)).all()
+            rc, _ = pair.o.push_op(values, grads, labels)
+            assert rc == 0
+        assert pair.assert_rows_match(all_signs([v for b in plans[k] for v in b[0]])) > 0.99
