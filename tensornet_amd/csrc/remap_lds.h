@@ -170,8 +170,8 @@ __global__ __launch_bounds__(1024) void k_lds_offsets(const uint32_t* __restrict
 
 __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     uint32_t* bcursor, uint64_t* __restrict__ pkey,
-                                                     uint32_t* __restrict__ pgi, uint32_t span_cap) {
+                                                     uint32_t* bcursor, ulonglong2* __restrict__ prec,
+                                                     uint32_t span_cap) {
     extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]: first the tile's count per bucket, then its write cursor
     uint32_t* lb = smem;
     uint32_t* hist = smem + N + 1;
@@ -207,8 +207,7 @@ __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict_
             const uint32_t local = bucket_of(d, sign) - b0;
             if (local < span) {
                 const uint32_t at = atomicAdd(&hist[local], 1u);
-                pkey[at] = sign;
-                pgi[at] = gi;
+                prec[at] = make_ulonglong2(sign, gi);  // one 16-byte store per lookup: these stores are what the pass costs
             }
         });
         __syncthreads();
@@ -223,7 +222,7 @@ __device__ __forceinline__ uint32_t lds_slot(uint64_t sign) { return (uint32_t)(
 // second-level bucket (recs[c * GRP_CAP ...], cursor2[c] = records handed in).
 template <bool EMIT>
 __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
-                                                   const uint64_t* __restrict__ pkey, const uint32_t* __restrict__ pgi,
+                                                   const ulonglong2* __restrict__ prec,
                                                    uint32_t* __restrict__ first_of, uint32_t* __restrict__ cnt_at,
                                                    DevStatus* status, uint32_t nb2, uint32_t* cursor2,
                                                    GroupRec* __restrict__ recs) {
@@ -255,8 +254,9 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
 #pragma unroll
             for (int j = 0; j < DEDUP_ITEMS; j++) {
                 const uint32_t i = base + j * DEDUP_THREADS + threadIdx.x;
-                sg[j] = (i < hi) ? pkey[i] : 0;
-                gp[j] = (i < hi) ? pgi[i] : 0xFFFFFFFFu;  // no position: nothing to do
+                const ulonglong2 r = (i < hi) ? prec[i] : make_ulonglong2(0, 0xFFFFFFFFull);  // no position: nothing to do
+                sg[j] = r.x;
+                gp[j] = (uint32_t)r.y;
             }
         };
         uint32_t c_min = 0xFFFFFFFFu;

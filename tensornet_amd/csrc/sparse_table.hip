@@ -368,8 +368,7 @@ struct Scratch {
     uint32_t* bcount;
     uint32_t* bstart;
     uint32_t* bcursor;
-    uint64_t* pkey;
-    uint32_t* pgi;
+    ulonglong2* prec;    // lookups by bucket: {sign, position}
     uint32_t* first_of;
     uint32_t* cnt_at;
     uint32_t* wordpre;  // first occurrences before every 64-lookup word
@@ -439,8 +438,7 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.bbase = c.take<uint4>(w.nb2);
         w.bstart = c.take<uint32_t>(dt_entries + 1);
         w.bcursor = c.take<uint32_t>(dt_entries + 1);
-        w.pkey = c.take<uint64_t>(L);
-        w.pgi = c.take<uint32_t>(L);
+        w.prec = c.take<ulonglong2>(L);
         w.first_of = c.take<uint32_t>(L);
         w.cnt_at = c.take<uint32_t>(L);
         w.wordpre = c.take<uint32_t>(L / 64 + 2);
@@ -606,14 +604,14 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy,
                       w.first_of, ds, w.span_cap);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
-        TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.pkey,
-                      w.pgi, w.span_cap);
+        TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.prec,
+                      w.span_cap);
         if (lds_groups)
             TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
-                      w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
+                      w.nbuckets, w.prec, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         else
             TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
-                      w.nbuckets, w.pkey, w.pgi, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
+                      w.nbuckets, w.prec, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         if (lds_groups) {
             // The grouping of the distinct records only needs what the dedup handed over: it runs on
             // the side stream beside the ranking of the first occurrences (LDS / latency bound
