@@ -67,22 +67,39 @@ __device__ __forceinline__ void adagrad_elem(float g, float& w, float& d2, float
     w -= a.lr * m / (sqrtf(g2) / sqrtf(d2) + a.eps);
 }
 
+// 16-byte accesses marked non-temporal: streamed data, read once and written once per step.
+typedef float native_float4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 stream_load(const float4* p) {
+    const native_float4 v = __builtin_nontemporal_load(reinterpret_cast<const native_float4*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stream_store(float4* p, float4 v) {
+    native_float4 n;
+    n.x = v.x;
+    n.y = v.y;
+    n.z = v.z;
+    n.w = v.w;
+    __builtin_nontemporal_store(n, reinterpret_cast<native_float4*>(p));
+}
+
 // n4 float4 groups starting at the (16-byte aligned) pointers.
 __global__ __launch_bounds__(256) void k_dense_adam_v4(const float4* __restrict__ g, float4* __restrict__ w,
                                                        float4* __restrict__ m, float4* __restrict__ v,
                                                        float4* __restrict__ out, int64_t n4, AdamArgs a) {
+    // every element is read once and written once per step: the accesses are marked non-temporal
+    // so that the stream does not displace the caches' contents
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-        float4 gg = g[i];
-        float4 ww = w[i], mm = m[i], vv = v[i];
+        float4 gg = stream_load(&g[i]);
+        float4 ww = stream_load(&w[i]), mm = stream_load(&m[i]), vv = stream_load(&v[i]);
         adam_elem(gg.x, ww.x, mm.x, vv.x, a);
         adam_elem(gg.y, ww.y, mm.y, vv.y, a);
         adam_elem(gg.z, ww.z, mm.z, vv.z, a);
         adam_elem(gg.w, ww.w, mm.w, vv.w, a);
-        w[i] = ww;
-        m[i] = mm;
-        v[i] = vv;
-        if (out) out[i] = ww;
+        stream_store(&w[i], ww);
+        stream_store(&m[i], mm);
+        stream_store(&v[i], vv);
+        if (out) stream_store(&out[i], ww);
     }
 }
 
