@@ -67,21 +67,6 @@ __device__ __forceinline__ void adagrad_elem(float g, float& w, float& d2, float
     w -= a.lr * m / (sqrtf(g2) / sqrtf(d2) + a.eps);
 }
 
-// 16-byte accesses marked non-temporal: streamed data, read once and written once per step.
-typedef float native_float4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ float4 stream_load(const float4* p) {
-    const native_float4 v = __builtin_nontemporal_load(reinterpret_cast<const native_float4*>(p));
-    return make_float4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ void stream_store(float4* p, float4 v) {
-    native_float4 n;
-    n.x = v.x;
-    n.y = v.y;
-    n.z = v.z;
-    n.w = v.w;
-    __builtin_nontemporal_store(n, reinterpret_cast<native_float4*>(p));
-}
-
 // n4 float4 groups starting at the (16-byte aligned) pointers.
 __global__ __launch_bounds__(256) void k_dense_adam_v4(const float4* __restrict__ g, float4* __restrict__ w,
                                                        float4* __restrict__ m, float4* __restrict__ v,

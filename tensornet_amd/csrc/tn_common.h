@@ -111,6 +111,22 @@ __device__ __forceinline__ uint32_t ld_relaxed(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// 16-byte accesses marked non-temporal, for data that is read once or written once per call and
+// should not displace what the caches hold.
+typedef float native_float4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 stream_load(const float4* p) {
+    const native_float4 v = __builtin_nontemporal_load(reinterpret_cast<const native_float4*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stream_store(float4* p, float4 v) {
+    native_float4 n;
+    n.x = v.x;
+    n.y = v.y;
+    n.z = v.z;
+    n.w = v.w;
+    __builtin_nontemporal_store(n, reinterpret_cast<native_float4*>(p));
+}
+
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // grow-only device buffer
