@@ -769,13 +769,16 @@ __global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict
 
 // Push: are the signs of this call the ones the plan was built from?  With CLICKS the same
 // pass adds the non-zero labels to the click sums of the plan's member lists, which start
-// at zero (sparse_table_ops.cc:283-296; on a mismatch the plan is discarded anyway).
+// at zero (sparse_table_ops.cc:283-296; on a mismatch the plan is discarded anyway).  A
+// mismatch is also written to host_mismatch (pinned host memory, cleared by the host before the
+// launch), which the host reads once the kernel is done.
 template <bool CLICKS>
 __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                        const uint64_t* __restrict__ vals_copy, DevStatus* status,
                                                        const uint32_t* __restrict__ u_of_gi,
-                                                       const uint2* __restrict__ where_u, Member* list) {
+                                                       const uint2* __restrict__ where_u, Member* list,
+                                                       uint32_t* host_mismatch) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
     const uint32_t stride = gridDim.x * blockDim.x;
@@ -789,7 +792,10 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
             if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
         }
     }
-    if (bad) atomicOr(&status->mismatch, 1u);
+    if (bad) {
+        atomicOr(&status->mismatch, 1u);
+        *host_mismatch = 1u;
+    }
 }
 
 // Push: batch_show = occurrences, batch_click = sum of labels per distinct sign

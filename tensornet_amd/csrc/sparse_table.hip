@@ -1335,18 +1335,19 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // after the pull, a further push on the same plan clears them first.
         const bool clicks = t->plan_has_show && with_click;
         const int vblocks = launch_grid(L, 256, GRID_CAP * 2);
+        // the outcome comes back through pinned host memory, written by the verify kernel itself
+        t->hpush->st.mismatch = 0;
+        uint32_t* host_mismatch = &t->hpush->st.mismatch;
         if (clicks) {
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
             TN_LAUNCH((k_verify_values<true>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.vals_copy,
-                      ds, p.u_of_gi, p.where_u, p.list);
+                      ds, p.u_of_gi, p.where_u, p.list, host_mismatch);
         } else {
             TN_LAUNCH((k_verify_values<false>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L,
-                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list);
+                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch);
         }
-        TN_LAUNCH(k_publish, dim3(1), dim3(64), st, ds, p.ubase, 0u, reinterpret_cast<uint32_t*>(t->hpush),
-                  (unsigned long long*)nullptr);
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // Counts and apply kernels are queued before the host knows the outcome: the counts only
         // touch the plan's member lists, which a mismatch discards anyway, and the apply kernels
