@@ -8,6 +8,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <unistd.h>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -120,7 +121,10 @@ static void gpu_checks() {
     // SparseTable::ShowDecay / Save / Load: a second table of the same name reads the files back
     EXPECT(t->ShowDecay(1) == TN_OK);
     const char* tmp = std::getenv("TMPDIR");
-    const std::string ckpt = std::string(tmp ? tmp : "/tmp") + "/tn_host_mirror_ckpt";
+    std::string pattern = std::string(tmp ? tmp : "/tmp") + "/tn_host_mirror_XXXXXX";  // a fresh directory per run
+    const char* made = mkdtemp(&pattern[0]);
+    EXPECT(made != nullptr);
+    const std::string ckpt = made ? made : pattern;
     EXPECT(t->Save(ckpt, "txt") == TN_OK);
     SparseTable* t2 = CreateSparseTable(opt, "gpu", D, 1, 0, "");
     EXPECT(t2 && t2 != t && t2->Load(ckpt, "txt") == TN_OK);
