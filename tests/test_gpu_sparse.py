@@ -701,3 +701,44 @@ def test_two_tables_driven_from_two_host_threads(tn, oracle):
             rc, _ = pair.o.push_op(values, grads, labels)
             assert rc == 0
         assert pair.assert_rows_match(all_signs([v for b in plans[k] for v in b[0]])) > 0.99
+
+
+def _mix64(x):
+    m = (1 << 64) - 1
+    x ^= x >> 33
+    x = (x * 0xff51afd7ed558ccd) & m
+    x ^= x >> 33
+    x = (x * 0xc4ceb9fe1a85ec53) & m
+    x ^= x >> 33
+    return x
+
+
+def test_probe_chains_wrap_around_the_end_of_the_table(tn, oracle):
+    """Collisions: signs whose home slots all lie in the last group of 8 slots of the table, three
+    times as many as the group holds, so that their probe sequences run over the end of the
+    table into its first groups; pulled, pushed, pulled again and found again by a push of
+    another batch (probe without insert)."""
+    D = 8
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=100, zero_init=True)
+    pair.populate(synth.splitmix64(np.arange(1, 4, dtype=np.uint64)))  # allocates the table
+    cap = tn.core.sparse_table_capacity(pair.h)
+    assert cap % 8 == 0 and cap < 400
+    rng = np.random.default_rng(3)
+    crowd = []
+    while len(crowd) < 24:
+        s = int(rng.integers(1, 1 << 62))
+        if (_mix64(s) * cap) >> 64 >= cap - 8:
+            crowd.append(s)
+    signs = np.array(crowd, dtype=np.int64)
+    values = [signs[:16], signs[8:]]  # overlapping slots: 8 of the signs get two records
+    counts = check_pull(pair, values)
+    assert tn.core.sparse_table_capacity(pair.h) == cap  # no growth: the chains are what is tested
+    grads = synth.make_grads(counts, D, 0.01, seed=5)
+    pair.push_op(values, grads, [np.ones(len(v), np.int64) for v in values])
+    assert pair.assert_rows_match(all_signs(values)) > 0.99
+    check_pull(pair, values)
+    other = [signs[::-1].copy()]  # another batch than the last pull's: its plan is built by the push
+    counts = pair.o.pull_op(other, [np.zeros((len(signs) + 1, pair.wf), np.float32)])[2]
+    grads = synth.make_grads(counts, D, 0.01, seed=6)
+    pair.push_op(other, grads, [np.zeros(len(signs), np.int64)])
+    assert pair.assert_rows_match(all_signs(values)) > 0.99
