@@ -67,7 +67,7 @@ def step_algorithmic_bytes(opt, dim, L, U):
 
 # Launched on the table's side stream, concurrently with kernels of the caller's stream (the
 # other apply kernels; the ranking kernels of the remap): not on the step's critical path.
-SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_vec", "k_group_count", "k_group_offsets")
+SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_vec", "k_group_count", "k_group_offsets", "k_probe_recs")
 BIG_GROUP = 16  # records from which a sign is applied by k_apply_big (sparse_table.hip)
 
 
@@ -92,13 +92,15 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
         "k_lds_assign": 4 * U,
         "k_lds_mapped": 12 * L,                # first position in, mapped id out
         "k_group_count": 24 * U,               # distinct records in, per-record placement out
-        "k_group_emit": 48 * U + 16 * G,       # records + placement in; member lists, per-record index, groups out
+        "k_group_emit": 52 * U + 20 * G,       # records, placement and rows in; member lists, per-record index and
+                                               # row, groups out
         # global-table fallback
         "k_remap_insert": 8 * L, "k_assign_rank": 8 * U, "k_write_mapped": 8 * L, "k_count_show": 8 * L,
         "k_mask_insert": 16 * U, "k_mask_compact": 16 * G, "k_mask_fill": 32 * U,
         "k_group_insert": 16 * U,
         # table
         "k_probe": 8 * G + 4 * G,              # one stored-key compare per distinct sign, row number out
+        "k_probe_recs": 8 * U + 8 * U + 4 * U, # the record's sign in, one stored-key compare, row number out
         "k_gather_vars": U * (2 * row + 4),    # row read + variable row write
         # push
         "k_verify_values": 24 * L,             # the op's signs against the pull's copy, labels

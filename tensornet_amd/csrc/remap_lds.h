@@ -631,6 +631,34 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
     }
 }
 
+// The table row of every distinct record, found or, for an absent sign, inserted and filled
+// (SparseKernelBlock::GetWeight, optimizer_kernel.h:299-308): rrow[record] = row, NO_ROW if the
+// table is full.  It needs nothing but the records the dedup handed over, so it runs on a
+// stream of its own beside the grouping and the ranking (random reads of the table against LDS
+// and streaming work).  A sign present in several slots is probed once per slot; whichever
+// thread claims a free slot first owns the insertion, the others find the key there.
+__global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+                                                    const GroupRec* __restrict__ recs, uint32_t* __restrict__ rrow,
+                                                    Store s, OptDev o, uint64_t seed, DevStatus* status) {
+    // whole wavefronts take part in every round (wave_alloc votes)
+    for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
+        const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+        const size_t first = (size_t)c * GRP_CAP;
+        for (uint32_t i0 = 0; i0 < n; i0 += 256) {
+            const uint32_t i = i0 + threadIdx.x;
+            bool is_new = false;
+            if (i < n) {
+                const uint64_t sign = recs[first + i].sign;
+                const uint32_t row = probe_slot<true>(s, sign, is_new);
+                rrow[first + i] = row;
+                if (row == NO_ROW) atomicOr(&status->err, DEV_ERR_TABLE_FULL);
+                if (is_new) init_row(s, o, seed, sign, row);  // the thread that claimed the row fills it
+            }
+            wave_alloc(is_new, &status->n_new);
+        }
+    }
+}
+
 // Numbers the groups and writes the member lists: groups with one record get
 // ids and member places counted up from 0 (place == id), groups with several
 // get ids counted down from ids_cap - 1 and slices carved from the top of the
@@ -640,7 +668,8 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
 // arrive in hash order: written record by record, every store is a transaction of its own
 // (several million per call, which is what the kernel's time was).  So the bucket's part of
 // the arrays is first put together in LDS and then copied out in order; only where_u, indexed
-// by the distinct index of the record, stays a scattered store.
+// by the distinct index of the record, stays a scattered store.  where_u[u] = {place in the member
+// list, table row of the record's sign (rrow, from k_probe_recs)}; the groups get the rows too.
 __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
@@ -650,12 +679,15 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
                                                     uint32_t big_k, uint64_t* __restrict__ grp_sign,
                                                     uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
-                                                    uint2* __restrict__ where_u) {
+                                                    uint2* __restrict__ where_u,
+                                                    const uint32_t* __restrict__ rrow,
+                                                    uint32_t* __restrict__ grp_row) {
     // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
     // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
     __shared__ Member s_list[GRP_CAP];
     __shared__ unsigned long long s_sign[GRP_CAP];
-    __shared__ uint32_t s_off[GRP_CAP], s_cnt[GRP_CAP];
+    __shared__ uint32_t s_off[GRP_CAP], s_row[GRP_CAP];
+    __shared__ uint16_t s_cnt[GRP_CAP];  // at most GRP_SLOTS records per group
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         if (n == 0) continue;
@@ -666,13 +698,14 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
         const uint32_t top = ids_cap - 1 - bb.z;         // member place of local member 0 of the several-record groups
         GroupRec rs[EMIT_RECS];
         uint2 as[EMIT_RECS];
-        uint32_t us[EMIT_RECS];
+        uint32_t us[EMIT_RECS], rows[EMIT_RECS];
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
             const uint32_t i = j * EMIT_THREADS + threadIdx.x;
             if (i < n) {
                 rs[j] = recs[first + i];
                 as[j] = aux[first + i];
+                rows[j] = rrow[first + i];
             }
         }
 #pragma unroll
@@ -696,17 +729,19 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
                 s_sign[idx] = r.sign;
                 s_off[idx] = g;
                 s_cnt[idx] = 1;
-                where_u[m.u] = make_uint2(g, g);
+                s_row[idx] = rows[j];
+                where_u[m.u] = make_uint2(g, rows[j]);
             } else {
                 const uint32_t g = ids_cap - 1 - (bb.y + idx);
                 const uint32_t before = a.y & 0xFFFFu;        // records of the bucket's earlier groups of this kind
                 const uint32_t t = before + k - 1 - place;    // local member: the group's last record first
                 s_list[n1 + t] = m;
-                where_u[m.u] = make_uint2(top - t, g);
+                where_u[m.u] = make_uint2(top - t, rows[j]);
                 if (place == 0) {
+                    s_row[n1 + idx] = rows[j];  // every record of the sign was given the same row
                     s_sign[n1 + idx] = r.sign;
                     s_off[n1 + idx] = top - (before + k - 1);
-                    s_cnt[n1 + idx] = k;
+                    s_cnt[n1 + idx] = (uint16_t)k;
                     if (is_big(k, big_k)) big_list[bb.w + bigidx] = g;
                 }
             }
@@ -718,6 +753,7 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
             grp_sign[g] = s_sign[i];
             grp_off[g] = s_off[i];
             grp_cnt[g] = s_cnt[i];
+            grp_row[g] = s_row[i];
         }
         for (uint32_t i = threadIdx.x; i < nr; i += EMIT_THREADS) list[top - i] = s_list[n1 + i];
         for (uint32_t i = threadIdx.x; i < nm; i += EMIT_THREADS) {
@@ -725,6 +761,7 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
             grp_sign[g] = s_sign[n1 + i];
             grp_off[g] = s_off[n1 + i];
             grp_cnt[g] = s_cnt[n1 + i];
+            grp_row[g] = s_row[n1 + i];
         }
         __syncthreads();
     }

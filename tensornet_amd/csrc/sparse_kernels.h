@@ -1153,6 +1153,7 @@ __global__ __launch_bounds__(256) void k_mask_fill(const DevStatus* status, cons
 
 // vars[slot][rank, :] = table row of the sign, for every distinct sign u of
 // every slot (PopulatePulledVariable_, sparse_table_ops.cc:244-265).
+// grp_row == nullptr: where_u[u].y is the row itself instead of the group that has it.
 template <int VEC>
 __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status, const uint32_t* __restrict__ grp_row,
                                                      const uint2* __restrict__ where_u,
@@ -1166,7 +1167,7 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
         const int64_t u = t / chunks;
         const int c = (int)(t - u * chunks);
-        const uint32_t row = grp_row[where_u[u].y];
+        const uint32_t row = grp_row ? grp_row[where_u[u].y] : where_u[u].y;
         const int sl = find_slot(ub, N, (uint32_t)u);  // the slot whose window of distinct indices holds u
         const int64_t r = (int64_t)u - (int64_t)ub[sl];
         const SlotDesc& d = descs[sl];

@@ -19,6 +19,7 @@ namespace {
 constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:266
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
+constexpr int PROBE_RECS_GRID = 1024;                // workgroups of k_probe_recs (measured: 512-1024 are best)
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
 constexpr size_t LDS_MIN_LOOKUPS = 32768;  // smaller batches are launch-bound: the shorter global-table path wins
 
@@ -59,7 +60,8 @@ struct SparseTable {
     DevBuf comb_buf;                // slot descriptors of a combine op
     DevBuf pooled_ws;               // scratch of a push of pooled gradients (sort buffers, reduced rows)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
-    hipEvent_t fork_ev = nullptr, join_ev = nullptr;
+    hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
+    hipEvent_t fork_ev = nullptr, join_ev = nullptr, join2_ev = nullptr;
     bool plan_clicks_dirty = false;  // a push has added clicks to the member lists of the current plan
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
@@ -183,7 +185,9 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipEventCreateWithFlags(&t->verify_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->fork_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->join_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->join2_ev, hipEventDisableTiming));
     TN_HIP(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));  // default priority
+    TN_HIP(hipStreamCreateWithFlags(&t->side2, hipStreamNonBlocking));
     return TN_OK;
 }
 
@@ -377,6 +381,7 @@ struct Scratch {
     uint32_t* cursor2;
     GroupRec* recs;
     uint2* aux;
+    uint32_t* rrow;      // per distinct record: table row of its sign
     uint4* bcounts;
     uint4* bbase;
     void* gt;  // GroupEntry[] or MaskEntry[]
@@ -434,6 +439,7 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.cursor2 = w.bcount + dt_entries + 1;
         w.recs = c.take<GroupRec>((size_t)w.nb2 * GRP_CAP);
         w.aux = c.take<uint2>((size_t)w.nb2 * GRP_CAP);
+        w.rrow = c.take<uint32_t>((size_t)w.nb2 * GRP_CAP);
         w.bcounts = c.take<uint4>(w.nb2);
         w.bbase = c.take<uint4>(w.nb2);
         w.bstart = c.take<uint32_t>(dt_entries + 1);
@@ -623,6 +629,12 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
                       big_threshold(s), w.aux, w.bcounts);
             TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
             TN_HIP(hipEventRecord(t->join_ev, t->side));
+            // ... and so do the rows of the records' signs, on a stream of their own
+            TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
+            // few workgroups: enough probes in flight for the memory system, most of every CU left to the grouping
+            TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), t->side2, w.nb2, w.cursor2, w.recs, w.rrow, s,
+                      make_optdev(t), t->seed, ds);
+            TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
@@ -650,8 +662,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
+        TN_HIP(hipStreamWaitEvent(st, t->join2_ev, 0));
         TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.bcounts, w.flag8, w.wordpre, L,
-                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u);
+                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row);
+        return TN_OK;  // the rows were found beside the grouping
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
     else
@@ -1174,12 +1188,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         const Store& s = t->store;
         DevStatus* ds = t->dplan;
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st));
+        // the grouping through LDS leaves the row of every distinct record in where_u itself
+        const uint32_t* rows_of_groups = (use_lds && N <= GRP_SLOTS) ? nullptr : p.grp_row;
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
-                      ds, p.grp_row, p.where_u, p.ubase, N, p.descs);
+                      ds, rows_of_groups, p.where_u, p.ubase, N, p.descs);
         else
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
-                      p.grp_row, p.where_u, p.ubase, N, p.descs);
+                      rows_of_groups, p.where_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
         TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
                   reinterpret_cast<uint32_t*>(t->hpull), s.count);
