@@ -63,6 +63,11 @@ struct SparseTable {
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     hipEvent_t fork_ev = nullptr, join_ev = nullptr, join2_ev = nullptr;
     bool plan_clicks_dirty = false;  // a push has added clicks to the member lists of the current plan
+    // Distinct records per lookup seen by the recent pulls (1 = every lookup distinct, the safe start):
+    // sizes the number of second-level buckets, whose room is fixed.  A batch with more distinct
+    // records than expected overflows a bucket and takes the fallback path once; the estimate is then reset.
+    double distinct_est = 1.0;
+    uint64_t pull_lookups = 0;  // lookups of the pull whose status is pending
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
     bool pull_pending = false;
@@ -247,6 +252,10 @@ void harvest(SparseTable* t) {
         t->booked = 0;
         t->last_counts.assign(N, 0);
         for (int s = 0; s < N; s++) t->last_counts[s] = (int64_t)h.ubase[s + 1] - (int64_t)h.ubase[s];
+        if (t->pull_lookups > 0) {  // rises at once, falls within about ten pulls
+            const double now = (double)h.ubase[N] / (double)t->pull_lookups;
+            t->distinct_est = std::min(1.0, std::max(now, 0.75 * t->distinct_est + 0.25 * now));
+        }
         latch(t, dev_err_code(h.st.err), std::string("sparse pull: ") + dev_err_text(h.st.err));
         for (int s = 0; s < N && s < (int)t->pending_rows.size(); s++)
             if (t->last_counts[s] >= t->pending_rows[s])  // CHECK_LT(signs.size(), max_var_count)
@@ -430,11 +439,14 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
 }
 
 // dt_entries: entries of the global dedup table, or (use_lds) the number of buckets.
-size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds) {
+size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds, double distinct_est = 1.0) {
     Carver c{base};
     if (use_lds) {
         w.nbuckets = (uint32_t)dt_entries;
-        w.nb2 = (uint32_t)std::max<size_t>(1, (L + GRP_TARGET - 1) / GRP_TARGET);
+        // second-level buckets: GRP_TARGET records each on average if the batch has the expected share of
+        // distinct records plus a quarter (GRP_CAP is the room of a bucket)
+        const double expected = std::min(1.0, distinct_est * 1.25) * (double)L;
+        w.nb2 = (uint32_t)std::max<size_t>(1, ((size_t)expected + GRP_TARGET - 1) / GRP_TARGET);
         w.bcount = c.take<uint32_t>(dt_entries + 1 + w.nb2);  // zeroed together
         w.cursor2 = w.bcount + dt_entries + 1;
         w.recs = c.take<GroupRec>((size_t)w.nb2 * GRP_CAP);
@@ -1178,8 +1190,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         Scratch w{};
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
         carve_plan((char*)t->plan_buf.p, p, N, L);
-        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds)));
-        carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds, t->distinct_est)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds, t->distinct_est);
         w.span_cap = span_cap;
         t->plan_valid = false;
         TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN, use_lds ? w.bcount : nullptr,
@@ -1201,6 +1213,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                   reinterpret_cast<uint32_t*>(t->hpull), s.count);
         t->pull_pending = true;
         t->pull_slots = N;
+        t->pull_lookups = (uint64_t)L;
         t->pending_rows.assign(var_rows, var_rows + N);
         // a push of the same batch may reuse the analysis
         t->plan_valid = true;
@@ -1215,6 +1228,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             // rows the failed attempt inserted belong to signs of this batch; keep them counted
             t->hpull->st.err &= ~DEV_ERR_REMAP_OVERFLOW;
             harvest(t);
+            t->distinct_est = 1.0;  // the batch had more distinct records than the buckets were sized for
             t->latched = TN_OK;
             t->latched_msg.clear();
             use_lds = false;

@@ -742,3 +742,30 @@ def test_probe_chains_wrap_around_the_end_of_the_table(tn, oracle):
     grads = synth.make_grads(counts, D, 0.01, seed=6)
     pair.push_op(other, grads, [np.zeros(len(signs), np.int64)])
     assert pair.assert_rows_match(all_signs(values)) > 0.99
+
+
+def test_batch_with_more_distinct_signs_than_the_recent_ones(tn, oracle):
+    """The second-level buckets of the grouping are sized from the share of distinct records the
+    recent pulls had.  Twenty batches of heavily repeated signs, then one of the same size in which
+    every lookup is distinct: it overflows buckets, takes the fallback path, and everything
+    still equals the oracle; the batch after it runs on buckets sized for the worst case again."""
+    D = 8
+    rng = np.random.default_rng(41)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 200001, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool[:1000].view(np.uint64))
+    slots, per = 16, 4000
+    for step in range(20):
+        values = [pool[rng.integers(0, 300, per)] for _ in range(slots)]  # 64000 lookups, a few hundred signs
+        if step % 7 == 0:
+            check_pull(pair, values)
+        else:
+            tn.ops.sparse_table_pull([torch.empty((per + 1, D), device="cuda") for _ in values],
+                                     [dev(v) for v in values], pair.h)
+    for step in range(2):
+        values = [pool[1000 + (step * slots + s) * per:1000 + (step * slots + s + 1) * per] for s in range(slots)]
+        counts = check_pull(pair, values)  # every lookup a new sign
+        assert counts.tolist() == [per] * slots
+        grads = synth.make_grads(counts, D, 0.01, seed=step)
+        pair.push_op(values, grads, [np.zeros(per, np.int64) for _ in values])
+        assert pair.assert_rows_match(all_signs(values)) > 0.99
