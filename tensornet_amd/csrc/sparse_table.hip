@@ -514,9 +514,14 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
         for (int s = 0; s < N && ok; s++) ok = (size_t)lens[s] <= (size_t)LDS_MAX_SUB * LDS_BUCKET_TARGET;
         *use_lds = ok;
         if (ok) {
+            // A bucket's LDS table holds its distinct signs: LDS_BUCKET_TARGET lookups per bucket if all
+            // of them could be distinct, up to twice as many when the recent pulls repeated most signs
+            // (the same estimate, with the same margin and the same fallback, as for the second level).
+            const double share = std::min(1.0, std::max(0.5, t->distinct_est * 1.25));
+            const size_t target = (size_t)((double)LDS_BUCKET_TARGET / share);
             size_t nb = 0;
             for (int s = 0; s < N; s++) {
-                size_t sub = std::max<size_t>(1, ((size_t)lens[s] + LDS_BUCKET_TARGET - 1) / LDS_BUCKET_TARGET);
+                size_t sub = std::max<size_t>(1, ((size_t)lens[s] + target - 1) / target);
                 descs[s].tbase = (uint32_t)nb;
                 descs[s].tcap = (uint32_t)sub;
                 nb += sub;
