@@ -47,7 +47,7 @@ constexpr int LDS_BUCKET_TARGET = 768;  // average lookups per bucket
 constexpr int LDS_MAX_SUB = 4096;       // buckets per slot at most
 constexpr int LDS_TABLE = 2048;         // entries of a bucket's LDS hash table
 constexpr int DEDUP_THREADS = 512;      // a bucket's phases are short and separated by barriers: many wavefronts hide them
-constexpr int DEDUP_ITEMS = 2;          // lookups a thread of k_lds_dedup holds in registers
+constexpr int DEDUP_ITEMS = 4;          // lookups a thread of k_lds_dedup holds in registers
 constexpr int LDS_SPAN2 = 512;          // second-level buckets whose counts one first-level bucket gathers in LDS
 constexpr int GRP_TARGET = 1024;        // records per second-level bucket if every lookup were distinct
 constexpr int GRP_CAP = 1536;           // room of a second-level bucket
