@@ -26,6 +26,14 @@
 //                          w -= lr*g/(|g|+eps)           (tests/test_oracle_dense.py)
 //   row initialiser        distribution only (mean/std), as the reference's
 //                          own generator is wall-clock seeded.
+//   ShowDecay / DeleteByShow  closed forms and hand-made cases for every
+//                          optimizer and both elimination logics   (tests/test_oracle_decay.py)
+//   checkpoint streams     sparse blocks (text and binary) against hand-written
+//                          files and struct layouts, old-format detection,
+//                          round trips (tests/test_oracle_checkpoint.py); the dense
+//                          table's text file against texts written out by hand
+//                          from the reference's stream operators
+//                          (tests/test_oracle_dense_checkpoint.py)
 // One detail is an assumption, stated in the functions concerned: unqualified
 // sqrt/abs/log on floats are taken to resolve to the float overloads (the
 // libstdc++ <math.h>/<stdlib.h> wrappers being pulled in by the reference's
