@@ -767,37 +767,6 @@ __global__ __launch_bounds__(256) void k_write_mapped(const SlotDesc* __restrict
     }
 }
 
-// Push: are the signs of this call the ones the plan was built from?  With CLICKS the same
-// pass adds the non-zero labels to the click sums of the plan's member lists, which start
-// at zero (sparse_table_ops.cc:283-296; on a mismatch the plan is discarded anyway).  A
-// mismatch is also written to host_mismatch (pinned host memory, cleared by the host before the
-// launch), which the host reads once the kernel is done.
-template <bool CLICKS>
-__global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
-                                                       const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                       const uint64_t* __restrict__ vals_copy, DevStatus* status,
-                                                       const uint32_t* __restrict__ u_of_gi,
-                                                       const uint2* __restrict__ where_u, Member* list,
-                                                       uint32_t* host_mismatch) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
-    load_lbase(lb, lbase, N);
-    const uint32_t stride = gridDim.x * blockDim.x;
-    bool bad = false;
-    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        const int sl = find_slot(lb, N, gi);
-        const SlotDesc& d = descs[sl];
-        bad |= (uint64_t)d.values[gi - lb[sl]] != vals_copy[gi];
-        if (CLICKS) {
-            const int label = (int)d.labels[gi - lb[sl]];
-            if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
-        }
-    }
-    if (bad) {
-        atomicOr(&status->mismatch, 1u);
-        *host_mismatch = 1u;
-    }
-}
-
 // Push: batch_show = occurrences, batch_click = sum of labels per distinct sign
 // (sparse_table_ops.cc:283-296; labels are narrowed to int as there), kept in
 // the member lists.  Every sign starts at show 1 / click 0 ...
@@ -1212,6 +1181,77 @@ __device__ __forceinline__ bool src_record(const PushSrc& p, Member member, cons
     return true;
 }
 
+// The same through the gradient addresses worked out beforehand (k_member_grads): the record's
+// member entry and its address are independent loads, the gradient is one round trip away
+// instead of two.  ga == nullptr: resolve here.
+__device__ __forceinline__ bool record_at(const PushSrc& p, const Member* mem, const float* const* ga, uint32_t j,
+                                          const float*& g, int& show, int& click) {
+    if (!ga) return src_record(p, mem[j], g, show, click);
+    const Member m = mem[j];
+    g = ga[j];
+    show = m.show;
+    click = m.click;
+    return g != nullptr;
+}
+
+// Gradient row of every record of the groups with several records (their member lists fill the
+// top of the member array): gaddr[place], nullptr where the op's gradient matrix has no such row.
+// One coalesced pass that takes the slot descriptor out of the per-record chains of the apply
+// kernels for those groups.
+__global__ __launch_bounds__(256) void k_member_grads(PushSrc src, const DevStatus* status,
+                                                      const Member* __restrict__ list,
+                                                      const float** __restrict__ gaddr, uint32_t ids_cap) {
+    if (status->mismatch | status->abort) return;
+    const uint32_t n_members = status->n_members;
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < n_members; t += stride) {
+        const uint32_t place = ids_cap - n_members + t;
+        const float* gp = nullptr;
+        int sh, ck;
+        gaddr[place] = src_record(src, list[place], gp, sh, ck) ? gp : nullptr;
+    }
+}
+
+// Push: are the signs of this call the ones the plan was built from?  With CLICKS the same
+// pass adds the non-zero labels to the click sums of the plan's member lists, which start
+// at zero (sparse_table_ops.cc:283-296; on a mismatch the plan is discarded anyway).  A
+// mismatch is also written to host_mismatch (pinned host memory, cleared by the host before the
+// launch), which the host reads once the kernel is done.  With gaddr != nullptr the first
+// threads also do the work of k_member_grads (one launch less; harmless on a mismatch).
+template <bool CLICKS>
+__global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
+                                                       const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                       const uint64_t* __restrict__ vals_copy, DevStatus* status,
+                                                       const uint32_t* __restrict__ u_of_gi,
+                                                       const uint2* __restrict__ where_u, Member* list,
+                                                       uint32_t* host_mismatch, PushSrc src,
+                                                       const float** __restrict__ gaddr) {
+    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    load_lbase(lb, lbase, N);
+    const uint32_t stride = gridDim.x * blockDim.x;
+    bool bad = false;
+    const uint32_t n_members = gaddr ? status->n_members : 0;
+    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
+        if (gi < n_members) {  // the member lists of the groups with several records fill the top of the array
+            const uint32_t place = L - n_members + gi;
+            const float* gp = nullptr;
+            int sh, ck;
+            gaddr[place] = src_record(src, list[place], gp, sh, ck) ? gp : nullptr;
+        }
+        const int sl = find_slot(lb, N, gi);
+        const SlotDesc& d = descs[sl];
+        bad |= (uint64_t)d.values[gi - lb[sl]] != vals_copy[gi];
+        if (CLICKS) {
+            const int label = (int)d.labels[gi - lb[sl]];
+            if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
+        }
+    }
+    if (bad) {
+        atomicOr(&status->mismatch, 1u);
+        *host_mismatch = 1u;
+    }
+}
+
 // The three update rules on one element.
 //   AdaGrad  ada_grad_kernel.cc:105-129     Adam  adam_kernel.cc:112-125
 //   Ftrl     ftrl_kernel.cc:57-80
@@ -1324,7 +1364,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                                                    const uint32_t* __restrict__ grp_off,
                                                    const uint32_t* __restrict__ grp_cnt,
                                                    const Member* __restrict__ list, uint32_t big_k,
-                                                   uint32_t ids_cap) {
+                                                   uint32_t ids_cap, const float* const* __restrict__ gaddr) {
     // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
     if (status->mismatch | status->abort) return;
     const uint32_t n_multi = status->n_multi;
@@ -1341,6 +1381,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
         const Member* mem = list + grp_off[g];
+        const float* const* ga = gaddr ? gaddr + grp_off[g] : nullptr;
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         float4 w = reinterpret_cast<float4*>(wp)[sub];
@@ -1360,7 +1401,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         bool any = false;
         const float* gp;
         int nshow = 0, nclick = 0;
-        bool nok = src_record(src, mem[0], gp, nshow, nclick);
+        bool nok = record_at(src, mem, ga, 0, gp, nshow, nclick);
         float4 gnext = make_float4(0.f, 0.f, 0.f, 0.f);
         if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
         for (uint32_t j = 0; j < k; j++) {
@@ -1368,7 +1409,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
             const int bshow = nshow, bclick = nclick;
             const bool ok = nok;
             if (j + 1 < k) {
-                nok = src_record(src, mem[j + 1], gp, nshow, nclick);
+                nok = record_at(src, mem, ga, j + 1, gp, nshow, nclick);
                 if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
             }
             if (!ok) {
@@ -1464,7 +1505,8 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                                                   const uint32_t* __restrict__ grp_row,
                                                   const uint32_t* __restrict__ grp_off,
                                                   const uint32_t* __restrict__ grp_cnt,
-                                                  const Member* __restrict__ list, int gbuf_floats) {
+                                                  const Member* __restrict__ list, int gbuf_floats,
+                                                  const float* const* __restrict__ gaddr) {
     extern __shared__ float gbuf[];  // gbuf_floats floats of staging, then the row: rw[D], ra[D], rb[D]
     __shared__ const float* gptr[BIG_CHUNK];
     __shared__ int gshow[BIG_CHUNK], gok[BIG_CHUNK];
@@ -1519,7 +1561,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             int sh = 0, ck = 0;
             if (lane < cn) {
                 const float* gp = nullptr;
-                ok = src_record(src, list[off + c0 + lane], gp, sh, ck);
+                ok = record_at(src, list + off + c0, gaddr ? gaddr + off + c0 : nullptr, lane, gp, sh, ck);
                 gptr[lane] = gp;
                 gshow[lane] = sh;
                 gok[lane] = ok ? 1 : 0;

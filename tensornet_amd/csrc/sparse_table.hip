@@ -364,6 +364,7 @@ struct Plan {
     uint2* where_u;        // record -> {its place in `list`, its group}
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     uint32_t* newlist;     // groups whose row was inserted by the pull
+    const float** gaddr;   // gradient row of every record of the groups with several records (a push fills it)
 };
 
 // Per-call scratch of the analysis.
@@ -415,6 +416,7 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.where_u = c.take<uint2>(n);
     p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
     p.newlist = c.take<uint32_t>(n);
+    p.gaddr = c.take<const float*>(n);
 }
 
 void carve_group_scratch(Carver& c, Scratch& w, size_t n) {
@@ -702,24 +704,31 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
 // stream beside it, forked from and joined back into the caller's stream by events.
 template <int KIND>
 int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
-                      const Plan& p, int64_t n_upper, hipStream_t st) {
+                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready) {
     const uint32_t big_k = big_threshold(s);
     const uint32_t ids_cap = (uint32_t)n_upper;
     const bool with_big = big_k != 0xFFFFFFFFu;
+    const float* const* gaddr = (with_big && !src.infos && !src.flat) ? p.gaddr : nullptr;
     if (with_big) {
+        // op-level gradients: their addresses for the records of the groups with several records, once, in a
+        // coalesced pass ahead of everything (beside k_apply_single it would take several times as long)
+        if (gaddr && !addr_ready)
+            TN_LAUNCH(k_member_grads, dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, src, ds, p.list,
+                      p.gaddr, ids_cap);
         TN_HIP(hipEventRecord(t->fork_ev, st));
         TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
         const int gfloats = big_gbuf_floats(s.D);
         TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
                       big_lds_bytes(s.D), t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
-                      p.list, gfloats);
+                      p.list, gfloats, gaddr);
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
         TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
                   o, src, ds, p.grp_row, p.list);                                                                 \
         TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256),    \
-                  with_big ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap); \
+                  with_big ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,    \
+                  gaddr);                                                                                         \
     } while (0)
     switch (lpg) {
         case 1: TN_LAUNCH_VEC(1); break;
@@ -741,8 +750,9 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
 }
 
 // Applies the grouped records; n_upper bounds the number of records.
+// addr_ready: p.gaddr already holds the gradient addresses of the multi-record groups' records.
 int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
-                 hipStream_t st) {
+                 hipStream_t st, bool addr_ready = false) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     int lpg = 0;
@@ -751,9 +761,9 @@ int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* d
         if (q >= 1 && q <= 32 && (q & (q - 1)) == 0) lpg = q;
     }
     switch (o.kind) {
-        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st);
-        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st);
-        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st);
+        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
+        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
+        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
     }
 }
 
@@ -1373,15 +1383,20 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // the outcome comes back through pinned host memory, written by the verify kernel itself
         t->hpush->st.mismatch = 0;
         uint32_t* host_mismatch = &t->hpush->st.mismatch;
+        // op-level gradients (not pooled): the verify pass also works out the gradient addresses of the records
+        // of the groups with several records (see k_member_grads)
+        const PushSrc vsrc = op_source(p, grad_dim);
+        const bool addr_in_verify = !pooled && big_threshold(t->store) != 0xFFFFFFFFu;
+        const float** vgaddr = addr_in_verify ? p.gaddr : nullptr;
         if (clicks) {
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
             TN_LAUNCH((k_verify_values<true>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.vals_copy,
-                      ds, p.u_of_gi, p.where_u, p.list, host_mismatch);
+                      ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         } else {
             TN_LAUNCH((k_verify_values<false>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L,
-                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch);
+                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         }
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // Counts and apply kernels are queued before the host knows the outcome: the counts only
@@ -1389,7 +1404,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // return at once when the mismatch flag is set.  The device never waits for the host.
         if (!t->plan_has_show) TN_TRY(launch_counts());
         TN_TRY(prepare_src());
-        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
+        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify));
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
