@@ -403,14 +403,36 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase, int N, uint32_t L,
     const uint8_t* __restrict__ flag8, const uint32_t* __restrict__ tileoff, const uint32_t* __restrict__ cnt_at,
     uint32_t* __restrict__ wordpre, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
-    uint32_t* __restrict__ uniq_slot, uint32_t* __restrict__ ushow) {
+    uint32_t* __restrict__ uniq_slot, uint32_t* __restrict__ ushow, const uint32_t* __restrict__ tilesum,
+    DevStatus* status) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     __shared__ uint32_t red[4];
     load_lbase(lb, lbase, N);
     const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
     uint32_t bits = 0;
     if (base < L) bits = flag8[base / REMAP_ITEMS];
-    uint32_t u = tileoff[blockIdx.x] + block_excl_scan_256<uint32_t>(__popc(bits), red, nullptr);
+    uint32_t off;
+    if (tilesum) {
+        // a few thousand tiles: every workgroup adds up the counts of the tiles before its own (they sit in
+        // L2), which costs less than a scan kernel of one workgroup between two launches
+        uint32_t part = 0;
+        for (uint32_t i = threadIdx.x; i < blockIdx.x; i += REMAP_THREADS) part += tilesum[i];
+        off = block_sum_256(part, red);
+    } else {
+        off = tileoff[blockIdx.x];
+    }
+    uint32_t total;
+    uint32_t u = off + block_excl_scan_256<uint32_t>(__popc(bits), red, &total);
+    if (tilesum && blockIdx.x == gridDim.x - 1) {  // what k_scan_tiles leaves besides the offsets
+        const uint32_t U = off + total;
+        if (threadIdx.x == 0) {
+            status->n_unique = U;
+            const uint32_t g = U + U / 2;
+            status->gcap = g < 16 ? 16 : g;
+        }
+        for (int sl = threadIdx.x; sl <= N; sl += REMAP_THREADS)
+            if (lb[sl] >= L) ubase[sl] = U;
+    }
     if (base >= L) return;
     if ((base & 63u) == 0) wordpre[base >> 6] = u;  // first occurrences before this 64-lookup word
     int sls[REMAP_ITEMS];
@@ -487,7 +509,9 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
                                                      uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
     __shared__ unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
     __shared__ unsigned long long mlo[GRP_TABLE + 1], mhi[GRP_TABLE + 1];
-    __shared__ uint32_t einfo[GRP_TABLE + 1], eoffs[GRP_TABLE + 1];
+    // Once every record knows its entry (rech) the keys are dead: the entries' group numbers and offsets
+    // take their place, which lets three workgroups instead of two share a CU's LDS.
+    uint2* const einfo = reinterpret_cast<uint2*>(keys);  // x: info word, y: records before the group
     __shared__ uint16_t rech[GRP_CAP];
     __shared__ uint32_t lb[GRP_SLOTS + 1];
     __shared__ unsigned long long sh[GRP_THREADS / 64];
@@ -557,12 +581,11 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
             if (k == 0) continue;
             const uint32_t e = j * GRP_THREADS + threadIdx.x;
             if (k == 1) {
-                einfo[e] = (uint32_t)(ex & 0xFFFF) | (1u << 24);
-                eoffs[e] = 0;
+                einfo[e] = make_uint2((uint32_t)(ex & 0xFFFF) | (1u << 24), 0u);
                 ex += 1ull;
             } else {
-                einfo[e] = (uint32_t)((ex >> 16) & 0xFFFF) | ((uint32_t)(ex >> 48) << 12) | (k << 24);
-                eoffs[e] = (uint32_t)((ex >> 32) & 0xFFFF);
+                einfo[e] = make_uint2((uint32_t)((ex >> 16) & 0xFFFF) | ((uint32_t)(ex >> 48) << 12) | (k << 24),
+                                      (uint32_t)((ex >> 32) & 0xFFFF));
                 ex += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
             }
         }
@@ -578,7 +601,8 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
                 place = (uint32_t)__popcll(mlo[h] & ((1ull << s1) - 1ull));
             else
                 place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (s1 - 64)) - 1ull));
-            aux[first + i] = make_uint2(einfo[h], eoffs[h] | (place << 16) | (s1 << 24));
+            const uint2 ei = einfo[h];
+            aux[first + i] = make_uint2(ei.x, ei.y | (place << 16) | (s1 << 24));
         }
         __syncthreads();
     }
@@ -670,7 +694,7 @@ __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t
 // the arrays is first put together in LDS and then copied out in order; only where_u, indexed
 // by the distinct index of the record, stays a scattered store.  where_u[u] = {place in the member
 // list, table row of the record's sign (rrow, from k_probe_recs)}; the groups get the rows too.
-__global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+__global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6, 8))) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
                                                     const uint4* __restrict__ bcounts,
@@ -681,18 +705,49 @@ __global__ __launch_bounds__(EMIT_THREADS) void k_group_emit(uint32_t nb2, const
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
                                                     uint2* __restrict__ where_u,
                                                     const uint32_t* __restrict__ rrow,
-                                                    uint32_t* __restrict__ grp_row) {
+                                                    uint32_t* __restrict__ grp_row, DevStatus* status) {
     // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
     // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
     __shared__ Member s_list[GRP_CAP];
     __shared__ unsigned long long s_sign[GRP_CAP];
     __shared__ uint32_t s_off[GRP_CAP], s_row[GRP_CAP];
     __shared__ uint16_t s_cnt[GRP_CAP];  // at most GRP_SLOTS records per group
+    __shared__ uint4 s_part[EMIT_THREADS / 64];
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
-        if (n == 0) continue;
+        uint4 bb;
+        if (bbase) {
+            if (n == 0) continue;
+            bb = bbase[c];
+        } else {
+            // One bucket per workgroup and a few thousand buckets: the counts of the buckets before this one
+            // (in L2) are added up here, which saves the launch of a scan kernel between the grouping's two
+            // passes; the last workgroup leaves the totals (what k_group_offsets leaves).
+            uint4 acc = make_uint4(0, 0, 0, 0);
+            for (uint32_t i = threadIdx.x; i < c; i += EMIT_THREADS) {
+                const uint4 v = bcounts[i];
+                acc = make_uint4(acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w);
+            }
+            for (int o = 32; o > 0; o >>= 1)
+                acc = make_uint4(acc.x + __shfl_xor(acc.x, o), acc.y + __shfl_xor(acc.y, o), acc.z + __shfl_xor(acc.z, o),
+                                 acc.w + __shfl_xor(acc.w, o));
+            if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = acc;
+            __syncthreads();
+            bb = make_uint4(0, 0, 0, 0);
+            for (int wv = 0; wv < EMIT_THREADS / 64; wv++) {
+                const uint4 v = s_part[wv];
+                bb = make_uint4(bb.x + v.x, bb.y + v.y, bb.z + v.z, bb.w + v.w);
+            }
+            if (c == nb2 - 1 && threadIdx.x == 0) {
+                const uint4 v = bcounts[c];
+                status->n_single = bb.x + v.x;
+                status->n_multi = bb.y + v.y;
+                status->n_members = bb.z + v.z;
+                status->n_big = bb.w + v.w;
+            }
+            if (n == 0) continue;  // (own sums: the workgroup has this one bucket, s_part is not written again)
+        }
         const size_t first = (size_t)c * GRP_CAP;
-        const uint4 bb = bbase[c];
         const uint4 bc = bcounts[c];
         const uint32_t n1 = bc.x, nm = bc.y, nr = bc.z;  // groups of one record, of several, records of the latter
         const uint32_t top = ids_cap - 1 - bb.z;         // member place of local member 0 of the several-record groups

@@ -19,7 +19,8 @@ namespace {
 constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:266
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
-constexpr int PROBE_RECS_GRID = 1024;                // workgroups of k_probe_recs (measured: 512-1024 are best)
+constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 512-1024 are best)
+constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to which no scan kernel runs between its launches
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
 constexpr size_t LDS_MIN_LOOKUPS = 32768;  // smaller batches are launch-bound: the shorter global-table path wins
 
@@ -623,6 +624,8 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     const Store& s = t->store;
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
     const bool lds_groups = use_lds && N <= GRP_SLOTS;
+    // second-level buckets up to which k_group_emit adds up the bucket counts itself (one bucket per workgroup)
+    const bool own_offsets = w.nb2 <= (uint32_t)GRID_CAP * 4;
     if (use_lds) {
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
         const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
@@ -646,7 +649,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
             TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), t->side, p.lbase, N, w.nb2, w.cursor2, w.recs,
                       big_threshold(s), w.aux, w.bcounts);
-            TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
+            if (!own_offsets) TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
             TN_HIP(hipEventRecord(t->join_ev, t->side));
             // ... and so do the rows of the records' signs, on a stream of their own
             TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
@@ -656,13 +659,16 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
-        TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
+        // up to SELF_SCAN_TILES tiles the ranking pass adds up the tile counts itself
+        const uint32_t* own_sums = w.ntiles <= SELF_SCAN_TILES ? w.tilesum : nullptr;
+        if (!own_sums)
+            TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
         if (lds_groups)
             TN_LAUNCH((k_lds_assign<false>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
         else
             TN_LAUNCH((k_lds_assign<true>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow);
+                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
         TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.flag8, w.wordpre,
                   p.u_of_gi);
     } else {
@@ -682,8 +688,9 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
         TN_HIP(hipStreamWaitEvent(st, t->join2_ev, 0));
-        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux, w.bbase, w.bcounts, w.flag8, w.wordpre, L,
-                  big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row);
+        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
+                  own_offsets ? nullptr : w.bbase, w.bcounts, w.flag8, w.wordpre, L, big_threshold(s),
+                  p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds);
         return TN_OK;  // the rows were found beside the grouping
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
