@@ -59,13 +59,16 @@ constexpr int EMIT_THREADS = 512;
 constexpr int EMIT_RECS = GRP_CAP / EMIT_THREADS;  // records per thread of k_group_emit
 constexpr int GRP_ITEMS = (GRP_TABLE + 1 + GRP_THREADS - 1) / GRP_THREADS;
 constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
+static_assert((uint64_t)LDS_MAX_SUB * LDS_BUCKET_TARGET <= 0xFFFFFFull && GRP_SLOTS <= 256,
+              "a record's word holds the occurrences of a sign in its slot and the slot");
 
 // A distinct (slot, sign) record on its way to the grouping.
 struct GroupRec {
     uint64_t sign;
     uint32_t gi;   // position of its first occurrence
-    uint32_t cnt;  // occurrences in its slot
+    uint32_t cnt;  // bits 0-23 occurrences in its slot, 24-31 the slot (< GRP_SLOTS)
 };
+constexpr uint32_t REC_CNT_MASK = 0xFFFFFFu;
 
 __device__ __forceinline__ uint32_t group_bucket(uint64_t sign, uint32_t nb2) {
     return (uint32_t)__umul64hi(mix64(sign), (uint64_t)nb2);
@@ -203,11 +206,12 @@ __global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict_
             }
         }
         __syncthreads();
-        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
+        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, const SlotDesc& d, uint64_t sign) {
             const uint32_t local = bucket_of(d, sign) - b0;
             if (local < span) {
                 const uint32_t at = atomicAdd(&hist[local], 1u);
-                prec[at] = make_ulonglong2(sign, gi);  // one 16-byte store per lookup: these stores are what the pass costs
+                // one 16-byte store per lookup (these stores are what the pass costs): sign, position, slot
+                prec[at] = make_ulonglong2(sign, (uint64_t)gi | ((uint64_t)(uint32_t)sl << 32));
             }
         });
         __syncthreads();
@@ -230,22 +234,13 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
     __shared__ uint32_t minpos[LDS_TABLE + 1];
     __shared__ uint32_t cnts[LDS_TABLE + 1];
     __shared__ uint32_t hist2[EMIT ? LDS_SPAN2 : 1];
-    __shared__ uint32_t c_lo_sh;
+    __shared__ uint32_t c_lo_sh, slot_sh;
     for (uint32_t b = blockIdx.x; b < nbuckets; b += gridDim.x) {
         const uint32_t lo = bstart[b], hi = bstart[b + 1];
         if (lo == hi) continue;
-        for (int i = threadIdx.x; i <= LDS_TABLE; i += DEDUP_THREADS) {
-            keys[i] = EMPTY_KEY;
-            minpos[i] = 0xFFFFFFFFu;
-            cnts[i] = 0;
-        }
-        if (EMIT) {
-            for (int i = threadIdx.x; i < LDS_SPAN2; i += DEDUP_THREADS) hist2[i] = 0;
-            if (threadIdx.x == 0) c_lo_sh = 0xFFFFFFFFu;
-        }
-        __syncthreads();
         // The bucket's lookups are taken DEDUP_ITEMS per thread at a time, all loads of a round
-        // issued together; a bucket that fits one round (the usual case) is read once.
+        // issued together; a bucket that fits one round (the usual case) is read once.  The first
+        // round's loads are in flight while the tables are cleared.
         uint64_t sg[DEDUP_ITEMS];
         uint32_t gp[DEDUP_ITEMS];
         const uint32_t round = DEDUP_THREADS * DEDUP_ITEMS;
@@ -257,11 +252,23 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                 const ulonglong2 r = (i < hi) ? prec[i] : make_ulonglong2(0, 0xFFFFFFFFull);  // no position: nothing to do
                 sg[j] = r.x;
                 gp[j] = (uint32_t)r.y;
+                if (EMIT && j == 0 && i == lo) slot_sh = (uint32_t)(r.y >> 32);  // every lookup of a bucket is of one slot
             }
         };
+        load_round(lo);
+        for (int i = threadIdx.x; i <= LDS_TABLE; i += DEDUP_THREADS) {
+            keys[i] = EMPTY_KEY;
+            minpos[i] = 0xFFFFFFFFu;
+            cnts[i] = 0;
+        }
+        if (EMIT) {
+            for (int i = threadIdx.x; i < LDS_SPAN2; i += DEDUP_THREADS) hist2[i] = 0;
+            if (threadIdx.x == 0) c_lo_sh = 0xFFFFFFFFu;
+        }
+        __syncthreads();
         uint32_t c_min = 0xFFFFFFFFu;
         for (uint32_t base = lo; base < hi; base += round) {
-            load_round(base);
+            if (base != lo) load_round(base);
 #pragma unroll
             for (int j = 0; j < DEDUP_ITEMS; j++) {
                 const uint64_t sign = sg[j];
@@ -352,7 +359,7 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                 GroupRec r;
                 r.sign = (e == LDS_TABLE) ? EMPTY_KEY : (uint64_t)keys[e];
                 r.gi = minpos[e];
-                r.cnt = cnt;
+                r.cnt = cnt | (slot_sh << 24);
                 const uint32_t c = group_bucket(r.sign, nb2);
                 const uint32_t local = c - c_lo;
                 const uint32_t at = (local < LDS_SPAN2) ? atomicAdd(&hist2[local], 1u) : atomicAdd(&cursor2[c], 1u);
@@ -503,8 +510,7 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
 //   y: bits 0-15 records of the bucket's earlier several-record groups, 16-23 place, 24-31 slot
 // and per bucket the number of groups with one record, with several, the
 // records of the latter, and the big groups.  At most GRP_SLOTS slots.
-__global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __restrict__ lbase, int N, uint32_t nb2,
-                                                     const uint32_t* __restrict__ cursor2,
+__global__ __launch_bounds__(GRP_THREADS) void k_group_count(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                      const GroupRec* __restrict__ recs, uint32_t big_k,
                                                      uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
     __shared__ unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
@@ -513,9 +519,7 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
     // take their place, which lets three workgroups instead of two share a CU's LDS.
     uint2* const einfo = reinterpret_cast<uint2*>(keys);  // x: info word, y: records before the group
     __shared__ uint16_t rech[GRP_CAP];
-    __shared__ uint32_t lb[GRP_SLOTS + 1];
     __shared__ unsigned long long sh[GRP_THREADS / 64];
-    load_lbase(lb, lbase, N);
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         if (n == 0) {
@@ -523,13 +527,8 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
             continue;
         }
         const size_t first = (size_t)c * GRP_CAP;
-        for (int i = threadIdx.x; i <= GRP_TABLE; i += GRP_THREADS) {
-            keys[i] = EMPTY_KEY;
-            mlo[i] = 0;
-            mhi[i] = 0;
-        }
-        __syncthreads();
         // all records of the bucket sit in registers (GRP_CAP = GRP_THREADS x GRP_RECS), loaded together
+        // and in flight while the table is cleared
         uint64_t sg[GRP_RECS];
         uint32_t sl[GRP_RECS];  // slot of the record, 0xFFFFFFFF = no record
 #pragma unroll
@@ -540,9 +539,15 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
             if (i < n) {
                 const GroupRec r = recs[first + i];
                 sg[j] = r.sign;
-                sl[j] = r.gi;
+                sl[j] = r.cnt >> 24;
             }
         }
+        for (int i = threadIdx.x; i <= GRP_TABLE; i += GRP_THREADS) {
+            keys[i] = EMPTY_KEY;
+            mlo[i] = 0;
+            mhi[i] = 0;
+        }
+        __syncthreads();
 #pragma unroll
         for (int j = 0; j < GRP_RECS; j++) {
             if (sl[j] == 0xFFFFFFFFu) continue;
@@ -557,7 +562,6 @@ __global__ __launch_bounds__(GRP_THREADS) void k_group_count(const uint32_t* __r
                     h = (h + 1) & (GRP_TABLE - 1);
                 }
             }
-            sl[j] = (uint32_t)find_slot(lb, N, sl[j]);
             atomicOr(sl[j] < 64 ? &mlo[h] : &mhi[h], 1ull << (sl[j] & 63));
             rech[j * GRP_THREADS + threadIdx.x] = (uint16_t)h;
         }
@@ -715,6 +719,20 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
     __shared__ uint4 s_part[EMIT_THREADS / 64];
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+        const size_t first = (size_t)c * GRP_CAP;
+        // the bucket's records first: their loads are in flight while the bucket's offsets are worked out
+        GroupRec rs[EMIT_RECS];
+        uint2 as[EMIT_RECS];
+        uint32_t us[EMIT_RECS], rows[EMIT_RECS];
+#pragma unroll
+        for (int j = 0; j < EMIT_RECS; j++) {
+            const uint32_t i = j * EMIT_THREADS + threadIdx.x;
+            if (i < n) {
+                rs[j] = recs[first + i];
+                as[j] = aux[first + i];
+                rows[j] = rrow[first + i];
+            }
+        }
         uint4 bb;
         if (bbase) {
             if (n == 0) continue;
@@ -747,22 +765,9 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             }
             if (n == 0) continue;  // (own sums: the workgroup has this one bucket, s_part is not written again)
         }
-        const size_t first = (size_t)c * GRP_CAP;
         const uint4 bc = bcounts[c];
         const uint32_t n1 = bc.x, nm = bc.y, nr = bc.z;  // groups of one record, of several, records of the latter
         const uint32_t top = ids_cap - 1 - bb.z;         // member place of local member 0 of the several-record groups
-        GroupRec rs[EMIT_RECS];
-        uint2 as[EMIT_RECS];
-        uint32_t us[EMIT_RECS], rows[EMIT_RECS];
-#pragma unroll
-        for (int j = 0; j < EMIT_RECS; j++) {
-            const uint32_t i = j * EMIT_THREADS + threadIdx.x;
-            if (i < n) {
-                rs[j] = recs[first + i];
-                as[j] = aux[first + i];
-                rows[j] = rrow[first + i];
-            }
-        }
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++)
             if (j * EMIT_THREADS + threadIdx.x < n) us[j] = rank_of(flag8, wordpre, rs[j].gi);
@@ -776,7 +781,7 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             Member m;
             m.u = us[j];
             m.slot = sl;
-            m.show = (int32_t)r.cnt;  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+            m.show = (int32_t)(r.cnt & REC_CNT_MASK);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             m.click = 0;
             if (k == 1) {
                 const uint32_t g = bb.x + idx;

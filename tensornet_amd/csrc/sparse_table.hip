@@ -647,7 +647,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
             TN_HIP(hipEventRecord(t->fork_ev, st));
             TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
-            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), t->side, p.lbase, N, w.nb2, w.cursor2, w.recs,
+            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), t->side, w.nb2, w.cursor2, w.recs,
                       big_threshold(s), w.aux, w.bcounts);
             if (!own_offsets) TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
             TN_HIP(hipEventRecord(t->join_ev, t->side));
