@@ -390,7 +390,15 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const u
     __shared__ uint32_t red[4];
     const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
     uint32_t bits = 0;
-    if (base < L) {
+    static_assert(REMAP_ITEMS == 8, "a thread's lookups are two 16-byte loads");
+    if (base + REMAP_ITEMS <= L) {
+        const uint4 a = reinterpret_cast<const uint4*>(first_of + base)[0];
+        const uint4 b = reinterpret_cast<const uint4*>(first_of + base)[1];
+        bits = (a.x == base ? 1u : 0u) | (a.y == base + 1 ? 2u : 0u) | (a.z == base + 2 ? 4u : 0u) |
+               (a.w == base + 3 ? 8u : 0u) | (b.x == base + 4 ? 16u : 0u) | (b.y == base + 5 ? 32u : 0u) |
+               (b.z == base + 6 ? 64u : 0u) | (b.w == base + 7 ? 128u : 0u);
+        flag8[base / REMAP_ITEMS] = (uint8_t)bits;
+    } else if (base < L) {
         for (int j = 0; j < REMAP_ITEMS; j++) {
             const uint32_t gi = base + j;
             if (gi >= L) break;
@@ -491,13 +499,44 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
                                                     uint32_t* __restrict__ u_of_gi) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
+    // four consecutive lookups per thread: one 16-byte load and store, one slot search
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        const uint32_t f = first_of[gi];
-        const uint32_t u = rank_of(flag8, wordpre, f);
-        u_of_gi[gi] = u | (f == gi ? FIRST_BIT : 0u);
-        const int sl = find_slot(lb, N, gi);
-        descs[sl].mapped[gi - lb[sl]] = (int64_t)(u - ubase[sl]);
+    const uint32_t quads = (L + 3) / 4;
+    for (uint32_t q = blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
+        const uint32_t g0 = q * 4;
+        uint32_t f[4], u[4];
+        if (g0 + 4 <= L) {
+            const uint4 v = reinterpret_cast<const uint4*>(first_of)[q];
+            f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) f[j] = g0 + j < L ? first_of[g0 + j] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) u[j] = rank_of(flag8, wordpre, f[j]);
+        if (g0 + 4 <= L) {
+            reinterpret_cast<uint4*>(u_of_gi)[q] =
+                make_uint4(u[0] | (f[0] == g0 ? FIRST_BIT : 0u), u[1] | (f[1] == g0 + 1 ? FIRST_BIT : 0u),
+                           u[2] | (f[2] == g0 + 2 ? FIRST_BIT : 0u), u[3] | (f[3] == g0 + 3 ? FIRST_BIT : 0u));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (g0 + j < L) u_of_gi[g0 + j] = u[j] | (f[j] == g0 + j ? FIRST_BIT : 0u);
+        }
+        int sl = find_slot(lb, N, g0);
+        int64_t* out = descs[sl].mapped - lb[sl];
+        uint32_t ub = ubase[sl];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t gi = g0 + j;
+            if (gi >= L) break;
+            if (gi >= lb[sl + 1]) {
+                do sl++; while (gi >= lb[sl + 1]);
+                out = descs[sl].mapped - lb[sl];
+                ub = ubase[sl];
+            }
+            out[gi] = (int64_t)(u[j] - ub);
+        }
     }
 }
 
