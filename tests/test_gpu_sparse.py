@@ -769,3 +769,56 @@ def test_batch_with_more_distinct_signs_than_the_recent_ones(tn, oracle):
         grads = synth.make_grads(counts, D, 0.01, seed=step)
         pair.push_op(values, grads, [np.zeros(per, np.int64) for _ in values])
         assert pair.assert_rows_match(all_signs(values)) > 0.99
+
+
+@pytest.mark.gpu
+def test_batch_beyond_the_sizes_the_fused_scans_cover(tn, oracle):
+    """18 M lookups in one call: more tiles and more second-level buckets than the ranking
+    and member-list kernels add up themselves, so the separate scan kernels run.  Too large
+    for the CPU oracle in seconds: the same size-independent properties as for cfg3."""
+    D, N, per_slot = 16, 24, 750000
+    opt = tn.core.AdaGrad(learning_rate=0.01, initial_g2sum=0.1)
+    h = tn.core.create_sparse_table(opt, "", D, False, "")
+    tn.core.reserve_sparse_table(h, 4 * 10 ** 6)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    # a shared vocabulary, so that signs repeat inside a slot and across slots
+    gvalues = [synth.splitmix64_torch(torch.randint(1, 3 * 10 ** 6, (per_slot + 1000 * s,), generator=gen,
+                                                    device="cuda")) for s in range(N)]
+    L = sum(len(v) for v in gvalues)
+    assert L > 8192 * 2048
+    uniq = torch.unique(torch.cat(gvalues))
+    w0 = synth.snapshot_rows_torch(uniq, D)
+    tn.ops.table_load_rows(h, uniq, w0)
+    rows = [len(v) + 1 for v in gvalues]
+    gvars = [torch.full((r, D), 9.0, device="cuda") for r in rows]
+    mapped = tn.ops.sparse_table_pull(gvars, gvalues, h)
+    counts = tn.ops.sparse_table_last_unique_counts(h, N)
+    for s in (0, 7, N - 1):
+        v, m = gvalues[s], mapped[s]
+        u, inv = torch.unique(v, return_inverse=True)
+        assert counts[s] == u.numel() == int(m.max()) + 1
+        first = torch.full((u.numel(),), len(v), dtype=torch.int64, device="cuda")
+        first.scatter_reduce_(0, inv, torch.arange(len(v), device="cuda"), reduce="amin")
+        first_by_id = torch.empty_like(first)
+        first_by_id[m[first]] = first
+        assert bool((first_by_id[1:] > first_by_id[:-1]).all())
+        assert torch.equal(m, m[first][inv])
+        assert torch.equal(gvars[s][m], synth.snapshot_rows_torch(v, D))
+        assert bool((gvars[s][counts[s]:] == 9.0).all())
+    # a constant gradient: a sign present in k slots gets k sequential Applies
+    g = 0.5
+    grads = [torch.full((c, D), g, device="cuda") for c in counts]
+    labels = [torch.ones_like(v) for v in gvalues]
+    tn.ops.sparse_table_push(gvalues, grads, labels, h)
+    tn.ops.sparse_table_sync(h)
+    w2, st2, found = tn.ops.table_export_rows(h, uniq)
+    assert bool(found.all())
+    k = torch.zeros(uniq.numel(), device="cuda")
+    for v in gvalues:
+        k[torch.searchsorted(uniq, torch.unique(v))] += 1
+    np.testing.assert_allclose(st2[:, 0].cpu().numpy(), (0.1 + k * g * g).cpu().numpy(), rtol=1e-5)
+    assert float(st2[:, 1].double().sum()) == float(L) == float(st2[:, 2].double().sum())  # shows, clicks
+    steps = torch.arange(1, int(k.max()) + 1, device="cuda", dtype=torch.float64)
+    cum = torch.cumsum(0.01 * g / torch.sqrt(0.1 + steps * g * g), 0)
+    expect = w0.double() - cum[(k - 1).long()][:, None]
+    np.testing.assert_allclose(w2.cpu().numpy(), expect.cpu().numpy(), rtol=RTOL, atol=1e-6)
