@@ -168,7 +168,7 @@ def cpu_baseline(cfg, values, grads_sigma):
     t1 = time.perf_counter()
     assert rc == 0
     grads = synth.make_grads(counts, dim, grads_sigma)
-    labels = [np.zeros(len(v), np.int64) for v in values]
+    labels = synth.make_labels(values, 0)
     t2 = time.perf_counter()
     rc, _ = t.push_op(values, grads, labels)
     t3 = time.perf_counter()
@@ -245,9 +245,9 @@ def main():
     batches = []
     rng = torch.Generator(device="cuda")
     rng.manual_seed(0)
-    for hb in host_batches:
+    for b, hb in enumerate(host_batches):
         values = [torch.from_numpy(v).cuda() for v in hb]
-        labels = [torch.zeros_like(v) for v in values]
+        labels = [torch.from_numpy(l).cuda() for l in synth.make_labels(hb, b)]
         # gradient matrices have one row per possible distinct sign; the op reads the first U_s
         grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
         vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
@@ -341,9 +341,10 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "%s: batch %d x %d slots, %s id lists, Zipf(%.2f) over %.0e vocab, dim %d %s, %d resident keys"
+            "workload": "%s: batch %d x %d slots, %s id lists, Zipf(%.2f) over %.0e vocab, dim %d %s, %d resident keys, "
+                        "feature labels 1 on %.0f %% of the lookups"
                         % (args.config, cfg["batch"], cfg["slots"], cfg["lens"], cfg["zipf_s"], cfg["vocab"], dim,
-                           opt_name, resident),
+                           opt_name, resident, 100 * synth.CLICK_RATE),
             "lookups_per_step": mean_L,
             "distinct_rows_per_step": mean_U,
             "globally_distinct_keys_batch0": G0,

@@ -1218,6 +1218,17 @@ __global__ __launch_bounds__(256) void k_member_grads(PushSrc src, const DevStat
 // mismatch is also written to host_mismatch (pinned host memory, cleared by the host before the
 // launch), which the host reads once the kernel is done.  With gaddr != nullptr the first
 // threads also do the work of k_member_grads (one launch less; harmless on a mismatch).
+//
+// One atomic per non-zero label would queue up on the entries of the frequent signs (a
+// sign that takes a few percent of a slot's lookups receives thousands of adds): a workgroup
+// first sums the labels of its tile per distinct record in an LDS table and then adds every
+// entry to memory once.  A label that finds the table crowded goes to memory directly.
+constexpr int VERIFY_ITEMS = 8;
+constexpr int VERIFY_TILE = 256 * VERIFY_ITEMS;  // lookups per tile
+constexpr int CLICK_BITS = 11;
+constexpr int CLICK_TABLE = 1 << CLICK_BITS;     // entries of the tile's click table
+constexpr int CLICK_TRIES = 16;
+
 template <bool CLICKS>
 __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
@@ -1227,23 +1238,83 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                                                        uint32_t* host_mismatch, PushSrc src,
                                                        const float** __restrict__ gaddr) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
+    __shared__ uint32_t ckey[CLICKS ? CLICK_TABLE : 1];
+    __shared__ int csum[CLICKS ? CLICK_TABLE : 1];
     load_lbase(lb, lbase, N);
-    const uint32_t stride = gridDim.x * blockDim.x;
     bool bad = false;
     const uint32_t n_members = gaddr ? status->n_members : 0;
-    for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        if (gi < n_members) {  // the member lists of the groups with several records fill the top of the array
-            const uint32_t place = L - n_members + gi;
-            const float* gp = nullptr;
-            int sh, ck;
-            gaddr[place] = src_record(src, list[place], gp, sh, ck) ? gp : nullptr;
-        }
-        const int sl = find_slot(lb, N, gi);
-        const SlotDesc& d = descs[sl];
-        bad |= (uint64_t)d.values[gi - lb[sl]] != vals_copy[gi];
+    const uint32_t ntiles = (L + VERIFY_TILE - 1) / VERIFY_TILE;
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         if (CLICKS) {
-            const int label = (int)d.labels[gi - lb[sl]];
-            if (label != 0) atomicAdd(&list[where_u[u_of_gi[gi] & ~FIRST_BIT].x].click, label);
+            for (int i = threadIdx.x; i < CLICK_TABLE; i += 256) {
+                ckey[i] = 0xFFFFFFFFu;  // no distinct index: they stay below FIRST_BIT
+                csum[i] = 0;
+            }
+            __syncthreads();
+        }
+        const uint32_t g0 = tile * VERIFY_TILE;
+        const uint32_t g1 = min(L, g0 + (uint32_t)VERIFY_TILE) - 1;
+        const int s0 = find_slot(lb, N, g0);
+        const bool one_slot = g1 < lb[s0 + 1];  // the usual case: the tile lies inside one slot
+        uint64_t now[VERIFY_ITEMS], then[VERIFY_ITEMS];
+        int label[VERIFY_ITEMS];
+        uint32_t u[VERIFY_ITEMS];
+#pragma unroll
+        for (int j = 0; j < VERIFY_ITEMS; j++) {
+            const uint32_t gi = g0 + j * 256 + threadIdx.x;
+            now[j] = then[j] = 0;
+            label[j] = 0;
+            u[j] = 0;
+            if (gi <= g1) {
+                const int sl = one_slot ? s0 : find_slot(lb, N, gi);
+                const SlotDesc& d = descs[sl];
+                now[j] = (uint64_t)d.values[gi - lb[sl]];
+                then[j] = vals_copy[gi];
+                if (CLICKS) {
+                    label[j] = (int)d.labels[gi - lb[sl]];
+                    u[j] = u_of_gi[gi] & ~FIRST_BIT;
+                }
+                if (gi < n_members) {  // the member lists of the groups with several records fill the top of the array
+                    const uint32_t place = L - n_members + gi;
+                    const float* gp = nullptr;
+                    int sh, ck;
+                    gaddr[place] = src_record(src, list[place], gp, sh, ck) ? gp : nullptr;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VERIFY_ITEMS; j++) {
+            bad |= now[j] != then[j];
+            if (CLICKS && label[j] != 0) {
+                uint32_t h = (u[j] * 2654435761u) >> (32 - CLICK_BITS);
+                bool placed = false;
+                for (int tries = 0; tries < CLICK_TRIES && !placed; tries++) {
+                    uint32_t old = ckey[h];
+                    if (old == 0xFFFFFFFFu) old = atomicCAS(&ckey[h], 0xFFFFFFFFu, u[j]);
+                    if (old == 0xFFFFFFFFu || old == u[j]) {
+                        atomicAdd(&csum[h], label[j]);
+                        placed = true;
+                    }
+                    h = (h + 1) & (CLICK_TABLE - 1);
+                }
+                if (!placed) atomicAdd(&list[where_u[u[j]].x].click, label[j]);
+            }
+        }
+        if (CLICKS) {
+            __syncthreads();
+            constexpr int PER = CLICK_TABLE / 256;
+            uint32_t place[PER];
+            int sum[PER];
+#pragma unroll
+            for (int j = 0; j < PER; j++) {
+                const int e = j * 256 + threadIdx.x;
+                sum[j] = csum[e];
+                place[j] = sum[j] != 0 ? where_u[ckey[e]].x : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < PER; j++)
+                if (sum[j] != 0) atomicAdd(&list[place[j]].click, sum[j]);
+            __syncthreads();
         }
     }
     if (bad) {

@@ -1386,7 +1386,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // On a plan with show counts the verify pass also sums the clicks; they start at zero
         // after the pull, a further push on the same plan clears them first.
         const bool clicks = t->plan_has_show && with_click;
-        const int vblocks = launch_grid(L, 256, GRID_CAP * 2);
+        const int vblocks = launch_grid((int64_t)(L + VERIFY_TILE - 1) / VERIFY_TILE, 1, GRID_CAP * 2);
         // the outcome comes back through pinned host memory, written by the verify kernel itself
         t->hpush->st.mismatch = 0;
         uint32_t* host_mismatch = &t->hpush->st.mismatch;

@@ -114,6 +114,15 @@ def make_batch(cfg, batch_index=0, scale=1.0):
     return out
 
 
+CLICK_RATE = 0.2  # share of lookups whose feature label is 1 (the label of their example)
+
+
+def make_labels(values, batch_index=0, rate=CLICK_RATE):
+    """Per-slot int64 feature labels (0 / 1) for the lookups of one batch."""
+    rng = np.random.default_rng(2_000_003 + batch_index)
+    return [(rng.random(len(v)) < rate).astype(np.int64) for v in values]
+
+
 def make_grads(counts, dim, sigma, seed=0):
     """Per-slot float32 [U_s, dim] gradients ~ N(0, sigma)."""
     rng = np.random.default_rng(1_000_003 + seed)
