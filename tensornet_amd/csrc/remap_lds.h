@@ -3,8 +3,8 @@
 //
 // A global hash table costs one or two random 64-byte granules and up to two
 // device atomics per lookup.  Here the lookups of every slot are first
-// partitioned by a hash of the sign into buckets of ~1536 lookups (an LDS
-// histogram and an LDS cursor per 4096-lookup tile: the only global atomics
+// partitioned by a hash of the sign into buckets of 768 to 1536 lookups (an LDS
+// histogram and an LDS cursor per 2048-lookup tile: the only global atomics
 // are one per tile and bucket); then one workgroup per bucket builds the
 // bucket's hash table in LDS -- sign, smallest position, number of
 // occurrences -- and writes for every lookup the position of its sign's first
@@ -14,21 +14,22 @@
 //
 //   k_lds_hist     bucket sizes (+ copy of the signs for the plan)
 //   k_lds_offsets  exclusive scan of the bucket sizes (one workgroup)
-//   k_lds_scatter  {sign, position} records grouped by bucket
+//   k_lds_scatter  {sign, position, slot} records grouped by bucket
 //   k_lds_dedup    per bucket: LDS hash table -> first_of[position], occurrence counts
 //   k_lds_flags    first-occurrence flags per tile (coalesced: first_of[gi] == gi)
-//   k_scan_tiles   (shared with the global-table path)
-//   k_lds_assign   ranks, distinct lists, show counts
+//   k_lds_assign   ranks, distinct lists, show counts; the tiles' offsets come from a sum over the
+//                  counts of the tiles before (k_scan_tiles, shared with the global-table path,
+//                  only when there are too many tiles for that)
 //   k_lds_mapped   mapped ids and the per-lookup distinct index
 //
 // With at most 128 slots the groups of equal signs over all slots come out of
 // LDS too: k_lds_dedup hands every distinct (slot, sign) record -- sign, first
-// position, occurrences -- to a second level of buckets chosen by the sign's
+// position, occurrences, slot -- to a second level of buckets chosen by the sign's
 // hash alone (fixed room per bucket, one global atomic per touched bucket), and
 // one workgroup per such bucket (k_group_count) finds the signs shared between
-// slots with an LDS table of slot masks; a scan over the buckets' counts
-// (k_group_offsets) then numbers the groups, and k_group_emit writes their
-// member lists.
+// slots with an LDS table of slot masks; k_group_emit numbers the groups from the
+// counts of the buckets before its own (summed by itself, or by the scan
+// k_group_offsets when there are too many buckets) and writes their member lists.
 //
 // If an LDS table ever overflows (more distinct signs in a bucket than it has
 // room for) DEV_ERR_REMAP_OVERFLOW is raised; every index written stays in
