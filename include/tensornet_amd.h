@@ -203,8 +203,13 @@ int tn_sparse_table_export_rows(uint32_t handle, const uint64_t* signs, int64_t 
  * the distinct signs of slot s (sparse_table_ops.cc:122-131) and copies the
  * pulled row of the j-th distinct sign into vars[s][j, :]; rows >= U_s are
  * left untouched.  U_s >= var_rows[s] is TN_ERR_VAR_CAPACITY.
- * The call returns after the stream work has completed (the reference op
- * blocks on a semaphore, sparse_table_ops.cc:236).
+ * The call returns when the per-slot counts and the errors of the call are
+ * known on the host (the reference op blocks on a semaphore until the pulled
+ * rows are there, sparse_table_ops.cc:236).  The outputs are complete in
+ * stream order, as the outputs of a GPU op kernel are: on large batches the
+ * copy of the pulled rows into vars may still be running on `stream` when the
+ * call returns; work enqueued on `stream` afterwards sees them, a host that
+ * reads them synchronises the stream (or calls tn_sparse_table_sync) first.
  */
 int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
                             float* const* vars, const int64_t* var_rows, int var_dim,

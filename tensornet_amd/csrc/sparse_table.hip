@@ -63,6 +63,11 @@ struct SparseTable {
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     hipEvent_t fork_ev = nullptr, join_ev = nullptr, join2_ev = nullptr;
+    // A pull whose status is final before its last kernel (the gather) publishes it on the side stream
+    // meanwhile and returns when it is there: ready_ev = the status can be published, pub_ev = it is on
+    // the host, tail_ev = the gather is done (what a call on another stream has to wait for).
+    hipEvent_t ready_ev = nullptr, pub_ev = nullptr, tail_ev = nullptr;
+    bool tail_recorded = false;
     bool plan_clicks_dirty = false;  // a push has added clicks to the member lists of the current plan
     // Distinct records per lookup seen by the recent pulls (1 = every lookup distinct, the safe start):
     // sizes the number of second-level buckets, whose room is fixed.  A batch with more distinct
@@ -192,6 +197,9 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipEventCreateWithFlags(&t->fork_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->join_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->join2_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->ready_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->pub_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->tail_ev, hipEventDisableTiming));
     TN_HIP(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));  // default priority
     TN_HIP(hipStreamCreateWithFlags(&t->side2, hipStreamNonBlocking));
     return TN_OK;
@@ -199,6 +207,8 @@ int ensure_side_buffers(SparseTable* t) {
 
 int ensure_allocated(SparseTable* t, hipStream_t st) {
     TN_TRY(ensure_side_buffers(t));
+    // work of the last pull that its caller did not wait for was queued on that call's stream
+    if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
     if (t->allocated) return TN_OK;
     uint64_t cap = DEFAULT_SLOTS;
     if (t->reserve_keys) cap = (uint64_t)((double)t->reserve_keys / MAX_LOAD) + 64;
@@ -1222,8 +1232,13 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         const Store& s = t->store;
         DevStatus* ds = t->dplan;
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, true, use_lds, st));
-        // the grouping through LDS leaves the row of every distinct record in where_u itself
+        // The grouping through LDS leaves the row of every distinct record in where_u itself, and the
+        // call's status (counts, new rows, errors) is final before the gather starts: it is published
+        // on the side stream beside the gather, and the call returns when the host has it.  The
+        // variables are complete in stream order, as the outputs of any call that takes a stream.
+        const bool early = use_lds && N <= GRP_SLOTS && !t->async_pull;
         const uint32_t* rows_of_groups = (use_lds && N <= GRP_SLOTS) ? nullptr : p.grp_row;
+        if (early) TN_HIP(hipEventRecord(t->ready_ev, st));
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
                       ds, rows_of_groups, p.where_u, p.ubase, N, p.descs);
@@ -1231,8 +1246,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
                       rows_of_groups, p.where_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
-        TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
+        if (early) {
+            TN_HIP(hipEventRecord(t->tail_ev, st));
+            t->tail_recorded = true;
+            TN_HIP(hipStreamWaitEvent(t->side, t->ready_ev, 0));
+        }
+        TN_LAUNCH(k_publish, dim3(1), dim3(256), early ? t->side : st, ds, p.ubase, (uint32_t)(N + 1),
                   reinterpret_cast<uint32_t*>(t->hpull), s.count);
+        if (early) TN_HIP(hipEventRecord(t->pub_ev, t->side));
         t->pull_pending = true;
         t->pull_slots = N;
         t->pull_lookups = (uint64_t)L;
@@ -1245,7 +1266,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         t->plan_lens.assign(value_lens, value_lens + N);
         t->plan_epoch = t->epoch;
         if (t->async_pull) return TN_OK;
-        TN_HIP(hipStreamSynchronize(st));
+        if (early)
+            TN_HIP(hipEventSynchronize(t->pub_ev));
+        else
+            TN_HIP(hipStreamSynchronize(st));
         if (use_lds && (t->hpull->st.err & DEV_ERR_REMAP_OVERFLOW)) {
             // rows the failed attempt inserted belong to signs of this batch; keep them counted
             t->hpull->st.err &= ~DEV_ERR_REMAP_OVERFLOW;
@@ -1255,6 +1279,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             t->latched_msg.clear();
             use_lds = false;
             continue;
+        }
+        if (early) {
+            harvest(t);
+            return take_latched(t);
         }
         return sync_table(t, st);
     }

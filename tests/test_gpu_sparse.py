@@ -822,3 +822,43 @@ def test_batch_beyond_the_sizes_the_fused_scans_cover(tn, oracle):
     cum = torch.cumsum(0.01 * g / torch.sqrt(0.1 + steps * g * g), 0)
     expect = w0.double() - cum[(k - 1).long()][:, None]
     np.testing.assert_allclose(w2.cpu().numpy(), expect.cpu().numpy(), rtol=RTOL, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
+    """A large pull returns when its counts and errors are on the host, while the copy of the
+    pulled rows may still be running on its stream.  A push and a second pull issued at once on
+    ANOTHER stream (which reuse the table's scratch memory) must wait for it by themselves."""
+    D = 16
+    rng = np.random.default_rng(77)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 60001, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool.view(np.uint64))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for step in range(3):
+        values = [pool[rng.integers(0, 60000, int(rng.integers(3000, 6000)))] for _ in range(16)]
+        rows = [len(v) + 1 for v in values]
+        cvars = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
+        rc, cmapped, counts = pair.o.pull_op(values, cvars)
+        assert rc == 0
+        grads = synth.make_grads(counts, D, 0.01, seed=step)
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        assert pair.o.push_op(values, grads, labels)[0] == 0
+        cvars2 = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
+        assert pair.o.pull_op(values, cvars2)[0] == 0
+        gvalues, ggrads, glabels = [dev(v) for v in values], [dev(g) for g in grads], [dev(l) for l in labels]
+        gvars = [torch.full((r, pair.wf), -7.0, device="cuda") for r in rows]
+        gvars2 = [torch.full((r, pair.wf), -7.0, device="cuda") for r in rows]
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s1):
+            gmapped = tn.ops.sparse_table_pull(gvars, gvalues, pair.h)
+        with torch.cuda.stream(s2):  # no synchronisation in between
+            tn.ops.sparse_table_push(gvalues, ggrads, glabels, pair.h)
+            gmapped2 = tn.ops.sparse_table_pull(gvars2, gvalues, pair.h)
+        torch.cuda.synchronize()
+        for s in range(len(values)):
+            assert np.array_equal(gmapped[s].cpu().numpy(), cmapped[s])
+            assert np.array_equal(gmapped2[s].cpu().numpy(), cmapped[s])
+            np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
+            np.testing.assert_allclose(gvars2[s].cpu().numpy(), cvars2[s], rtol=RTOL, atol=ATOL)
