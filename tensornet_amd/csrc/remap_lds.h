@@ -421,7 +421,9 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_assign(
     uint32_t* __restrict__ wordpre, uint32_t* __restrict__ ubase, uint64_t* __restrict__ uniq_sign,
     uint32_t* __restrict__ uniq_slot, uint32_t* __restrict__ ushow, const uint32_t* __restrict__ tilesum,
     DevStatus* status) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    // lb[N + 1], sized by the launch: a fixed array for the largest slot count would take 16 KB of LDS per
+    // workgroup away from the grouping kernel that runs beside this one
+    extern __shared__ uint32_t lb[];
     __shared__ uint32_t red[4];
     load_lbase(lb, lbase, N);
     const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
@@ -498,7 +500,7 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
                                                     const uint8_t* __restrict__ flag8,
                                                     const uint32_t* __restrict__ wordpre,
                                                     uint32_t* __restrict__ u_of_gi) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    extern __shared__ uint32_t lb[];  // lb[N + 1], sized by the launch (see k_lds_assign)
     load_lbase(lb, lbase, N);
     // four consecutive lookups per thread: one 16-byte load and store, one slot search
     const uint32_t stride = gridDim.x * blockDim.x;

@@ -1237,7 +1237,7 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                                                        const uint2* __restrict__ where_u, Member* list,
                                                        uint32_t* host_mismatch, PushSrc src,
                                                        const float** __restrict__ gaddr) {
-    __shared__ uint32_t lb[MAX_SLOTS + 1];
+    extern __shared__ uint32_t lb[];  // lb[N + 1], sized by the launch: more tiles in flight per CU than with a fixed array
     __shared__ uint32_t ckey[CLICKS ? CLICK_TABLE : 1];
     __shared__ int csum[CLICKS ? CLICK_TABLE : 1];
     load_lbase(lb, lbase, N);

@@ -673,14 +673,15 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         const uint32_t* own_sums = w.ntiles <= SELF_SCAN_TILES ? w.tilesum : nullptr;
         if (!own_sums)
             TN_LAUNCH(k_scan_tiles, dim3(1), dim3(1024), st, w.tilesum, w.tileoff, w.ntiles, p.lbase, p.ubase, N, L, ds);
+        const size_t lb_lds = ((size_t)N + 1) * sizeof(uint32_t);
         if (lds_groups)
-            TN_LAUNCH((k_lds_assign<false>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
+            TN_LAUNCH_LDS((k_lds_assign<false>), dim3(w.ntiles), dim3(REMAP_THREADS), lb_lds, st, p.descs, p.lbase, N, L,
+                          w.flag8, w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
         else
-            TN_LAUNCH((k_lds_assign<true>), dim3(w.ntiles), dim3(REMAP_THREADS), st, p.descs, p.lbase, N, L, w.flag8,
-                      w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
-        TN_LAUNCH(k_lds_mapped, dim3(lblocks), dim3(256), st, p.descs, p.lbase, p.ubase, N, L, w.first_of, w.flag8, w.wordpre,
-                  p.u_of_gi);
+            TN_LAUNCH_LDS((k_lds_assign<true>), dim3(w.ntiles), dim3(REMAP_THREADS), lb_lds, st, p.descs, p.lbase, N, L,
+                          w.flag8, w.tileoff, w.cnt_at, w.wordpre, p.ubase, p.uniq_sign, p.uniq_slot, p.ushow, own_sums, ds);
+        TN_LAUNCH_LDS(k_lds_mapped, dim3(lblocks), dim3(256), lb_lds, st, p.descs, p.lbase, p.ubase, N, L, w.first_of,
+                      w.flag8, w.wordpre, p.u_of_gi);
     } else {
         TN_LAUNCH(k_fill_ff, dim3(launch_grid((int64_t)w.dt_entries, 256, GRID_CAP * 2)), dim3(256), st,
                   reinterpret_cast<uint4*>(w.dt), w.dt_entries);
@@ -1415,6 +1416,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // after the pull, a further push on the same plan clears them first.
         const bool clicks = t->plan_has_show && with_click;
         const int vblocks = launch_grid((int64_t)(L + VERIFY_TILE - 1) / VERIFY_TILE, 1, GRID_CAP * 2);
+        const size_t vlds = ((size_t)N + 1) * sizeof(uint32_t);
         // the outcome comes back through pinned host memory, written by the verify kernel itself
         t->hpush->st.mismatch = 0;
         uint32_t* host_mismatch = &t->hpush->st.mismatch;
@@ -1427,11 +1429,11 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
-            TN_LAUNCH((k_verify_values<true>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.vals_copy,
-                      ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
+            TN_LAUNCH_LDS((k_verify_values<true>), dim3(vblocks), dim3(256), vlds, st, p.descs, p.lbase, N, (uint32_t)L,
+                          p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         } else {
-            TN_LAUNCH((k_verify_values<false>), dim3(vblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L,
-                      p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
+            TN_LAUNCH_LDS((k_verify_values<false>), dim3(vblocks), dim3(256), vlds, st, p.descs, p.lbase, N, (uint32_t)L,
+                          p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         }
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // Counts and apply kernels are queued before the host knows the outcome: the counts only
