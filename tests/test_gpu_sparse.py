@@ -862,3 +862,27 @@ def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
             assert np.array_equal(gmapped2[s].cpu().numpy(), cmapped[s])
             np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
             np.testing.assert_allclose(gvars2[s].cpu().numpy(), cvars2[s], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("extra", [0, 1, 3, 4, 5, 7, 2047])
+def test_batch_sizes_around_the_tile_and_vector_boundaries(tn, oracle, extra):
+    """The ranking kernels take 4 or 8 lookups per thread with 16-byte accesses and handle the last,
+    incomplete group one by one: total sizes of every remainder, slot boundaries that are no
+    multiple of the vector widths."""
+    D = 8
+    rng = np.random.default_rng(900 + extra)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=200000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 20001, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool[:15000].view(np.uint64))
+    total = 16 * 2048 + extra
+    cuts = np.sort(rng.choice(np.arange(1, total), 6, replace=False))
+    lens = np.diff(np.concatenate([[0], cuts, [total]]))
+    lens = np.concatenate([lens[:3], [0], lens[3:]])  # an empty slot in the middle
+    values = [pool[rng.integers(0, 20000, int(n))] for n in lens]
+    assert sum(len(v) for v in values) == total
+    counts = check_pull(pair, values)
+    grads = synth.make_grads(counts, D, 0.01, seed=extra)
+    labels = [rng.integers(-1, 3, len(v)).astype(np.int64) for v in values]
+    pair.push_op(values, grads, labels)
+    assert pair.assert_rows_match(all_signs(values)) > 0.99
