@@ -479,6 +479,10 @@ def main():
             "ms_per_step": dsec * 1e3,
             "algorithmic_GBps": 28 * total / dsec / 1e9,  # read g,w,m,v ; write w,m,v
             "frac_of_hbm_peak": 28 * total / dsec / HBM_PEAK,
+            # with the new weights also written back into the op's variable (the pull half of the op),
+            # which is what FETCH_SIZE / WRITE_SIZE show for the kernel: 16 B read, 16 B written per parameter
+            "hbm_traffic_GBps": 32 * total / dsec / 1e9,
+            "traffic_frac_of_hbm_peak": 32 * total / dsec / HBM_PEAK,
         }
         del w, g
 
