@@ -20,6 +20,11 @@ constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:26
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
 constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 512-1024 are best)
+// Below this many lookups a call keeps all its kernels on the caller's stream.  The kernels of a smaller
+// batch are too short for the overlap on the side streams to win back what the events that fork and
+// join them cost the host (measured: 106 k lookups 0.22 -> 0.17 ms per pull + push, 2.1 M 0.33 -> 0.31 ms,
+// 5 M 0.67 -> 0.71 ms).
+constexpr size_t ONE_STREAM_LOOKUPS = 3u << 20;
 constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to which no scan kernel runs between its launches
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
 constexpr size_t LDS_MIN_LOOKUPS = 32768;  // smaller batches are launch-bound: the shorter global-table path wins
@@ -68,6 +73,7 @@ struct SparseTable {
     // the host, tail_ev = the gather is done (what a call on another stream has to wait for).
     hipEvent_t ready_ev = nullptr, pub_ev = nullptr, tail_ev = nullptr;
     bool tail_recorded = false;
+    bool one_stream = false;        // the running call is small: its kernels all go to the caller's stream
     bool plan_clicks_dirty = false;  // a push has added clicks to the member lists of the current plan
     // Distinct records per lookup seen by the recent pulls (1 = every lookup distinct, the safe start):
     // sizes the number of second-level buckets, whose room is fixed.  A batch with more distinct
@@ -655,18 +661,23 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             // the side stream beside the ranking of the first occurrences (LDS / latency bound
             // against streaming kernels) and joins before the member lists are written.
             const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
-            TN_HIP(hipEventRecord(t->fork_ev, st));
-            TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
-            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), t->side, w.nb2, w.cursor2, w.recs,
+            hipStream_t sd = t->one_stream ? st : t->side, sd2 = t->one_stream ? st : t->side2;
+            if (!t->one_stream) {
+                TN_HIP(hipEventRecord(t->fork_ev, st));
+                TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+            }
+            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), sd, w.nb2, w.cursor2, w.recs,
                       big_threshold(s), w.aux, w.bcounts);
-            if (!own_offsets) TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), t->side, w.bcounts, w.bbase, w.nb2, ds);
-            TN_HIP(hipEventRecord(t->join_ev, t->side));
-            // ... and so do the rows of the records' signs, on a stream of their own
-            TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
+            if (!own_offsets) TN_LAUNCH(k_group_offsets, dim3(1), dim3(1024), sd, w.bcounts, w.bbase, w.nb2, ds);
+            if (!t->one_stream) {
+                TN_HIP(hipEventRecord(t->join_ev, t->side));
+                // ... and so do the rows of the records' signs, on a stream of their own
+                TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
+            }
             // few workgroups: enough probes in flight for the memory system, most of every CU left to the grouping
-            TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), t->side2, w.nb2, w.cursor2, w.recs, w.rrow, s,
+            TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), sd2, w.nb2, w.cursor2, w.recs, w.rrow, s,
                       make_optdev(t), t->seed, ds);
-            TN_HIP(hipEventRecord(t->join2_ev, t->side2));
+            if (!t->one_stream) TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
         // up to SELF_SCAN_TILES tiles the ranking pass adds up the tile counts itself
@@ -697,8 +708,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
-        TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
-        TN_HIP(hipStreamWaitEvent(st, t->join2_ev, 0));
+        if (!t->one_stream) {
+            TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
+            TN_HIP(hipStreamWaitEvent(st, t->join2_ev, 0));
+        }
         TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
                   own_offsets ? nullptr : w.bbase, w.bcounts, w.flag8, w.wordpre, L, big_threshold(s),
                   p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds);
@@ -733,11 +746,13 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
         if (gaddr && !addr_ready)
             TN_LAUNCH(k_member_grads, dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, src, ds, p.list,
                       p.gaddr, ids_cap);
-        TN_HIP(hipEventRecord(t->fork_ev, st));
-        TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+        if (!t->one_stream) {
+            TN_HIP(hipEventRecord(t->fork_ev, st));
+            TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+        }
         const int gfloats = big_gbuf_floats(s.D);
         TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
-                      big_lds_bytes(s.D), t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
+                      big_lds_bytes(s.D), t->one_stream ? st : t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
                       p.list, gfloats, gaddr);
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
@@ -745,7 +760,7 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
         TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
                   o, src, ds, p.grp_row, p.list);                                                                 \
         TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256),    \
-                  with_big ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,    \
+                  with_big && !t->one_stream ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,    \
                   gaddr);                                                                                         \
     } while (0)
     switch (lpg) {
@@ -760,7 +775,7 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
                       p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);
     }
 #undef TN_LAUNCH_VEC
-    if (with_big) {
+    if (with_big && !t->one_stream) {
         TN_HIP(hipEventRecord(t->join_ev, t->side));
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
     }
@@ -1218,6 +1233,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             t->last_counts.assign(N, 0);
             return take_latched(t);
         }
+        t->one_stream = L < ONE_STREAM_LOOKUPS;
         TN_TRY(ensure_room(t, (uint64_t)L, st));
         Plan p{};
         Scratch w{};
@@ -1237,7 +1253,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         // call's status (counts, new rows, errors) is final before the gather starts: it is published
         // on the side stream beside the gather, and the call returns when the host has it.  The
         // variables are complete in stream order, as the outputs of any call that takes a stream.
-        const bool early = use_lds && N <= GRP_SLOTS && !t->async_pull;
+        const bool early = use_lds && N <= GRP_SLOTS && !t->async_pull && !t->one_stream;
         const uint32_t* rows_of_groups = (use_lds && N <= GRP_SLOTS) ? nullptr : p.grp_row;
         if (early) TN_HIP(hipEventRecord(t->ready_ev, st));
         if (vec)
@@ -1337,6 +1353,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         harvest(t);
     }
     if (L == 0) return TN_OK;
+    t->one_stream = L < ONE_STREAM_LOOKUPS;
     Plan p{};
     Scratch w{};
     // Same batch as the last pull?  Necessary conditions on the host, the signs
