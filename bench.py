@@ -32,17 +32,17 @@ def log(msg):
 # WRITE_SIZE x 1.0: the factors that make the counters reproduce the known traffic of the dense Adam stream).
 # Counters cannot be read from inside this script; the figures are refreshed together with that summary.
 MEASURED_TRAFFIC = {
-    "k_show_decay": 85646300000,
+    "k_show_decay": 85646700000,
     "k_reduce_pooled": 393500000,
     "k_gather_vars": 372900000,
     "k_combine_fwd": 356200000,
     "k_apply_single": 341500000,
     "k_reduce_long": 236600000,
-    "k_lds_dedup": 226900000,
-    "k_verify_values": 207000000,
-    "k_group_emit": 204300000,
+    "k_lds_dedup": 226800000,
+    "k_verify_values": 207500000,
+    "k_group_emit": 204200000,
     "k_probe_recs": 191000000,
-    "k_lds_scatter": 165300000,
+    "k_lds_scatter": 165500000,
     "k_lookup_keys": 123300000,
     "k_apply_vec": 121300000,
     "k_lds_hist": 100900000,
