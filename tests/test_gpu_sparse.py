@@ -831,13 +831,16 @@ def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
     ANOTHER stream (which reuse the table's scratch memory) must wait for it by themselves."""
     D = 16
     rng = np.random.default_rng(77)
-    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000, zero_init=True)
-    pool = synth.splitmix64(np.arange(1, 60001, dtype=np.uint64)).view(np.int64)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=1200000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 600001, dtype=np.uint64)).view(np.int64)
     pair.populate(pool.view(np.uint64))
     s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
     torch.cuda.synchronize()
-    for step in range(3):
-        values = [pool[rng.integers(0, 60000, int(rng.integers(3000, 6000)))] for _ in range(16)]
+    for step in range(2):
+        # step 0: a batch large enough for the side streams (more than 3 M lookups), step 1: a small one
+        per_slot = (200000, 230000) if step == 0 else (3000, 6000)
+        values = [pool[rng.integers(0, 600000, int(rng.integers(*per_slot)))] for _ in range(16)]
+        assert (sum(len(v) for v in values) > 3 << 20) == (step == 0)
         rows = [len(v) + 1 for v in values]
         cvars = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
         rc, cmapped, counts = pair.o.pull_op(values, cvars)
