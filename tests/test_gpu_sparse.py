@@ -889,3 +889,34 @@ def test_batch_sizes_around_the_tile_and_vector_boundaries(tn, oracle, extra):
     labels = [rng.integers(-1, 3, len(v)).astype(np.int64) for v in values]
     pair.push_op(values, grads, labels)
     assert pair.assert_rows_match(all_signs(values)) > 0.99
+
+
+@pytest.mark.gpu
+def test_variable_too_small_is_reported_on_a_large_batch(tn, oracle):
+    """More than 3 M lookups (the pull returns while its last kernel still runs): a variable with
+    fewer rows than its slot has distinct signs is still TN_ERR_VAR_CAPACITY (sparse_table_ops.cc:136),
+    nothing is written beyond its rows, and the table serves the next call."""
+    D = 16
+    opt = tn.core.AdaGrad(learning_rate=0.01, initial_g2sum=0.1)
+    h = tn.core.create_sparse_table(opt, "", D, False, "")
+    tn.core.reserve_sparse_table(h, 10 ** 6)
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    gvalues = [synth.splitmix64_torch(torch.randint(1, 500000, (210000,), generator=gen, device="cuda"))
+               for _ in range(16)]
+    assert sum(len(v) for v in gvalues) > 3 << 20
+    rows = [len(v) + 1 for v in gvalues]
+    small = 1000
+    guard = torch.full((small + 64, D), 9.0, device="cuda")  # the variable is its first `small` rows
+    gvars = [torch.full((r, D), 9.0, device="cuda") for r in rows]
+    gvars[3] = guard[:small]
+    with pytest.raises(tn.TensorNetError) as e:
+        tn.ops.sparse_table_pull(gvars, gvalues, h)
+    assert e.value.code == 4
+    torch.cuda.synchronize()
+    assert bool((guard[small:] == 9.0).all())
+    gvars[3] = torch.full((rows[3], D), 9.0, device="cuda")
+    mapped = tn.ops.sparse_table_pull(gvars, gvalues, h)
+    counts = tn.ops.sparse_table_last_unique_counts(h, 16)
+    torch.cuda.synchronize()
+    for s in (0, 3, 15):
+        assert counts[s] == torch.unique(gvalues[s]).numel() == int(mapped[s].max()) + 1
