@@ -484,6 +484,26 @@ def main():
             "hbm_traffic_GBps": 32 * total / dsec / 1e9,
             "traffic_frac_of_hbm_peak": 32 * total / dsec / HBM_PEAK,
         }
+        # the same array under dense AdaGrad: g, w, d2sum, g2sum, m read; w, d2sum, g2sum, m written (+ the variable)
+        gh = tn.core.create_dense_table(tn.core.AdaGrad(learning_rate=1e-3, initial_g2sum=0.1))
+        tn.ops.dense_table_init([w], gh)
+        for _ in range(3):
+            tn.ops.dense_table_push_pull([w], [g], 1e-3, gh)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(20):
+            tn.ops.dense_table_push_pull([w], [g], 1e-3, gh)
+        e1.record()
+        torch.cuda.synchronize()
+        gsec = e0.elapsed_time(e1) / 20 * 1e-3
+        out["dense_adagrad"] = {
+            "params": total,
+            "ms_per_step": gsec * 1e3,
+            "algorithmic_GBps": 36 * total / gsec / 1e9,
+            "frac_of_hbm_peak": 36 * total / gsec / HBM_PEAK,
+            "hbm_traffic_GBps": 40 * total / gsec / 1e9,
+            "traffic_frac_of_hbm_peak": 40 * total / gsec / HBM_PEAK,
+        }
         del w, g
 
     if not args.no_cpu:

@@ -102,6 +102,27 @@ __global__ __launch_bounds__(256) void k_dense_adam_s(const float* __restrict__ 
     }
 }
 
+// The same for AdaGrad (ada_grad_kernel.cc:25-48): five arrays in, four (five with the variable) out.
+__global__ __launch_bounds__(256) void k_dense_adagrad_v4(const float4* __restrict__ g, float4* __restrict__ w,
+                                                          float4* __restrict__ d2, float4* __restrict__ g2,
+                                                          float4* __restrict__ m, float4* __restrict__ out, int64_t n4,
+                                                          AdaGradArgs a) {
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+        float4 gg = stream_load(&g[i]);
+        float4 ww = stream_load(&w[i]), dd = stream_load(&d2[i]), ss = stream_load(&g2[i]), mm = stream_load(&m[i]);
+        adagrad_elem(gg.x, ww.x, dd.x, ss.x, mm.x, a);
+        adagrad_elem(gg.y, ww.y, dd.y, ss.y, mm.y, a);
+        adagrad_elem(gg.z, ww.z, dd.z, ss.z, mm.z, a);
+        adagrad_elem(gg.w, ww.w, dd.w, ss.w, mm.w, a);
+        stream_store(&w[i], ww);
+        stream_store(&d2[i], dd);
+        stream_store(&g2[i], ss);
+        stream_store(&m[i], mm);
+        if (out) stream_store(&out[i], ww);
+    }
+}
+
 __global__ __launch_bounds__(256) void k_dense_adagrad_s(const float* __restrict__ g, float* __restrict__ w,
                                                          float* __restrict__ d2, float* __restrict__ g2,
                                                          float* __restrict__ m, float* __restrict__ out, int64_t n,
@@ -337,8 +358,17 @@ int tn_dense_table_push_pull(uint32_t handle, int N, float* const* vars, const f
                 TN_LAUNCH(k_dense_adam_s, dim3(blocks), dim3(256), st, g + done, t->w + off + done, t->s0 + off + done, t->s1 + off + done, out ? out + done : nullptr, n - done, aa);
             }
         } else {
-            int blocks = launch_grid(n, 256, 1 << 20);
-            TN_LAUNCH(k_dense_adagrad_s, dim3(blocks), dim3(256), st, g, t->w + off, t->s0 + off, t->s1 + off, t->s2 + off, out, n, ga);
+            bool vec = (off % 4 == 0) && aligned16(g) && (!out || aligned16(out));
+            int64_t n4 = vec ? n / 4 : 0;
+            if (n4 > 0) {
+                int blocks = launch_grid(n4, 256, 1 << 20);
+                TN_LAUNCH(k_dense_adagrad_v4, dim3(blocks), dim3(256), st, (const float4*)g, (float4*)(t->w + off), (float4*)(t->s0 + off), (float4*)(t->s1 + off), (float4*)(t->s2 + off), (float4*)out, n4, ga);
+            }
+            int64_t done = n4 * 4;
+            if (done < n) {
+                int blocks = launch_grid(n - done, 256, 1 << 20);
+                TN_LAUNCH(k_dense_adagrad_s, dim3(blocks), dim3(256), st, g + done, t->w + off + done, t->s0 + off + done, t->s1 + off + done, t->s2 + off + done, out ? out + done : nullptr, n - done, ga);
+            }
         }
     }
     TN_HIP(hipGetLastError());

@@ -44,21 +44,24 @@ def test_dense_adam_push_pull(tn, oracle, sizes):
     assert same > 0.99
 
 
-def test_dense_adagrad_push_pull(tn, oracle):
-    total = 5000
+@pytest.mark.parametrize("sizes", [[5000], [7, 1, 8], [1000, 24, 4099, 3, 77]])
+def test_dense_adagrad_push_pull(tn, oracle, sizes):
+    """Aligned bodies go through the 16-byte kernel, odd offsets and tails through the scalar one."""
+    total = sum(sizes)
     rng = np.random.default_rng(4)
     hp = dict(initial_g2sum=0.5, epsilon=1e-3, grad_decay_rate=0.9, mom_decay_rate=0.5)
     h = tn.core.create_dense_table(tn.core.AdaGrad(**hp))
     d = oracle.Dense(oracle.ADAGRAD, total, **hp)
     w0 = rng.uniform(-1, 1, total).astype(np.float32)
     d.set_weight(w0)
-    var = dev(w0)
-    tn.ops.dense_table_init([var], h)
+    vars_ = [dev(w0[a:b]) for a, b in split(total, sizes)]
+    tn.ops.dense_table_init(vars_, h)
     for _ in range(4):
         g = rng.standard_normal(total).astype(np.float32)
         d.apply(g, 0.1)
-        tn.ops.dense_table_push_pull([var], [dev(g)], 0.1, h)
-    np.testing.assert_allclose(var.cpu().numpy(), d.get_weight(), rtol=RTOL, atol=ATOL)
+        tn.ops.dense_table_push_pull(vars_, [dev(g[a:b]) for a, b in split(total, sizes)], 0.1, h)
+    np.testing.assert_allclose(torch.cat(vars_).cpu().numpy(), d.get_weight(), rtol=RTOL, atol=ATOL)
+    assert torch.equal(tn.ops.dense_table_get_weight(h), torch.cat(vars_))
 
 
 def test_dense_errors(tn):
