@@ -199,23 +199,11 @@ def main():
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
     ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
-    ap.add_argument("--ceilings", action="store_true",
-                    help="first run tensornet_amd/ubench_random (random-access rates of the device, 64 GiB "
-                         "table) and carry its figures in the line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
               "(every box has one GPU, nothing here uses collectives)" % args.gpus, file=sys.stderr)
         sys.exit(2)
-
-    ceilings = None
-    if args.ceilings:
-        # a child process, before this one touches the GPU: it takes a table-sized allocation of its own
-        import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tensornet_amd", "ubench_random")
-        ub_text = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=300).stdout
-        log(ub_text)
-        ceilings = json.loads(ub_text.strip().split("\n")[-1])
 
     import numpy as np
     import torch
@@ -371,8 +359,6 @@ def main():
         "side_stream_kernels": [k for k in per_step if k.startswith(SIDE_STREAM_KERNELS)],
         "batch_shape": mean_shape,
     }
-    if ceilings is not None:
-        out["random_access_ceilings"] = ceilings
 
     # ---- side measurement: the combiner around the ops on the device ---------------
     # pull -> embedding_lookup_sparse (mean) -> push of the pooled gradients, same batches

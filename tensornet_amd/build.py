@@ -46,22 +46,6 @@ def build(verbose=True):
     return LIB
 
 
-UBENCH_SRC = os.path.join(CSRC, "ubench_random.hip")
-UBENCH_BIN = os.path.join(HERE, "ubench_random")
-
-
-def build_ubench(verbose=True):
-    """Builds the stand-alone program that measures the device's random-access ceilings
-    (bench.py --ceilings runs it)."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", UBENCH_SRC, "-o", UBENCH_BIN]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
-    return UBENCH_BIN
-
-
 def build_host_test(verbose=True):
     """Builds the C++ program that drives the library through include/tensornet_amd.hpp."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -76,5 +60,4 @@ def build_host_test(verbose=True):
 if __name__ == "__main__":
     build()
     build_host_test()
-    build_ubench()
     sys.exit(0)

@@ -147,6 +147,12 @@ def set_sparse_table_seed(table_handle, seed):
     _lib.check(_lib.load().tn_sparse_table_set_seed(table_handle, int(seed) & 0xFFFFFFFFFFFFFFFF))
 
 
+def set_sparse_table_async(table_handle, async_pull):
+    """With async_pull the pull op only enqueues its work (its counts and errors are collected by the next
+    call on the table, or by sparse_table_sync); by default it waits for them, as the reference's op does."""
+    _lib.check(_lib.load().tn_sparse_table_set_async(table_handle, 1 if async_pull else 0))
+
+
 def sparse_table_key_count(table_handle):
     n = C.c_uint64()
     _lib.check(_lib.load().tn_sparse_table_key_count(table_handle, C.byref(n)))

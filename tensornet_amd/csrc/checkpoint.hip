@@ -182,7 +182,10 @@ int save_table(uint32_t handle, const char* filepath, const char* mode) {
         } else {
             head = std::string("opt_name:") + opt_name(ti.kind) + "\ndim:" + std::to_string(ti.dim) + "\n";
         }
-        gzwrite(files[b], head.data(), (unsigned)head.size());
+        if (gzwrite(files[b], head.data(), (unsigned)head.size()) != (int)head.size()) {
+            close_all();
+            return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_save: write failed in " + path);
+        }
     }
     uint64_t cap = 0;
     int rc = tn_sparse_table_capacity(handle, &cap);
@@ -222,8 +225,15 @@ int save_table(uint32_t handle, const char* filepath, const char* mode) {
         for (int b = 0; b < kBlocks; b++)
             if (!ok[b]) rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_save: write failed in " + ti.dir);
     }
-    for (int b = 0; b < kBlocks && rc == TN_OK; b++) gzwrite(files[b], "\n", 1);  // the std::endl after the block
-    close_all();
+    for (int b = 0; b < kBlocks && rc == TN_OK; b++)  // the std::endl after the block
+        if (gzwrite(files[b], "\n", 1) != 1) rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_save: write failed in " + ti.dir);
+    // closing flushes what zlib still holds: a full disk shows here at the latest
+    for (gzFile& f : files)
+        if (f) {
+            if (gzclose(f) != Z_OK && rc == TN_OK)
+                rc = fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_save: closing a block file failed in " + ti.dir);
+            f = nullptr;
+        }
     return rc;
 }
 

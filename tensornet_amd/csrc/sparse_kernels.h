@@ -1129,6 +1129,9 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
                                                      const uint32_t* __restrict__ ubase, int N,
                                                      const SlotDesc* __restrict__ descs) {
     __shared__ uint32_t ub[MAX_SLOTS + 1];
+    // A remap whose LDS tables overflowed dropped records: their where_u entries were never written (the
+    // host repeats the call on the other path).  The flag is final before this kernel starts.
+    if (status->err & DEV_ERR_REMAP_OVERFLOW) return;
     load_lbase(ub, ubase, N);
     const int chunks = s.wdim / VEC;
     const int64_t total = (int64_t)status->n_unique * chunks;
@@ -1144,7 +1147,7 @@ __global__ __launch_bounds__(256) void k_gather_vars(Store s, DevStatus* status,
             if (c == 0) atomicOr(&status->err, DEV_ERR_VAR_CAPACITY);
             continue;
         }
-        if (row == NO_ROW) continue;
+        if (row > s.cap) continue;  // NO_ROW, or no row number at all: never address the table with it
         if (VEC == 4) {
             float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
             *reinterpret_cast<float4*>(d.var + r * s.wdim + c * 4) = v;

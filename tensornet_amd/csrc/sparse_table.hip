@@ -59,6 +59,7 @@ struct SparseTable {
     DevStatus* dplan = nullptr;     // device: status / counts of the op-level plan
     HostStatus* hpull = nullptr;    // pinned
     HostStatus* hpush = nullptr;    // pinned
+    unsigned long long* hcount = nullptr;  // pinned: the number of resident keys is read into it
     char* hstage = nullptr;         // pinned staging of slot descriptors
     size_t hstage_bytes = 0;
     hipEvent_t stage_ev = nullptr;  // staging buffer free again
@@ -151,6 +152,8 @@ bool interleaved(const Store& s) { return s.wstride != s.wlen; }
 
 int state_floats(const SparseTable* t) { return (t->opt->kind == OPT_ADAGRAD) ? 4 : 2 * t->dim + 2; }
 
+void free_store(Store& s);
+
 int alloc_store(const SparseTable* t, uint64_t cap, Store& s, hipStream_t st) {
     layout(t, s);
     if (cap < 64) cap = 64;
@@ -159,23 +162,35 @@ int alloc_store(const SparseTable* t, uint64_t cap, Store& s, hipStream_t st) {
     s.cap = cap;
     choose_strides(s, cap);
     const size_t rows = (size_t)cap + 1;
+    // whatever was allocated before a failure is released again: the caller keeps no half-built store
+    auto oom = [&](const char* what, hipError_t e) {
+        const std::string msg = std::string("hipMalloc ") + what + ": " + hipGetErrorString(e);
+        free_store(s);
+        return fail(TN_ERR_OUT_OF_MEMORY, msg);
+    };
     hipError_t e;
     e = hipMalloc((void**)&s.keys, rows * sizeof(uint64_t) + 64);
-    if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc keys: ") + hipGetErrorString(e));
+    if (e != hipSuccess) return oom("keys", e);
     e = hipMalloc((void**)&s.w, rows * s.wstride * sizeof(float));
-    if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc weights: ") + hipGetErrorString(e));
+    if (e != hipSuccess) return oom("weights", e);
     if (interleaved(s)) {
         s.st = s.w + s.wlen;
     } else {
         e = hipMalloc((void**)&s.st, rows * s.sstride * sizeof(float));
-        if (e != hipSuccess) return fail(TN_ERR_OUT_OF_MEMORY, std::string("hipMalloc state: ") + hipGetErrorString(e));
+        if (e != hipSuccess) return oom("state", e);
     }
     void* small = nullptr;
-    TN_HIP(hipMalloc(&small, 64));
+    e = hipMalloc(&small, 64);
+    if (e != hipSuccess) return oom("counters", e);
     s.count = (unsigned long long*)small;
     s.special = (uint32_t*)((char*)small + 8);
-    TN_HIP(hipMemsetAsync(small, 0, 64, st));
-    TN_HIP(hipMemsetAsync(s.keys, 0xFF, rows * sizeof(uint64_t), st));
+    e = hipMemsetAsync(small, 0, 64, st);
+    if (e == hipSuccess) e = hipMemsetAsync(s.keys, 0xFF, rows * sizeof(uint64_t), st);
+    if (e != hipSuccess) {
+        const std::string msg = std::string("hipMemsetAsync (new table): ") + hipGetErrorString(e);
+        free_store(s);
+        return fail(TN_ERR_HIP, msg);
+    }
     return TN_OK;
 }
 
@@ -196,6 +211,7 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipHostMalloc((void**)&t->hpush, sizeof(HostStatus), hipHostMallocDefault));
     std::memset(t->hpull, 0, sizeof(HostStatus));
     std::memset(t->hpush, 0, sizeof(HostStatus));
+    TN_HIP(hipHostMalloc((void**)&t->hcount, 64, hipHostMallocDefault));
     t->hstage_bytes = (size_t)MAX_SLOTS * sizeof(SlotDesc) + (MAX_SLOTS + 1) * sizeof(uint32_t);
     TN_HIP(hipHostMalloc((void**)&t->hstage, t->hstage_bytes, hipHostMallocDefault));
     TN_HIP(hipEventCreateWithFlags(&t->stage_ev, hipEventDisableTiming));
@@ -320,12 +336,13 @@ int grow_to(SparseTable* t, uint64_t cap, hipStream_t st) {
     return TN_OK;
 }
 
+// The number of resident keys, read on the stream `st` itself (a copy on the null stream would wait for,
+// and hold up, every blocking stream of the process: other tables' calls).
 int read_count(SparseTable* t, hipStream_t st, uint64_t* out) {
+    TN_HIP(hipMemcpyAsync(t->hcount, t->store.count, sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
     TN_HIP(hipStreamSynchronize(st));
-    unsigned long long cnt = 0;
-    TN_HIP(hipMemcpy(&cnt, t->store.count, sizeof(cnt), hipMemcpyDeviceToHost));
-    t->count_upper = cnt;
-    *out = cnt;
+    t->count_upper = *t->hcount;
+    *out = *t->hcount;
     return TN_OK;
 }
 
@@ -875,11 +892,14 @@ int tn_sparse_table_key_count(uint32_t handle, uint64_t* count) {
     std::lock_guard<std::mutex> lk(t->mu);
     *count = 0;
     if (!t->allocated) return TN_OK;
-    if (t->last_stream) TN_HIP(hipStreamSynchronize(t->last_stream));
-    TN_HIP(hipDeviceSynchronize());
-    unsigned long long cnt = 0;
-    TN_HIP(hipMemcpy(&cnt, t->store.count, sizeof(cnt), hipMemcpyDeviceToHost));
-    t->count_upper = cnt;
+    // Only this table's own work is waited for: the count is kept by kernels on the stream of the table's last
+    // call (a pull that publishes its status on the side stream has waited for that before it returned).
+    if (t->push_pending || t->pull_pending) {
+        TN_HIP(hipStreamSynchronize(t->last_stream));
+        harvest(t);
+    }
+    uint64_t cnt = 0;
+    TN_TRY(read_count(t, t->last_stream, &cnt));
     *count = cnt;
     return TN_OK;
 }
@@ -1347,11 +1367,13 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         if (pooled) descs[s].mapped = const_cast<int64_t*>(example_ids[s]);  // example index of every lookup
         vec = vec && aligned16(grads[s]);
     }
-    t->last_stream = st;
     if (t->push_pending || t->pull_pending) {
+        // a call pending on another stream (an asynchronous pull) builds the plan this push reads
+        if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
         TN_HIP(hipStreamSynchronize(st));
         harvest(t);
     }
+    t->last_stream = st;
     if (L == 0) return TN_OK;
     t->one_stream = L < ONE_STREAM_LOOKUPS;
     Plan p{};

@@ -202,6 +202,51 @@ def test_table_level_pull_push_with_repeated_records(tn, oracle):
         pair.assert_rows_match(base)
 
 
+def test_hand_computed_known_answers_on_the_device(tn, oracle):
+    """The exact known answers of tests/golden/optim_kat.json (hand-computed from the reference's update rules,
+    power-of-two operands, both Ftrl branches and the case that tells float abs from an integer abs) through
+    the device path: load the row, push one record, read the row back -- bit for bit."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "optim_kat.json")) as f:
+        kat = json.load(f)
+    sign = np.asarray([0x1234567890ABCDEF], dtype=np.uint64)
+
+    def i2f(i):
+        return float(np.asarray([i], dtype=np.int32).view(np.float32)[0])
+
+    def run(opt, dim, hyper, w0, st0, grad, show, click=0):
+        h = tn.core.create_sparse_table(getattr(tn.core, opt)(**hyper), "", dim, False, "")
+        tn.core.reserve_sparse_table(h, 64)
+        tn.ops.table_load_rows(h, dev(sign.view(np.int64)), dev(np.asarray([w0], np.float32)),
+                               dev(np.asarray([st0], np.float32)))
+        rec = tn.ops.make_sign_infos(dev(sign.view(np.int64)), dev(np.asarray([show], np.int64)),
+                                     dev(np.asarray([click], np.int64)))
+        tn.ops.table_push(h, rec, dev(np.asarray([grad], np.float32)))
+        tn.ops.sparse_table_sync(h)
+        w, st, found = tn.ops.table_export_rows(h, dev(sign.view(np.int64)))
+        assert int(found[0]) == 1
+        return w[0].cpu().numpy(), st[0].cpu().numpy()
+
+    for c in kat["adagrad"]:
+        w, st = run("AdaGrad", c["dim"], c["hyper"], c["w0"], c["state0"][:3] + [i2f(c["state0"][3])], c["grad"],
+                    c["show"], c["click"])
+        assert w.tolist() == c["w1"] and st[:3].tolist() == c["state1"][:3]
+        assert int(st[3:4].view(np.int32)[0]) == c["state1"][3]
+    for c in kat["adam"]:
+        D = c["dim"]
+        w, st = run("Adam", D, c["hyper"], c["w0"], c["m0"] + c["v0"] + [0.0, i2f(0)], c["grad"], c["show"])
+        assert w.tolist() == c["w1"] and st[:D].tolist() == c["m1"] and st[D:2 * D].tolist() == c["v1"]
+        assert int(st[2 * D + 1:2 * D + 2].view(np.int32)[0]) == c["delta_show1"]
+    for c in kat["ftrl"]:
+        D = c["dim"]
+        w, st = run("Ftrl", D, c["hyper"], c["w0"], c["z0"] + c["n0"] + [0.0, i2f(0)], c["grad"], c["show"])
+        assert w.tolist() == c["w1"], c["_why"]
+        assert st[:D].tolist() == c["z1"] and st[D:2 * D].tolist() == c["n1"]
+        assert int(st[2 * D + 1:2 * D + 2].view(np.int32)[0]) == c["delta_show1"]
+
+
 def test_errors_come_back_as_codes(tn, oracle):
     D = 8
     pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP)
@@ -679,6 +724,10 @@ def test_two_tables_driven_from_two_host_threads(tn, oracle):
                     tn.ops.sparse_table_push([dev(v) for v in values], [dev(g) for g in grads],
                                              [dev(l) for l in labels], pair.h)
                     tn.ops.sparse_table_sync(pair.h)
+                    # statistics of BOTH tables while the other thread drives its own: a key count waits
+                    # for its table's work only (a device-wide wait here would serialise the two threads)
+                    for other in pairs:
+                        assert 20000 <= tn.core.sparse_table_key_count(other.h) <= vocab
                     results[k].append(([m.cpu().numpy() for m in mapped], [v.cpu().numpy() for v in gvars], counts,
                                        grads))
         except Exception as e:  # surfaced in the main thread
@@ -865,6 +914,46 @@ def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
             assert np.array_equal(gmapped2[s].cpu().numpy(), cmapped[s])
             np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
             np.testing.assert_allclose(gvars2[s].cpu().numpy(), cvars2[s], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.gpu
+def test_push_on_another_stream_waits_for_an_asynchronous_pull(tn, oracle):
+    """With asynchronous pulls the op only enqueues its kernels.  A push of the same batch issued at once on
+    ANOTHER stream reads the plan those kernels are still building: it has to wait for the pull's stream by
+    itself (as a second pull does)."""
+    D = 16
+    rng = np.random.default_rng(78)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 200001, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool[:150000].view(np.uint64))
+    tn.core.set_sparse_table_async(pair.h, True)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    try:
+        for step in range(3):
+            values = [pool[rng.integers(0, 200000, int(rng.integers(20000, 40000)))] for _ in range(12)]
+            rows = [len(v) + 1 for v in values]
+            cvars = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
+            rc, cmapped, counts = pair.o.pull_op(values, cvars)
+            assert rc == 0
+            grads = synth.make_grads(counts, D, 0.01, seed=step)
+            labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+            assert pair.o.push_op(values, grads, labels)[0] == 0
+            gvalues, ggrads, glabels = [dev(v) for v in values], [dev(g) for g in grads], [dev(l) for l in labels]
+            gvars = [torch.full((r, pair.wf), -7.0, device="cuda") for r in rows]
+            torch.cuda.synchronize()
+            with torch.cuda.stream(s1):
+                gmapped = tn.ops.sparse_table_pull(gvars, gvalues, pair.h)
+            with torch.cuda.stream(s2):  # no synchronisation in between
+                tn.ops.sparse_table_push(gvalues, ggrads, glabels, pair.h)
+            tn.ops.sparse_table_sync(pair.h)
+            torch.cuda.synchronize()
+            assert tn.ops.sparse_table_last_unique_counts(pair.h, len(values)) == counts.tolist()
+            for s in range(len(values)):
+                assert np.array_equal(gmapped[s].cpu().numpy(), cmapped[s])
+                np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
+            assert pair.assert_rows_match(all_signs(values)) > 0.99
+    finally:
+        tn.core.set_sparse_table_async(pair.h, False)
 
 
 @pytest.mark.gpu
