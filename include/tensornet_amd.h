@@ -170,6 +170,21 @@ int tn_sparse_table_row_layout(uint32_t handle, int* weight_floats, int* state_f
 int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream);
 
 /*
+ * The same pull for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no hipMalloc / hipFree:
+ * the row numbers and the new-row list of the call live in a static device array of the library (8 MiB + 256 B,
+ * held by every GPU the library runs on until the process ends), so
+ *   - n is at most 1048576 signs per call (TN_ERR_UNSUPPORTED beyond that);
+ *   - the table's storage must already exist (any earlier call through another entry point creates it) and
+ *     must have room for n more signs without growing (TN_ERR_UNSUPPORTED / TN_ERR_TABLE_FULL otherwise:
+ *     size it with tn_sparse_table_reserve first);
+ *   - the current device must be the table's.
+ * Calls are serialised by a lock of the library and each waits for its own work before it returns, so calls
+ * from several host threads do not race on the array; results are those of tn_sparse_table_pull, bit for bit.
+ */
+int tn_sparse_table_pull_static(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream);
+
+/*
  * SparseTable::Push (core/ps/table/sparse_table.cc:68-83): apply n records
  * (device infos[n], device grads[n*dim]) in ARRAY ORDER; a sign occurring k
  * times gets k sequential optimizer Applies.  A sign that was never pulled is

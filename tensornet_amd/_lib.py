@@ -104,6 +104,7 @@ SIGNATURES = {
     "tn_sparse_table_capacity": (C.c_int, [C.c_uint32, C.POINTER(C.c_uint64)]),
     "tn_sparse_table_row_layout": (C.c_int, [C.c_uint32, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "tn_sparse_table_pull": (C.c_int, [C.c_uint32, _P, C.c_int64, C.c_int, _P, _P]),
+    "tn_sparse_table_pull_static": (C.c_int, [C.c_uint32, _P, C.c_int64, C.c_int, _P, _P]),
     "tn_sparse_table_push": (C.c_int, [C.c_uint32, _P, _P, C.c_int64, C.c_int, _P]),
     "tn_sparse_table_load_rows": (C.c_int, [C.c_uint32, _P, _P, _P, C.c_int64, _P]),
     "tn_sparse_table_export_rows": (C.c_int, [C.c_uint32, _P, C.c_int64, _P, _P, _P, _P]),

@@ -7,6 +7,15 @@
 #include <algorithm>
 #include <cstring>
 
+// Device memory of tn_sparse_table_pull_static, the one entry point that allocates nothing: the call's
+// status block, then the row number and the new-row list of every requested sign.  Every GPU the library
+// runs on holds its own copy until the process ends; host code reaches it through the address that
+// hipGetSymbolAddress returns for the current device (static_scratch below), never through this name.
+constexpr int64_t TN_STATIC_MAX_SIGNS = 1 << 20;
+constexpr size_t TN_STATIC_STATUS_BYTES = 256;
+constexpr size_t TN_STATIC_SCRATCH_BYTES = TN_STATIC_STATUS_BYTES + 2 * (size_t)TN_STATIC_MAX_SIGNS * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[TN_STATIC_SCRATCH_BYTES];
+
 namespace tn {
 
 // sort_pairs.hip
@@ -993,6 +1002,99 @@ int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int 
     t->pull_slots = 0;
     t->pending_rows.clear();
     return sync_table(t, st);
+}
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mu;  // one call at a time uses a GPU's scratch array
+unsigned char* g_static_ptr[STATIC_MAX_DEVICES] = {};
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+int static_scratch(int* device, unsigned char** out) {
+    int dev = 0;
+    TN_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES)
+        return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_pull_static: device number beyond " + std::to_string(STATIC_MAX_DEVICES));
+    if (!g_static_ptr[dev]) {
+        unsigned char* ptr = nullptr;
+        TN_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(TN_ERR_HIP, "tn_sparse_table_pull_static: no address for the scratch array");
+        g_static_ptr[dev] = ptr;
+    }
+    *device = dev;
+    *out = g_static_ptr[dev];
+    return TN_OK;
+}
+}  // namespace
+
+int tn_sparse_table_pull_static(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_pull_static: bad table handle " + std::to_string(handle));
+    if (n < 0 || (n > 0 && (!signs || !out)))
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_pull_static: NULL buffer");
+    if (n > TN_STATIC_MAX_SIGNS)
+        return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_pull_static: " + std::to_string(n) + " signs, at most " +
+                                            std::to_string(TN_STATIC_MAX_SIGNS) + " per call (use tn_sparse_table_pull)");
+    std::lock_guard<std::mutex> sk(g_static_mu);
+    std::lock_guard<std::mutex> lk(t->mu);
+    hipStream_t st = (hipStream_t)stream;
+    int dev = 0;
+    unsigned char* ptr = nullptr;
+    TN_TRY(static_scratch(&dev, &ptr));
+    if (!t->allocated)
+        return fail(TN_ERR_UNSUPPORTED, "tn_sparse_table_pull_static: the table has no storage yet (its first call through "
+                                        "another entry point allocates it); this entry point allocates nothing");
+    if (dev != t->device)
+        return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_pull_static: the table lives on device " +
+                                                 std::to_string(t->device) + ", the current device is " + std::to_string(dev));
+    // work of the last pull that its caller did not wait for was queued on that call's stream
+    if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
+    const int wdim = t->dim + (t->use_cvm ? 2 : 0);
+    if (dim != wdim)
+        return fail(TN_ERR_DIM_MISMATCH, "tn_sparse_table_pull_static: dim " + std::to_string(dim) +
+                                             " but table rows hold " + std::to_string(wdim));
+    if (t->push_pending || t->pull_pending) {
+        if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
+        TN_HIP(hipStreamSynchronize(st));
+        harvest(t);
+    }
+    t->last_stream = st;
+    if (n == 0) return sync_table(t, st);
+    const Store& s = t->store;
+    // every requested sign may be new; a table that would have to grow for them needs a new allocation
+    if ((double)(t->count_upper + (uint64_t)n) > MAX_LOAD * (double)s.cap) {
+        uint64_t cnt = 0;  // the bound may be loose: read the true count (pinned memory, no allocation)
+        TN_TRY(read_count(t, st, &cnt));
+        if ((double)(cnt + (uint64_t)n) > MAX_LOAD * (double)s.cap)
+            return fail(TN_ERR_TABLE_FULL, "tn_sparse_table_pull_static: the table would have to grow for " +
+                                               std::to_string(n) + " more signs, which needs an allocation "
+                                               "(tn_sparse_table_reserve beforehand, or tn_sparse_table_pull)");
+    }
+    t->count_upper += (uint64_t)n;
+    t->booked = (uint64_t)n;
+    DevStatus* ds = reinterpret_cast<DevStatus*>(ptr);
+    uint32_t* rows = reinterpret_cast<uint32_t*>(ptr + TN_STATIC_STATUS_BYTES);
+    uint32_t* newlist = rows + TN_STATIC_MAX_SIGNS;
+    const OptDev o = make_optdev(t);
+    const int blocks = launch_grid(n, 256, GRID_CAP * 2);
+    // the array keeps the last call's contents: the status block is cleared here, rows[0 .. n) and
+    // newlist[0 .. new rows) are written by this call's probe before anything reads them
+    TN_LAUNCH(k_reset_status, dim3(1), dim3(64), st, ds, (uint32_t)n, 0u);
+    TN_LAUNCH((k_probe<true>), dim3(blocks), dim3(256), st, s, signs, n, (const DevStatus*)nullptr, 0u, rows, newlist, ds,
+              (uint32_t)DEV_ERR_TABLE_FULL, o, t->seed);
+    TN_LAUNCH(k_init_rows, dim3(blocks), dim3(256), st, s, o, t->seed, signs, rows, newlist, ds);
+    TN_LAUNCH(k_finish_insert, dim3(1), dim3(64), st, s, ds);
+    if (wdim % 4 == 0 && s.wstride % 4 == 0 && aligned16(out))
+        TN_LAUNCH((k_gather_rows<4>), dim3(launch_grid(n * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s, rows, n, out);
+    else
+        TN_LAUNCH((k_gather_rows<1>), dim3(launch_grid(n * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, rows, n, out);
+    TN_HIP(hipGetLastError());
+    TN_HIP(hipMemcpyAsync(&t->hpull->st, ds, sizeof(DevStatus), hipMemcpyDeviceToHost, st));
+    t->hpull->ubase[0] = 0;
+    t->pull_pending = true;
+    t->pull_slots = 0;
+    t->pending_rows.clear();
+    return sync_table(t, st);  // the scratch array is free again when the lock is released
 }
 
 int tn_sparse_table_push(uint32_t handle, const tn_sign_info* infos, const float* grads, int64_t n, int dim,
