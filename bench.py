@@ -194,7 +194,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg3")
     ap.add_argument("--resident", type=int, default=None, help="resident keys (default: the config's)")
-    ap.add_argument("--batches", type=int, default=4, help="distinct pre-generated batches cycled through")
+    ap.add_argument("--profile-steps", type=int, default=8,
+                    help="further steps, on batches of their own, run with HIP events around every launch")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
     ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
@@ -228,20 +229,28 @@ def main():
     populate(tn, h, resident, dim)
 
     # ---- inputs, resident in HBM -------------------------------------------------
-    nb = max(1, args.batches)
-    host_batches = [synth.make_batch(cfg, b) for b in range(nb)]
-    batches = []
+    # One seeded batch per step, none used twice: every step, timed or not, meets its own share of signs the
+    # table does not hold yet (cfg3: the Zipf tail beyond the 5e8 resident ids, about 1 % of the lookups) and
+    # inserts them inside the step (SparseKernelBlock::GetWeight, core/ps/optimizer/optimizer_kernel.h:299-308).
+    psteps = max(1, min(args.profile_steps, args.steps))
+    nb = args.warmup + args.steps + psteps
     rng = torch.Generator(device="cuda")
     rng.manual_seed(0)
-    for b, hb in enumerate(host_batches):
+    t_gen = time.time()
+    host_batch0 = None
+    batches = []
+    for b in range(nb):
+        hb = synth.make_batch(cfg, b)
+        if b == 0:
+            host_batch0 = hb
         values = [torch.from_numpy(v).cuda() for v in hb]
         labels = [torch.from_numpy(l).cuda() for l in synth.make_labels(hb, b)]
         # gradient matrices have one row per possible distinct sign; the op reads the first U_s
         grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
         vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
         batches.append((values, labels, grads, vars_))
-    L = sum(len(v) for v in host_batches[0])
-    n_slots = len(host_batches[0])
+    log("generated %d batches in %.1f s" % (nb, time.time() - t_gen))
+    n_slots = len(batches[0][0])
 
     # The ops are bound to their tensors once, as an op kernel of a built graph is: the timed
     # region holds the calls through the C ABI, not Python's per-tensor argument marshalling.
@@ -249,7 +258,7 @@ def main():
              for values, labels, grads, vars_ in batches]
 
     def step(i):
-        pull, push = bound[i % nb]
+        pull, push = bound[i]
         pull()
         push()
 
@@ -257,43 +266,39 @@ def main():
         step(i)
     tn.ops.sparse_table_sync(h)
     torch.cuda.synchronize()
-    # per-batch sizes (U from the last pull of each batch; G measured once below)
-    Ls, Us = [], []
-    for i in range(nb):
-        values, labels, grads, vars_ = batches[i]
-        tn.ops.sparse_table_pull(vars_, values, h)
-        Us.append(sum(tn.ops.sparse_table_last_unique_counts(h, n_slots)))
-        Ls.append(sum(v.numel() for v in values))
-    shapes = [batch_shape(b[0]) for b in batches]
-    G0 = shapes[0]["G"]
-    torch.cuda.synchronize()
+    timed = range(args.warmup, args.warmup + args.steps)
+    Ls = [sum(v.numel() for v in batches[i][0]) for i in timed]
+    keys_before = tn.core.sparse_table_key_count(h)
 
     # ---- timed region ------------------------------------------------------------
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
+    Us = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ev0.record()
-    for i in range(args.steps):
+    for i in timed:
         step(i)
     ev1.record()
     tn.ops.sparse_table_sync(h)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    total_L = sum(Ls[i % nb] for i in range(args.steps))
-    total_U = sum(Us[i % nb] for i in range(args.steps))
+    new_keys = tn.core.sparse_table_key_count(h) - keys_before
+    # per-slot distinct signs of the timed batches: counted by torch on the device, after the clock has stopped
+    Us = [sum(int(torch.unique(v).numel()) for v in batches[i][0]) for i in timed]
+    total_L, total_U = sum(Ls), sum(Us)
     value = total_L / wall
     alg = step_algorithmic_bytes(opt_name, dim, total_L, total_U)
-    log("timed %d steps: %.3f ms/step (events %.3f ms/step), %.3e keys/s" %
-        (args.steps, ms_per_step, ev0.elapsed_time(ev1) / args.steps, value))
+    log("timed %d steps: %.3f ms/step (events %.3f ms/step), %.3e keys/s, %.0f new keys per step" %
+        (args.steps, ms_per_step, ev0.elapsed_time(ev1) / args.steps, value, new_keys / args.steps))
 
     # ---- per-kernel durations, HIP events around every launch --------------------
     lib = tn.load()
     lib.tn_profile_reset()
     lib.tn_profile_enable(1)
-    psteps = min(args.steps, 10)
-    for i in range(psteps):
+    prof_range = range(args.warmup + args.steps, nb)
+    for i in prof_range:
         step(i)
     tn.ops.sparse_table_sync(h)
     torch.cuda.synchronize()
@@ -303,6 +308,8 @@ def main():
     per_step = {k: (c / psteps, ms / psteps) for k, (c, ms) in prof.items()}
     kernel_ms = sum(ms for _, ms in per_step.values())
     # the dominant kernel of the step's critical path
+    shapes = [batch_shape(batches[i][0]) for i in list(prof_range)[:2]]
+    G0 = shapes[0]["G"]
     mean_shape = {k: sum(sh[k] for sh in shapes) / len(shapes) for k in shapes[0]}
     dominant = max((kv for kv in per_step.items() if not kv[0].startswith(SIDE_STREAM_KERNELS)
                     and kernel_algorithmic_bytes(kv[0], opt_name, dim, mean_shape) > 0), key=lambda kv: kv[1][1])
@@ -335,8 +342,9 @@ def main():
                            opt_name, resident, 100 * synth.CLICK_RATE),
             "lookups_per_step": mean_L,
             "distinct_rows_per_step": mean_U,
-            "globally_distinct_keys_batch0": G0,
+            "globally_distinct_keys_of_a_batch": G0,
             "distinct_batches": nb,
+            "new_keys_per_step": new_keys / args.steps,
         },
         "rows_per_s": total_U / wall,
         "step_algorithmic_GBps": alg / wall / 1e9,
@@ -365,7 +373,7 @@ def main():
     if not args.no_combiner:
         crng = np.random.default_rng(0)
         cb = []
-        for values, labels, grads, vars_ in batches:
+        for values, labels, grads, vars_ in batches[:4]:  # batches the table has seen: a side measurement
             ex = [torch.from_numpy(np.sort(crng.integers(0, cfg["batch"], v.numel()))).cuda() for v in values]
             pooled = [torch.randn((cfg["batch"], dim), device="cuda", generator=rng) * cfg["grad_sigma"] for _ in values]
             pull = tn.ops.BoundSparseTablePull(vars_, values, h)
@@ -373,7 +381,7 @@ def main():
             cb.append((pull, push, vars_, ex))
 
         def cstep(i):
-            pull, push, vars_, ex = cb[i % nb]
+            pull, push, vars_, ex = cb[i % len(cb)]
             mapped = pull()
             tn.ops.embedding_lookup_sparse(vars_, mapped, ex, cfg["batch"], h, "mean")
             push()
@@ -493,7 +501,7 @@ def main():
         del w, g
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg, host_batches[0], cfg["grad_sigma"])
+        out["cpu_baseline"] = cpu_baseline(cfg, host_batch0, cfg["grad_sigma"])
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out), flush=True)

@@ -707,13 +707,22 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
 // stream of its own beside the grouping and the ranking (random reads of the table against LDS
 // and streaming work).  A sign present in several slots is probed once per slot; whichever
 // thread claims a free slot first owns the insertion, the others find the key there.
+// A new row is not filled here: one or two lanes of a wavefront drawing sixteen normal deviates would hold up
+// the other sixty (with 1 % of the lookups new, most wavefronts have such a lane); the record is listed in
+// newlist and k_init_new_recs fills the rows with every lane busy.
 __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, uint32_t* __restrict__ rrow,
-                                                    Store s, OptDev o, uint64_t seed, DevStatus* status) {
-    // whole wavefronts take part in every round (wave_alloc votes)
+                                                    uint32_t* __restrict__ newlist, Store s, DevStatus* status) {
+    // The new rows of a bucket are collected in LDS and get their places in newlist with ONE atomic on the
+    // call's counter: an atomic per wavefront (tens of thousands on one address, about 11 ns each one after
+    // the other) took longer than all the probes together.
+    __shared__ uint32_t s_new[GRP_CAP];
+    __shared__ uint32_t s_count, s_base;
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
+        if (threadIdx.x == 0) s_count = 0;
+        __syncthreads();
         for (uint32_t i0 = 0; i0 < n; i0 += 256) {
             const uint32_t i = i0 + threadIdx.x;
             bool is_new = false;
@@ -722,9 +731,49 @@ __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t
                 const uint32_t row = probe_slot<true>(s, sign, is_new);
                 rrow[first + i] = row;
                 if (row == NO_ROW) atomicOr(&status->err, DEV_ERR_TABLE_FULL);
-                if (is_new) init_row(s, o, seed, sign, row);  // the thread that claimed the row fills it
             }
-            wave_alloc(is_new, &status->n_new);
+            if (is_new) s_new[atomicAdd(&s_count, 1u)] = i;  // rare: about one record in forty
+        }
+        __syncthreads();
+        const uint32_t cnt = s_count;
+        if (cnt) {
+            if (threadIdx.x == 0) s_base = atomicAdd(&status->n_new, cnt);
+            __syncthreads();
+            for (uint32_t j = threadIdx.x; j < cnt; j += 256) newlist[s_base + j] = (uint32_t)(first + s_new[j]);
+        }
+        __syncthreads();
+    }
+}
+
+// Fills the rows k_probe_recs inserted (the row initialiser of init_row): one lane per pair of elements, the
+// first lane of a row also its padding columns and optimizer state.
+__global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64_t seed,
+                                                       const GroupRec* __restrict__ recs,
+                                                       const uint32_t* __restrict__ rrow,
+                                                       const uint32_t* __restrict__ newlist, const DevStatus* status) {
+    const uint32_t n_new = status->n_new;
+    const uint32_t pairs = (uint32_t)(s.D + 1) / 2;
+    const uint64_t total = (uint64_t)n_new * pairs;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const float stddev = (float)(1.0 / sqrt((double)s.D));
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
+        const uint32_t j = (uint32_t)(t / pairs), q = (uint32_t)(t - (uint64_t)j * pairs);
+        const uint32_t i = newlist[j];
+        const uint64_t sign = recs[i].sign;
+        const uint64_t row = rrow[i];
+        float* w = s.w + row * s.wstride;
+        const int c = 2 * (int)q;
+        float2 z = make_float2(0.f, 0.f);
+        if (!o.zero_init) {
+            z = normal_pair(rnd64(seed, sign, (uint64_t)q));
+            z.x = (z.x * stddev) * o.initial_scale;
+            z.y = (z.y * stddev) * o.initial_scale;
+        }
+        w[c] = z.x;
+        if (c + 1 < s.D) w[c + 1] = z.y;
+        if (q == 0) {
+            for (int e = s.D; e < s.wlen; e++) w[e] = 0.f;  // cvm columns / padding
+            init_state(s, o, s.st + row * s.sstride);
         }
     }
 }

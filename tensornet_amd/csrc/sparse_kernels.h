@@ -249,24 +249,45 @@ __global__ __launch_bounds__(256) void k_probe(Store s, const uint64_t* __restri
                                                const DevStatus* groups_of, uint32_t ids_cap,
                                                uint32_t* __restrict__ rows, uint32_t* __restrict__ newlist,
                                                DevStatus* status, uint32_t miss_err, OptDev o, uint64_t seed) {
+    __shared__ uint32_t wcount[4];
+    __shared__ uint32_t block_base;
     const uint32_t n_single = groups_of ? groups_of->n_single : 0, n_multi = groups_of ? groups_of->n_multi : 0;
     const int64_t n = groups_of ? (int64_t)n_single + n_multi : n_host;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride) {
-        const int64_t i = groups_of ? (int64_t)group_id((uint32_t)t, n_single, n_multi, ids_cap) : t;
-        const uint64_t sign = signs[i];
-        bool is_new;
-        const uint32_t row = probe_slot<INSERT>(s, sign, is_new);
-        rows[i] = row;
-        if (row == NO_ROW && miss_err) atomicOr(&status->err, miss_err);
+    // every thread of the workgroup takes part in every round: the places of the new rows of a round are handed
+    // out with one atomic per workgroup (atomics on the one counter run one after the other, about 11 ns each)
+    for (int64_t t0 = (int64_t)blockIdx.x * blockDim.x; t0 < n; t0 += stride) {
+        const int64_t t = t0 + threadIdx.x;
+        bool is_new = false;
+        int64_t i = 0;
+        uint64_t sign = 0;
+        uint32_t row = NO_ROW;
+        if (t < n) {
+            i = groups_of ? (int64_t)group_id((uint32_t)t, n_single, n_multi, ids_cap) : t;
+            sign = signs[i];
+            row = probe_slot<INSERT>(s, sign, is_new);
+            rows[i] = row;
+            if (row == NO_ROW && miss_err) atomicOr(&status->err, miss_err);
+        }
         if (INSERT) {
-            uint32_t j = wave_alloc(is_new, &status->n_new);
+            const unsigned long long mask = __ballot(is_new);
+            const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+            if (lane == 0) wcount[wave] = (uint32_t)__popcll(mask);
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const uint32_t total = wcount[0] + wcount[1] + wcount[2] + wcount[3];
+                block_base = total ? atomicAdd(&status->n_new, total) : 0u;
+            }
+            __syncthreads();
             if (is_new) {
+                uint32_t j = block_base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                for (int wv = 0; wv < wave; wv++) j += wcount[wv];
                 if (newlist)
                     newlist[j] = (uint32_t)i;  // initialised by k_init_rows
                 else
                     init_row(s, o, seed, sign, row);  // the thread that claimed the row fills it
             }
+            __syncthreads();
         }
     }
 }

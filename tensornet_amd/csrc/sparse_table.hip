@@ -28,6 +28,7 @@ namespace {
 constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:266
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
+constexpr int INIT_NEW_GRID = 512;    // workgroups of k_init_new_recs (the number of new rows is known on the device only)
 constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 512-1024 are best)
 // Below this many lookups a call keeps all its kernels on the caller's stream.  The kernels of a smaller
 // batch are too short for the overlap on the side streams to win back what the events that fork and
@@ -701,8 +702,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
                 TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
             }
             // few workgroups: enough probes in flight for the memory system, most of every CU left to the grouping
-            TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), sd2, w.nb2, w.cursor2, w.recs, w.rrow, s,
-                      make_optdev(t), t->seed, ds);
+            TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), sd2, w.nb2, w.cursor2, w.recs, w.rrow,
+                      p.newlist, s, ds);
+            TN_LAUNCH(k_init_new_recs, dim3(INIT_NEW_GRID), dim3(256), sd2, s, make_optdev(t), t->seed, w.recs, w.rrow,
+                      p.newlist, ds);
             if (!t->one_stream) TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
