@@ -139,7 +139,7 @@ enum { STATUS_KEEP = 0, STATUS_NEW_PLAN = 1, STATUS_REUSE_PLAN = 2 };
 __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ host_src, uint32_t* __restrict__ dst_a,
                                                   uint32_t words_a, uint32_t* __restrict__ dst_b, uint32_t words_b,
                                                   DevStatus* status, int status_mode, uint32_t* __restrict__ zero,
-                                                  uint32_t n_zero) {
+                                                  uint32_t n_zero, const DevStatus* plan_status) {
     const uint32_t stride = gridDim.x * blockDim.x;
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     for (uint32_t i = tid; i < words_a + words_b; i += stride) {
@@ -150,6 +150,8 @@ __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ h
     }
     for (uint32_t i = tid; i < n_zero; i += stride) zero[i] = 0;
     if (tid == 0 && status_mode != STATUS_KEEP) {
+        // a push on the last pull's plan has a status block of its own: the plan's counts, fresh flags
+        if (status_mode == STATUS_REUSE_PLAN && plan_status != status) *status = *plan_status;
         status->err = 0;
         status->mismatch = 0;
         status->abort = 0;

@@ -39,6 +39,8 @@ constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to w
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
 constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS wins: it also takes fewer launches (cfg1, 8 k lookups: 0.154 -> 0.136 ms)
 
+enum { FLOW_NONE = 0, FLOW_PULL = 1, FLOW_PUSH = 2 };
+
 struct HostStatus {
     DevStatus st;
     uint32_t ubase[MAX_SLOTS + 1];
@@ -67,6 +69,7 @@ struct SparseTable {
     uint64_t plan_epoch = 0;
     DevStatus* dstatus = nullptr;   // device: status of table-level calls
     DevStatus* dplan = nullptr;     // device: status / counts of the op-level plan
+    DevStatus* dpush = nullptr;     // device: status of a push that reuses the plan (the plan's counts, flags of its own)
     HostStatus* hpull = nullptr;    // pinned
     HostStatus* hpush = nullptr;    // pinned
     unsigned long long* hcount = nullptr;  // pinned: the number of resident keys is read into it
@@ -78,7 +81,18 @@ struct SparseTable {
     DevBuf pooled_ws;               // scratch of a push of pooled gradients (sort buffers, reduced rows)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
+    // The slot descriptors of a call reach the device here while the caller's stream still runs the tail of the
+    // call before (a pull's gather, a push's updates): the kernel reads pinned host memory, whose round trips
+    // would otherwise stand at the head of every call.
+    hipStream_t aux = nullptr;
     hipEvent_t fork_ev = nullptr, join_ev = nullptr, join2_ev = nullptr;
+    hipEvent_t apply_ev = nullptr;  // a push's updates are done (its status is published beside what follows)
+    // The call before this one on the table, if it left work behind on `flow_stream` that the next call of the
+    // training loop may overlap with: FLOW_PULL = a pull that returned before its gather, FLOW_PUSH = a push
+    // on that pull's plan.  Every entry point clears it (ensure_allocated); pull and push set it again.
+    int flow = 0;
+    hipStream_t flow_stream = nullptr;
+    bool push_pub_on_side = false;  // the pending push's status is published on the side stream
     // A pull whose status is final before its last kernel (the gather) publishes it on the side stream
     // meanwhile and returns when it is there: ready_ev = the status can be published, pub_ev = it is on
     // the host, tail_ev = the gather is done (what a call on another stream has to wait for).
@@ -214,9 +228,10 @@ void free_store(Store& s) {
 
 int ensure_side_buffers(SparseTable* t) {
     if (t->dstatus) return TN_OK;
-    TN_HIP(hipMalloc((void**)&t->dstatus, 2 * sizeof(DevStatus)));
-    TN_HIP(hipMemset(t->dstatus, 0, 2 * sizeof(DevStatus)));
+    TN_HIP(hipMalloc((void**)&t->dstatus, 3 * sizeof(DevStatus)));
+    TN_HIP(hipMemset(t->dstatus, 0, 3 * sizeof(DevStatus)));
     t->dplan = t->dstatus + 1;
+    t->dpush = t->dstatus + 2;
     TN_HIP(hipHostMalloc((void**)&t->hpull, sizeof(HostStatus), hipHostMallocDefault));
     TN_HIP(hipHostMalloc((void**)&t->hpush, sizeof(HostStatus), hipHostMallocDefault));
     std::memset(t->hpull, 0, sizeof(HostStatus));
@@ -232,8 +247,10 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipEventCreateWithFlags(&t->ready_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->pub_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->tail_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->apply_ev, hipEventDisableTiming));
     TN_HIP(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));  // default priority
     TN_HIP(hipStreamCreateWithFlags(&t->side2, hipStreamNonBlocking));
+    TN_HIP(hipStreamCreateWithFlags(&t->aux, hipStreamNonBlocking));
     return TN_OK;
 }
 
@@ -241,6 +258,7 @@ int ensure_allocated(SparseTable* t, hipStream_t st) {
     TN_TRY(ensure_side_buffers(t));
     // work of the last pull that its caller did not wait for was queued on that call's stream
     if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
+    t->flow = FLOW_NONE;  // pull and push read it before they get here and set it again
     if (t->allocated) return TN_OK;
     uint64_t cap = DEFAULT_SLOTS;
     if (t->reserve_keys) cap = (uint64_t)((double)t->reserve_keys / MAX_LOAD) + 64;
@@ -278,6 +296,11 @@ void harvest(SparseTable* t) {
     // a pending push is older than a pending pull (a push collects everything before it starts)
     if (t->push_pending) {
         t->push_pending = false;
+        if (t->push_pub_on_side) {  // its status went out on the side stream, behind its updates
+            t->push_pub_on_side = false;
+            const hipError_t e = hipStreamSynchronize(t->side);
+            if (e != hipSuccess) latch(t, TN_ERR_HIP, std::string("sparse push: ") + hipGetErrorString(e));
+        }
         const HostStatus& h = *t->hpush;
         int N = t->push_slots;
         if (N > 0) {
@@ -393,6 +416,7 @@ struct Carver {
 // from the per-call scratch.
 struct Plan {
     SlotDesc* descs;
+    SlotDesc* push_descs;  // descriptors of the push that reuses the plan (the pull's gather may still read `descs`)
     uint32_t* lbase;
     uint32_t* ubase;
     uint64_t* vals_copy;   // signs of every lookup, concatenated
@@ -473,6 +497,7 @@ void carve_group_scratch(Carver& c, Scratch& w, size_t n) {
 size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     Carver c{base};
     p.descs = c.take<SlotDesc>(N);
+    p.push_descs = c.take<SlotDesc>(N);
     p.lbase = c.take<uint32_t>(N + 1);
     p.ubase = c.take<uint32_t>(N + 1);
     p.vals_copy = c.take<uint64_t>(L);
@@ -590,33 +615,34 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
     return TN_OK;
 }
 
-// Slot descriptors to the device; the same launch prepares the plan's status block
-// (status_mode) and clears `zero[0 .. n_zero)`.
-int upload_slots(SparseTable* t, const Plan& p, const std::vector<SlotDesc>& descs,
-                 const std::vector<uint32_t>& lbase, hipStream_t st, int status_mode, uint32_t* zero = nullptr,
-                 uint32_t n_zero = 0) {
+// Slot descriptors to the device (dst_descs; the slots' first lookups to dst_lbase unless nullptr); the same
+// launch prepares the call's status block `ds` (status_mode) and clears `zero[0 .. n_zero)`.  It runs on `run_on`.
+int upload_slots(SparseTable* t, SlotDesc* dst_descs, uint32_t* dst_lbase, DevStatus* ds,
+                 const std::vector<SlotDesc>& descs, const std::vector<uint32_t>& lbase, hipStream_t run_on,
+                 int status_mode, uint32_t* zero = nullptr, uint32_t n_zero = 0) {
     if (t->stage_pending) {
         TN_HIP(hipEventSynchronize(t->stage_ev));
         t->stage_pending = false;
     }
     const size_t db = descs.size() * sizeof(SlotDesc);
-    const size_t lb = lbase.size() * sizeof(uint32_t);
+    const size_t lb = dst_lbase ? lbase.size() * sizeof(uint32_t) : 0;
     std::memcpy(t->hstage, descs.data(), db);
-    std::memcpy(t->hstage + db, lbase.data(), lb);
-    TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)std::max<size_t>((db + lb) / 4, n_zero), 256, 64)), dim3(256), st,
-              reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(p.descs), (uint32_t)(db / 4),
-              p.lbase, (uint32_t)(lb / 4), t->dplan, status_mode, zero, n_zero);
-    TN_HIP(hipEventRecord(t->stage_ev, st));
+    if (lb) std::memcpy(t->hstage + db, lbase.data(), lb);
+    TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)std::max<size_t>((db + lb) / 4, n_zero), 256, 64)), dim3(256),
+              run_on, reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(dst_descs),
+              (uint32_t)(db / 4), dst_lbase, (uint32_t)(lb / 4), ds, status_mode, zero, n_zero,
+              (const DevStatus*)t->dplan);
+    TN_HIP(hipEventRecord(t->stage_ev, run_on));
     t->stage_pending = true;
     return TN_OK;
 }
 
-PushSrc op_source(const Plan& p, int dim) {
+PushSrc op_source(const Plan& p, int dim, const SlotDesc* descs = nullptr) {
     PushSrc src{};
     src.uniq_sign = p.uniq_sign;
     src.uniq_slot = p.uniq_slot;
     src.ubase = p.ubase;
-    src.descs = p.descs;
+    src.descs = descs ? descs : p.descs;
     src.dim = dim;
     return src;
 }
@@ -1320,6 +1346,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     if (!vars || !var_rows || !mapped_values) return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePull: NULL argument");
     std::lock_guard<std::mutex> lk(t->mu);
     hipStream_t st = (hipStream_t)stream;
+    // the call before was a push on the last pull's plan, on this stream: its updates may still be running
+    bool behind_push = t->flow == FLOW_PUSH && t->flow_stream == st;
     TN_TRY(ensure_allocated(t, st));
     const int wdim = t->dim + (t->use_cvm ? 2 : 0);
     if (var_dim != wdim)
@@ -1368,8 +1396,15 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds, t->distinct_est);
         w.span_cap = span_cap;
         t->plan_valid = false;
-        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN, use_lds ? w.bcount : nullptr,
-                            use_lds ? w.nbuckets + 1 + w.nb2 : 0));
+        // Behind a push of the training loop the descriptors go in on the auxiliary stream, beside that push's
+        // updates: those read the push's own descriptors and status block, and nothing of the scratch buffer.
+        // (Same slot count: the arrays at the head of the plan buffer keep their places.)
+        const bool hoist = behind_push && attempt == 0 && !t->one_stream && N == t->plan_N;
+        behind_push = false;
+        if (hoist && t->tail_recorded) TN_HIP(hipStreamWaitEvent(t->aux, t->tail_ev, 0));  // the gather that read p.descs
+        TN_TRY(upload_slots(t, p.descs, p.lbase, t->dplan, descs, lbase, hoist ? t->aux : st, STATUS_NEW_PLAN,
+                            use_lds ? w.bcount : nullptr, use_lds ? w.nbuckets + 1 + w.nb2 : 0));
+        if (hoist) TN_HIP(hipStreamWaitEvent(st, t->stage_ev, 0));
 
         const Store& s = t->store;
         DevStatus* ds = t->dplan;
@@ -1423,7 +1458,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             continue;
         }
         if (early) {
+            t->push_pub_on_side = false;  // a push's status went out on the side stream ahead of this call's
             harvest(t);
+            t->flow = FLOW_PULL;
+            t->flow_stream = st;
             return take_latched(t);
         }
         return sync_table(t, st);
@@ -1450,6 +1488,8 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         return fail(TN_ERR_INVALID_ARGUMENT, "SparseTablePush (pooled): bad batch size or combiner");
     std::lock_guard<std::mutex> lk(t->mu);
     hipStream_t st = (hipStream_t)stream;
+    // the call before was a pull on this stream that returned before its gather
+    const bool behind_pull = t->flow == FLOW_PULL && t->flow_stream == st;
     TN_TRY(ensure_allocated(t, st));
     const int wdim = t->dim + (t->use_cvm ? 2 : 0);
     if (grad_dim != wdim)
@@ -1487,22 +1527,26 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     // themselves are compared on the device.
     bool reuse = t->plan_valid && t->plan_epoch == t->epoch && t->plan_N == N &&
                  std::equal(value_lens, value_lens + N, t->plan_lens.begin());
-    DevStatus* ds = t->dplan;
+    // A push on the last pull's plan has its own descriptors and status block (the plan's counts, flags of its
+    // own): the pull's gather may still be running, and the next pull may stage its slots while this push's
+    // updates run.  A push that analyses its batch itself uses the plan's.
+    DevStatus* ds = reuse ? t->dpush : t->dplan;
+    const SlotDesc* pd = nullptr;  // set with the plan
     const int lblocks = launch_grid(L, 256, GRID_CAP * 2);
     const bool with_click = t->opt->kind == OPT_ADAGRAD;  // the only optimizer that reads batch_click
     // show / click counts of the batch into the member lists of a plan that has none
     auto launch_counts = [&]() -> int {
         TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 0);
         TN_LAUNCH(k_count_show, dim3(launch_grid((int64_t)(L + COUNT_TILE - 1) / COUNT_TILE, 1, GRID_CAP)), dim3(256),
-                  st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, p.where_u, p.list, with_click ? 1 : 0);
+                  st, pd, p.lbase, N, (uint32_t)L, p.u_of_gi, p.where_u, p.list, with_click ? 1 : 0);
         return TN_OK;
     };
     // Where the apply kernels find the gradient of a record.  Pooled gradients are first reduced
     // to one row per distinct sign: stable sort of (distinct index, position) pairs, then one
     // ordered sum per distinct index.
-    PushSrc src = op_source(p, grad_dim);
+    PushSrc src{};
     auto prepare_src = [&]() -> int {
-        src = op_source(p, grad_dim);
+        src = op_source(p, grad_dim, pd);
         if (!pooled) return TN_OK;
         int bits = 1;
         while (bits < 32 && (1ull << bits) < L) bits++;
@@ -1528,7 +1572,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         TN_TRY(t->pooled_ws.ensure(align_up(c.off, 256)));
         Carver c2{(char*)t->pooled_ws.p};
         carve(c2);
-        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, p.descs, p.lbase, N, (uint32_t)L, p.u_of_gi, batch, keys,
+        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, pd, p.lbase, N, (uint32_t)L, p.u_of_gi, batch, keys,
                   vals, ds, long_count);
         TN_TRY(sort_pairs_u32_u64(temp, temp_bytes, keys, skeys, vals, svals, L, bits, st));
         TN_LAUNCH(k_segment_starts, dim3(lblocks), dim3(256), st, skeys, (uint32_t)L, ds, seg_off);
@@ -1538,16 +1582,16 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         const int long_blocks = launch_grid((int64_t)L / LONG_SEGMENT + 1, 1, GRID_CAP);
         if (vec) {
             TN_LAUNCH((k_reduce_pooled<4>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
-                      p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
+                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
                       long_count);
-            TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim, combiner,
+            TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), st, pd, p.ubase, N, grad_dim, combiner,
                       seg_off, svals, flat, long_list, long_count, ds);
         } else {
             TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
-                      p.descs, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
+                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
                       long_count);
             if (long_min != 0xFFFFFFFFu)
-                TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), st, p.descs, p.ubase, N, grad_dim,
+                TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), st, pd, p.ubase, N, grad_dim,
                           combiner, seg_off, svals, flat, long_list, long_count, ds);
         }
         src.flat = flat;
@@ -1555,7 +1599,13 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     };
     if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
-        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_REUSE_PLAN));
+        pd = p.push_descs;
+        // behind a pull that returned before its gather the descriptors go in on the auxiliary stream, beside
+        // that gather (the plan's counts are final from ready_ev on)
+        const bool hoist = behind_pull && !t->one_stream;
+        if (hoist) TN_HIP(hipStreamWaitEvent(t->aux, t->ready_ev, 0));
+        TN_TRY(upload_slots(t, p.push_descs, nullptr, ds, descs, lbase, hoist ? t->aux : st, STATUS_REUSE_PLAN));
+        if (hoist) TN_HIP(hipStreamWaitEvent(st, t->stage_ev, 0));
         // On a plan with show counts the verify pass also sums the clicks; they start at zero
         // after the pull, a further push on the same plan clears them first.
         const bool clicks = t->plan_has_show && with_click;
@@ -1566,17 +1616,17 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         uint32_t* host_mismatch = &t->hpush->st.mismatch;
         // op-level gradients (not pooled): the verify pass also works out the gradient addresses of the records
         // of the groups with several records (see k_member_grads)
-        const PushSrc vsrc = op_source(p, grad_dim);
+        const PushSrc vsrc = op_source(p, grad_dim, pd);
         const bool addr_in_verify = !pooled && big_threshold(t->store) != 0xFFFFFFFFu;
         const float** vgaddr = addr_in_verify ? p.gaddr : nullptr;
         if (clicks) {
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
-            TN_LAUNCH_LDS((k_verify_values<true>), dim3(vblocks), dim3(256), vlds, st, p.descs, p.lbase, N, (uint32_t)L,
+            TN_LAUNCH_LDS((k_verify_values<true>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L,
                           p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         } else {
-            TN_LAUNCH_LDS((k_verify_values<false>), dim3(vblocks), dim3(256), vlds, st, p.descs, p.lbase, N, (uint32_t)L,
+            TN_LAUNCH_LDS((k_verify_values<false>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L,
                           p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
         }
         TN_HIP(hipEventRecord(t->verify_ev, st));
@@ -1593,21 +1643,35 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // another batch than the last pull's: analyse it here, on the global-table path
         // (its status cannot be waited for, a push only enqueues)
         t->plan_valid = false;
+        ds = t->dplan;
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
         carve_plan((char*)t->plan_buf.p, p, N, L);
+        pd = p.descs;
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, false)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, false);
-        TN_TRY(upload_slots(t, p, descs, lbase, st, STATUS_NEW_PLAN));
+        TN_TRY(upload_slots(t, p.descs, p.lbase, ds, descs, lbase, st, STATUS_NEW_PLAN));
         TN_TRY(launch_build_plan(t, p, w, N, (uint32_t)L, false, false, st));
         TN_TRY(launch_counts());
         TN_TRY(prepare_src());
         TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st));
     }
     TN_HIP(hipGetLastError());
-    TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush),
-              (unsigned long long*)nullptr);
+    // The status of a large push goes out on the side stream, behind the updates and beside whatever the caller's
+    // stream runs next (a pull's status follows it on that stream, so whoever has that one has this one too).
+    const bool pub_on_side = reuse && !t->one_stream;
+    if (pub_on_side) {
+        TN_HIP(hipEventRecord(t->apply_ev, st));
+        TN_HIP(hipStreamWaitEvent(t->side, t->apply_ev, 0));
+    }
+    TN_LAUNCH(k_publish, dim3(1), dim3(256), pub_on_side ? t->side : st, ds, p.ubase, (uint32_t)(N + 1),
+              reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr);
     t->push_pending = true;
+    t->push_pub_on_side = pub_on_side;
     t->push_slots = N;
+    if (reuse) {
+        t->flow = FLOW_PUSH;
+        t->flow_stream = st;
+    }
     return TN_OK;
 }
 
@@ -1689,7 +1753,8 @@ int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* cons
         std::memcpy(t->hstage + db, lbase.data(), lb);
         TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)(db + lb) / 4, 256, 64)), dim3(256), st,
                   reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(ddescs), (uint32_t)(db / 4),
-                  dlbase, (uint32_t)(lb / 4), t->dstatus, (int)STATUS_NEW_PLAN, (uint32_t*)nullptr, 0u);
+                  dlbase, (uint32_t)(lb / 4), t->dstatus, (int)STATUS_NEW_PLAN, (uint32_t*)nullptr, 0u,
+                  (const DevStatus*)t->dstatus);
         TN_HIP(hipEventRecord(t->stage_ev, st));
         t->stage_pending = true;
         // where the lookups of every example start, then one thread group per (slot, example)
