@@ -129,21 +129,12 @@ def batch_shape(values):
     }
 
 
-def populate(tn, handle, resident, dim, chunk=1 << 23):
-    """Loads splitmix64(1..resident) with the synthetic snapshot rows, in chunks."""
-    import torch
-
+def populate(tn, handle, resident, dim):
+    """Loads splitmix64(1..resident) with the synthetic snapshot rows."""
     from tensornet_amd import synth
 
     t0 = time.time()
-    for lo in range(1, resident + 1, chunk):
-        hi = min(resident + 1, lo + chunk)
-        ids = torch.arange(lo, hi, dtype=torch.int64, device="cuda")
-        signs = synth.splitmix64_torch(ids)
-        w = synth.snapshot_rows_torch(signs, dim)
-        tn.ops.table_load_rows(handle, signs, w)
-        del ids, signs, w
-    torch.cuda.synchronize()
+    synth.populate_table(tn, handle, resident, dim)
     log("populated %d keys in %.1f s" % (resident, time.time() - t0))
 
 

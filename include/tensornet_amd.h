@@ -142,6 +142,15 @@ int tn_sparse_table_create(tn_opt_t opt, const char* name, int dimension, int us
 /* Size the HBM table for at least max_keys resident keys at load factor <= 0.75. */
 int tn_sparse_table_reserve(uint32_t handle, uint64_t max_keys);
 
+/*
+ * Drops every row of the table and gives its device memory back (the table itself, its handle and its
+ * settings stay; the next call allocates an empty table again).  The reference's tables live in host hash maps
+ * until the process ends (SparseTableRegistry, core/ps/table/sparse_table.cc:150-186) and have no such call;
+ * a table that fills most of a GPU's memory needs one, for hosts that rebuild their tables (and for tests).
+ * Waits for the table's pending work first.
+ */
+int tn_sparse_table_clear(uint32_t handle);
+
 /* Seed of the on-device row initialiser (the reference seeds from the wall
  * clock, core/utility/random.h:30-42; here new rows are a pure function of
  * (seed, sign)). */

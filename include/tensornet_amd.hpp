@@ -168,6 +168,7 @@ public:
     }
     // HBM sizing (no counterpart in the reference, whose host maps grow by themselves).
     int Reserve(uint64_t max_keys) { return tn_sparse_table_reserve(handle_, max_keys); }
+    int Clear() { return tn_sparse_table_clear(handle_); }
     int Sync() { return tn_sparse_table_sync(handle_); }
 
 private:

@@ -99,6 +99,7 @@ SIGNATURES = {
         [C.c_int32, C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_char_p, C.POINTER(C.c_uint32)],
     ),
     "tn_sparse_table_reserve": (C.c_int, [C.c_uint32, C.c_uint64]),
+    "tn_sparse_table_clear": (C.c_int, [C.c_uint32]),
     "tn_sparse_table_set_seed": (C.c_int, [C.c_uint32, C.c_uint64]),
     "tn_sparse_table_key_count": (C.c_int, [C.c_uint32, C.POINTER(C.c_uint64)]),
     "tn_sparse_table_capacity": (C.c_int, [C.c_uint32, C.POINTER(C.c_uint64)]),

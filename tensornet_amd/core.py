@@ -143,6 +143,12 @@ def reserve_sparse_table(table_handle, max_keys):
     _lib.check(_lib.load().tn_sparse_table_reserve(table_handle, int(max_keys)))
 
 
+def clear_sparse_table(table_handle):
+    """Drops every row of the table and frees its device memory (no counterpart in the
+    reference, whose tables live in host memory until the process ends)."""
+    _lib.check(_lib.load().tn_sparse_table_clear(table_handle))
+
+
 def set_sparse_table_seed(table_handle, seed):
     _lib.check(_lib.load().tn_sparse_table_set_seed(table_handle, int(seed) & 0xFFFFFFFFFFFFFFFF))
 

@@ -916,6 +916,34 @@ int tn_sparse_table_reserve(uint32_t handle, uint64_t max_keys) {
     return grow_to(t, want, st);
 }
 
+int tn_sparse_table_clear(uint32_t handle) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_clear: bad table handle " + std::to_string(handle));
+    std::lock_guard<std::mutex> lk(t->mu);
+    if (!t->allocated) return TN_OK;
+    // everything the table has queued, on whichever stream
+    if (t->last_stream) TN_HIP(hipStreamSynchronize(t->last_stream));
+    TN_HIP(hipStreamSynchronize(t->side));
+    TN_HIP(hipStreamSynchronize(t->side2));
+    TN_HIP(hipStreamSynchronize(t->aux));
+    harvest(t);
+    free_store(t->store);
+    t->ws.release();
+    t->plan_buf.release();
+    t->comb_buf.release();
+    t->pooled_ws.release();
+    t->allocated = false;
+    t->plan_valid = false;
+    t->tail_recorded = false;
+    t->flow = FLOW_NONE;
+    t->count_upper = 0;
+    t->booked = 0;
+    t->epoch++;
+    t->latched = TN_OK;
+    t->latched_msg.clear();
+    return TN_OK;
+}
+
 int tn_sparse_table_set_seed(uint32_t handle, uint64_t seed) {
     SparseTable* t = get_table(handle);
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_set_seed: bad table handle " + std::to_string(handle));

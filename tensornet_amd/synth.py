@@ -127,3 +127,18 @@ def make_grads(counts, dim, sigma, seed=0):
     """Per-slot float32 [U_s, dim] gradients ~ N(0, sigma)."""
     rng = np.random.default_rng(1_000_003 + seed)
     return [(rng.standard_normal((int(u), dim)) * sigma).astype(np.float32) for u in counts]
+
+
+def populate_table(tn, handle, resident, dim, chunk=1 << 23):
+    """Loads the resident set splitmix64(1..resident) with its snapshot rows into a sparse
+    table on the GPU, in chunks (signs and rows are generated on the device)."""
+    import torch
+
+    for lo in range(1, resident + 1, chunk):
+        hi = min(resident + 1, lo + chunk)
+        ids = torch.arange(lo, hi, dtype=torch.int64, device="cuda")
+        signs = splitmix64_torch(ids)
+        w = snapshot_rows_torch(signs, dim)
+        tn.ops.table_load_rows(handle, signs, w)
+        del ids, signs, w
+    torch.cuda.synchronize()

@@ -7,7 +7,7 @@ import torch
 
 from tensornet_amd import synth
 
-from helpers import ATOL, RTOL, Pair, all_signs, dev
+from helpers import ATOL, RTOL, Pair, all_signs, check_pull, dev
 
 pytestmark = pytest.mark.gpu
 
@@ -23,21 +23,6 @@ def random_batch(rng, slots, max_len, vocab, ragged=True):
         n = int(rng.integers(0, max_len + 1)) if ragged else max_len
         out.append(pool[rng.integers(0, vocab, n)])
     return out
-
-
-def check_pull(pair, values, var_rows=None, loose_col=None):
-    """loose_col: a column compared with the update tolerance instead of bit for bit
-    (the cvm log column, whose value depends on the libm in use)."""
-    gm, gv, cm, cv, counts = pair.pull_op(values, var_rows)
-    for s in range(len(values)):
-        assert (gm[s].cpu().numpy() == cm[s]).all(), "mapped ids of slot %d" % s
-        g, c = gv[s].cpu().numpy(), cv[s]
-        if loose_col is not None:
-            np.testing.assert_allclose(g[:, loose_col], c[:, loose_col], rtol=RTOL, atol=ATOL)
-            g, c = np.delete(g, loose_col, 1), np.delete(c, loose_col, 1)
-        # bit-exact rows, including the untouched tail of the variable
-        assert (g.view(np.int32) == c.view(np.int32)).all(), "var rows of slot %d" % s
-    return counts
 
 
 def test_cfg1_pull_then_push(tn, oracle):
