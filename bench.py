@@ -400,8 +400,12 @@ def main():
         comb_bytes = {
             # signs' ids + example ids in, one output row per (slot, example) out, variable rows read once
             "k_combine_fwd": 16 * mean_L + 4 * dim * (cfg["batch"] * n_slots + mean_U),
-            # example ids + distinct index in, sort key + value out
-            "k_lookup_keys": 24 * mean_L,
+            # example ids in, value out
+            "k_lookup_keys": 16 * mean_L,
+            # distinct index (twice: count, place) + value in, index + value out at their place in the sign's segment
+            "k_place_lookups": 28 * mean_L,
+            # index + value in, value out at its rank in the segment
+            "k_rank_short": 20 * mean_L,
             # sorted values in, pooled rows read once, one reduced row per distinct sign out
             "k_reduce_pooled": 8 * mean_L + 4 * dim * (cfg["batch"] * n_slots + mean_U),
         }
@@ -410,11 +414,9 @@ def main():
             "ms_per_step": cms,
             "keys_per_s": mean_L / (cms * 1e-3),
             "kernels_ms_per_step": {k: round(v, 4) for k, v in cprof.items()
-                                    if k.startswith(("k_combine", "k_example", "k_lookup_keys", "k_segment", "k_reduce"))},
+                                    if k.startswith(("k_combine", "k_example", "k_lookup_keys", "k_place", "k_rank", "k_order", "k_reduce"))},
             "kernels_frac_of_hbm_peak": {k: round(comb_bytes[k.split("<")[0]] / (v * 1e-3) / HBM_PEAK, 4)
                                          for k, v in cprof.items() if k.split("<")[0] in comb_bytes},
-            "note": "the stable radix sort between k_lookup_keys and k_segment_starts is rocPRIM's; its time is "
-                    "in ms_per_step only",
         }
         log("combiner step: %.3f ms/step; %s" % (cms, out["combiner_step"]["kernels_ms_per_step"]))
 

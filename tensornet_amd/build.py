@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtensornet_amd.so")
-SOURCES = ["core.hip", "dense_table.hip", "sparse_table.hip", "sort_pairs.hip", "checkpoint.hip"]
+SOURCES = ["core.hip", "dense_table.hip", "sparse_table.hip", "checkpoint.hip"]
 HEADERS = ["tn_common.h", "sparse_kernels.h"]
 
 FLAGS = [

@@ -9,8 +9,9 @@
 //   backward  g[u, :]   = sum over the lookups i of distinct sign u, in order, of dout[b(i), :] * (1 / d(n_b(i)))
 //
 // Both are deterministic: sums run in occurrence order.  The backward pass
-// gets the lookups of every distinct sign side by side from a stable sort of
-// (distinct index, position) pairs.
+// gets the lookups of every distinct sign side by side, in position order, from a
+// counting sort per slot followed by an ordering of every sign's lookups by example
+// (k_place_lookups, k_rank_short, k_rank_mid, k_order_huge).
 #ifndef TN_COMBINE_KERNELS_H_
 #define TN_COMBINE_KERNELS_H_
 
@@ -129,21 +130,20 @@ __global__ __launch_bounds__(256) void k_zero_f32(float* __restrict__ out, int64
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = 0.f;
 }
 
-// Backward, step 1: sort keys (distinct index of every lookup) and values: the lookup's
-// example in the high word, the number of lookups of that example in the low word -- all the
-// reduction needs to know about the lookup, so that it reads them in sorted order instead of
-// chasing positions.  The first lookup of an example writes the values of all its lookups.
+// Backward, step 1: the value of every lookup: its example in the high word, the number of
+// lookups of that example in the low word -- all the reduction needs to know about the lookup, so
+// that it reads them in the order of the distinct signs instead of chasing positions.  The first
+// lookup of an example writes the values of all its lookups.
 __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict__ descs,
                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     const uint32_t* __restrict__ u_of_gi, int64_t batch,
-                                                     uint32_t* __restrict__ keys, uint64_t* __restrict__ vals,
-                                                     DevStatus* status, uint32_t* long_count) {
+                                                     int64_t batch, uint64_t* __restrict__ vals, DevStatus* status,
+                                                     uint32_t* long_count) {
     __shared__ uint32_t lb[MAX_SLOTS + 1];
     load_lbase(lb, lbase, N);
-    if (blockIdx.x == 0 && threadIdx.x == 0) *long_count = 0;  // list of the frequent signs, filled by k_reduce_pooled
+    // [0] list of the frequent signs, filled by k_reduce_pooled; [1], [2] lists of k_place_lookups
+    if (blockIdx.x == 0 && threadIdx.x < 3) long_count[threadIdx.x] = 0;
     const uint32_t stride = gridDim.x * blockDim.x;
     for (uint32_t gi = blockIdx.x * blockDim.x + threadIdx.x; gi < L; gi += stride) {
-        keys[gi] = u_of_gi[gi] & ~FIRST_BIT;
         const int sl = find_slot(lb, N, gi);
         const SlotDesc& d = descs[sl];
         const int64_t* ex = example_of(d);
@@ -164,15 +164,181 @@ __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict_
     }
 }
 
-// Step 2 (after the sort): where the lookups of every distinct index start.
-__global__ __launch_bounds__(256) void k_segment_starts(const uint32_t* __restrict__ skeys, uint32_t L,
-                                                        const DevStatus* status, uint32_t* __restrict__ seg_off) {
+// Step 2: the values of the lookups of every distinct index side by side, in position order:
+// svals[seg_off[u] .. seg_off[u + 1]).  The example ids of a slot ascend with the position and two lookups of
+// one sign in one example carry the same value, so "position order" is "ascending value" and ties do not
+// matter: no stable sort is needed.
+//   k_place_lookups  one workgroup per slot (the distinct indices of a slot's lookups fill a window of their
+//                    own, ascending with the slots): counts the lookups of every index in an LDS array, scans
+//                    the counts into seg_off, and puts every lookup into its index's segment -- in the order the
+//                    atomics arrive; indices with ORDER_MID lookups or more are listed for the kernels below
+//   k_rank_short     a lookup of a short segment finds its place by counting the values of its segment below it
+//   k_rank_mid       a sorting network in LDS, one workgroup per segment of ORDER_MID .. ORDER_HUGE - 1 lookups
+//   k_order_huge     the few longer segments: counting sort over the example ids, one workgroup each
+// A slot with more distinct signs than the LDS array holds (lds_cap) keeps its counters in `gcur`.
+constexpr int PLACE_THREADS = 1024;
+constexpr int PLACE_ITEMS = 8;
+constexpr uint32_t ORDER_MID = 64;
+constexpr uint32_t ORDER_HUGE = 1024;
+
+__global__ __launch_bounds__(PLACE_THREADS) void k_place_lookups(
+    const uint32_t* __restrict__ lbase, const uint32_t* __restrict__ ubase, int N, uint32_t L,
+    const uint32_t* __restrict__ u_of_gi, const uint64_t* __restrict__ vals, uint32_t* __restrict__ tkey,
+    uint64_t* __restrict__ tval, uint32_t* __restrict__ seg_off, uint32_t* __restrict__ gcur, uint32_t lds_cap,
+    uint32_t* __restrict__ mid_list, uint32_t* __restrict__ huge_list, uint32_t* counts, const DevStatus* status) {
+    extern __shared__ uint32_t lcur[];
+    __shared__ uint32_t red[PLACE_THREADS / 64];
+    __shared__ uint32_t carry_sh;
+    if (status->abort) return;
+    const int sl = blockIdx.x;
+    const uint32_t l0 = lbase[sl], len = lbase[sl + 1] - l0;
+    const uint32_t ub = ubase[sl], us = ubase[sl + 1] - ub;
+    if (sl == N - 1 && threadIdx.x == 0) seg_off[ubase[N]] = L;
+    if (len == 0) return;
+    uint32_t* const cur = us <= lds_cap ? lcur : gcur + ub;
+    const uint32_t* const keys = u_of_gi + l0;
+    for (uint32_t i = threadIdx.x; i < us; i += PLACE_THREADS) cur[i] = 0;
+    __syncthreads();
+    // (eight lookups per thread at a time, their loads in flight together: one workgroup streams the whole slot)
+    for (uint32_t i0 = threadIdx.x; i0 < len; i0 += PLACE_THREADS * PLACE_ITEMS) {
+        uint32_t k[PLACE_ITEMS];
+#pragma unroll
+        for (int j = 0; j < PLACE_ITEMS; j++) {
+            const uint32_t i = i0 + j * PLACE_THREADS;
+            k[j] = i < len ? (keys[i] & ~FIRST_BIT) - ub : 0xFFFFFFFFu;
+        }
+#pragma unroll
+        for (int j = 0; j < PLACE_ITEMS; j++)
+            if (k[j] != 0xFFFFFFFFu) atomicAdd(&cur[k[j]], 1u);
+    }
+    if (threadIdx.x == 0) carry_sh = l0;  // the lookups of the slots before come first
+    __syncthreads();
+    for (uint32_t i0 = 0; i0 < us; i0 += PLACE_THREADS) {
+        const uint32_t i = i0 + threadIdx.x;
+        const uint32_t cnt = i < us ? ld_relaxed(cur + i) : 0u;  // (counted by atomics: not through the L1 cache)
+        uint32_t total;
+        const uint32_t at = carry_sh + block_excl_scan<uint32_t, PLACE_THREADS / 64>(cnt, red, &total);
+        if (i < us) {
+            cur[i] = at;
+            seg_off[ub + i] = at;
+            if (cnt >= ORDER_HUGE)
+                huge_list[atomicAdd(&counts[2], 1u)] = ub + i;
+            else if (cnt >= ORDER_MID)
+                mid_list[atomicAdd(&counts[1], 1u)] = ub + i;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) carry_sh += total;
+        __syncthreads();
+    }
+    for (uint32_t i0 = threadIdx.x; i0 < len; i0 += PLACE_THREADS * PLACE_ITEMS) {
+        uint32_t k[PLACE_ITEMS];
+        uint64_t v[PLACE_ITEMS];
+#pragma unroll
+        for (int j = 0; j < PLACE_ITEMS; j++) {
+            const uint32_t i = i0 + j * PLACE_THREADS;
+            k[j] = i < len ? (keys[i] & ~FIRST_BIT) - ub : 0xFFFFFFFFu;
+            v[j] = i < len ? vals[l0 + i] : 0ull;
+        }
+#pragma unroll
+        for (int j = 0; j < PLACE_ITEMS; j++) {
+            if (k[j] == 0xFFFFFFFFu) continue;
+            const uint32_t at = atomicAdd(&cur[k[j]], 1u);
+            tkey[at] = ub + k[j];
+            tval[at] = v[j];
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void k_rank_short(uint32_t L, const uint32_t* __restrict__ tkey,
+                                                    const uint64_t* __restrict__ tval,
+                                                    const uint32_t* __restrict__ seg_off, uint64_t* __restrict__ svals,
+                                                    const DevStatus* status) {
     if (status->abort) return;
     const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < L; i += stride) {
-        const uint32_t k = skeys[i];
-        if (i == 0 || skeys[i - 1] != k) seg_off[k] = i;
-        if (i == L - 1) seg_off[status->n_unique] = L;
+    for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < L; t += stride) {
+        const uint32_t u = tkey[t];
+        const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
+        if (hi - lo >= ORDER_MID) continue;
+        const uint64_t v = tval[t];
+        uint32_t rank = 0;
+        for (uint32_t j = lo; j < hi; j++) {
+            const uint64_t o = tval[j];
+            rank += (o < v || (o == v && j < t)) ? 1u : 0u;
+        }
+        svals[lo + rank] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_rank_mid(const uint32_t* __restrict__ mid_list, const uint32_t* counts,
+                                                  const uint32_t* __restrict__ seg_off,
+                                                  const uint64_t* __restrict__ tval, uint64_t* __restrict__ svals,
+                                                  const DevStatus* status) {
+    __shared__ uint64_t seg[ORDER_HUGE];
+    if (status->abort) return;
+    const uint32_t n_mid = counts[1];
+    for (uint32_t k = blockIdx.x; k < n_mid; k += gridDim.x) {
+        const uint32_t u = mid_list[k];
+        const uint32_t lo = seg_off[u], n = seg_off[u + 1] - lo;  // ORDER_MID <= n < ORDER_HUGE
+        uint32_t p2 = ORDER_MID;
+        while (p2 < n) p2 <<= 1;
+        // bitonic sorting network over the segment padded with the largest value to a power of two
+        for (uint32_t i = threadIdx.x; i < p2; i += 256) seg[i] = i < n ? tval[lo + i] : ~0ull;
+        __syncthreads();
+        for (uint32_t size = 2; size <= p2; size <<= 1) {
+            for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+                for (uint32_t t = threadIdx.x; t < p2 / 2; t += 256) {
+                    const uint32_t a = 2 * t - (t & (stride - 1));  // lower element of the t-th pair
+                    const uint32_t b = a + stride;
+                    const bool up = (a & size) == 0;
+                    const uint64_t x = seg[a], y = seg[b];
+                    if ((x > y) == up) {
+                        seg[a] = y;
+                        seg[b] = x;
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        for (uint32_t i = threadIdx.x; i < n; i += 256) svals[lo + i] = seg[i];
+        __syncthreads();
+    }
+}
+
+// cnt: `batch` counters in LDS (in_lds) or in a part of gcnt of the workgroup's own.
+__global__ __launch_bounds__(256) void k_order_huge(const uint32_t* __restrict__ huge_list, const uint32_t* counts,
+                                                    const uint32_t* __restrict__ seg_off,
+                                                    const uint64_t* __restrict__ tval, uint64_t* __restrict__ svals,
+                                                    uint32_t batch, int in_lds, uint32_t* __restrict__ gcnt,
+                                                    const DevStatus* status) {
+    extern __shared__ uint32_t lcnt[];
+    __shared__ uint32_t red[4];
+    __shared__ uint32_t carry_sh;
+    if (status->abort) return;
+    uint32_t* const cnt = in_lds ? lcnt : gcnt + (size_t)blockIdx.x * batch;
+    const uint32_t n_huge = counts[2];
+    for (uint32_t k = blockIdx.x; k < n_huge; k += gridDim.x) {
+        const uint32_t u = huge_list[k];
+        const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
+        for (uint32_t i = threadIdx.x; i < batch; i += 256) cnt[i] = 0;
+        if (threadIdx.x == 0) carry_sh = 0;
+        __syncthreads();
+        for (uint32_t j = lo + threadIdx.x; j < hi; j += 256) atomicAdd(&cnt[(uint32_t)(tval[j] >> 32)], 1u);
+        __syncthreads();
+        for (uint32_t i0 = 0; i0 < batch; i0 += 256) {
+            const uint32_t i = i0 + threadIdx.x;
+            const uint32_t c = i < batch ? ld_relaxed(cnt + i) : 0u;
+            uint32_t total;
+            const uint32_t at = carry_sh + block_excl_scan_256<uint32_t>(c, red, &total);
+            if (i < batch) cnt[i] = at;
+            __syncthreads();
+            if (threadIdx.x == 0) carry_sh += total;
+            __syncthreads();
+        }
+        for (uint32_t j = lo + threadIdx.x; j < hi; j += 256) {
+            const uint64_t v = tval[j];
+            svals[lo + atomicAdd(&cnt[(uint32_t)(v >> 32)], 1u)] = v;
+        }
+        __syncthreads();
     }
 }
 

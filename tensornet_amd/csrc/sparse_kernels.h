@@ -133,13 +133,15 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
 // memory is device-accessible): cheaper than a copy command each.  The same
 // launch prepares the call's status block (STATUS_NEW_PLAN: everything cleared;
 // STATUS_REUSE_PLAN: a push on the last pull's plan keeps the counts and clears
-// the flags) and clears `zero[0 .. n_zero)`.
+// the flags), clears `zero[0 .. n_zero)` and copies copy_n words from copy_src to copy_dst.
 enum { STATUS_KEEP = 0, STATUS_NEW_PLAN = 1, STATUS_REUSE_PLAN = 2 };
 
 __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ host_src, uint32_t* __restrict__ dst_a,
                                                   uint32_t words_a, uint32_t* __restrict__ dst_b, uint32_t words_b,
                                                   DevStatus* status, int status_mode, uint32_t* __restrict__ zero,
-                                                  uint32_t n_zero, const DevStatus* plan_status) {
+                                                  uint32_t n_zero, const DevStatus* plan_status,
+                                                  const uint32_t* __restrict__ copy_src, uint32_t* __restrict__ copy_dst,
+                                                  uint32_t copy_n) {
     const uint32_t stride = gridDim.x * blockDim.x;
     const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;
     for (uint32_t i = tid; i < words_a + words_b; i += stride) {
@@ -149,6 +151,7 @@ __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ h
             dst_b[i - words_a] = host_src[i];
     }
     for (uint32_t i = tid; i < n_zero; i += stride) zero[i] = 0;
+    for (uint32_t i = tid; i < copy_n; i += stride) copy_dst[i] = copy_src[i];
     if (tid == 0 && status_mode != STATUS_KEEP) {
         // a push on the last pull's plan has a status block of its own: the plan's counts, fresh flags
         if (status_mode == STATUS_REUSE_PLAN && plan_status != status) *status = *plan_status;

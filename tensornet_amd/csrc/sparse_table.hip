@@ -18,11 +18,6 @@ static __device__ __align__(256) unsigned char scratch[TN_STATIC_SCRATCH_BYTES];
 
 namespace tn {
 
-// sort_pairs.hip
-int sort_pairs_temp_bytes(size_t n, int key_bits, size_t* bytes);
-int sort_pairs_u32_u64(void* temp, size_t temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
-                       const uint64_t* vals_in, uint64_t* vals_out, size_t n, int key_bits, hipStream_t st);
-
 namespace {
 
 constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:266
@@ -78,7 +73,8 @@ struct SparseTable {
     hipEvent_t stage_ev = nullptr;  // staging buffer free again
     hipEvent_t verify_ev = nullptr; // a push's comparison of the signs has been published
     DevBuf comb_buf;                // slot descriptors of a combine op
-    DevBuf pooled_ws;               // scratch of a push of pooled gradients (sort buffers, reduced rows)
+    DevBuf pooled_ws;               // scratch of a push of pooled gradients (ordered lookups, reduced rows)
+    size_t place_lds = 0, huge_lds = 0;  // dynamic LDS of k_place_lookups / k_order_huge on this device (0: not asked yet)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     // The slot descriptors of a call reach the device here while the caller's stream still runs the tail of the
@@ -417,6 +413,7 @@ struct Carver {
 struct Plan {
     SlotDesc* descs;
     SlotDesc* push_descs;  // descriptors of the push that reuses the plan (the pull's gather may still read `descs`)
+    uint32_t* push_ubase;  // ... and its copy of ubase, which its status is published from (the next pull rewrites ubase)
     uint32_t* lbase;
     uint32_t* ubase;
     uint64_t* vals_copy;   // signs of every lookup, concatenated
@@ -500,6 +497,7 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     p.push_descs = c.take<SlotDesc>(N);
     p.lbase = c.take<uint32_t>(N + 1);
     p.ubase = c.take<uint32_t>(N + 1);
+    p.push_ubase = c.take<uint32_t>(N + 1);
     p.vals_copy = c.take<uint64_t>(L);
     p.u_of_gi = c.take<uint32_t>(L);
     p.uniq_sign = c.take<uint64_t>(L);
@@ -619,7 +617,8 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
 // launch prepares the call's status block `ds` (status_mode) and clears `zero[0 .. n_zero)`.  It runs on `run_on`.
 int upload_slots(SparseTable* t, SlotDesc* dst_descs, uint32_t* dst_lbase, DevStatus* ds,
                  const std::vector<SlotDesc>& descs, const std::vector<uint32_t>& lbase, hipStream_t run_on,
-                 int status_mode, uint32_t* zero = nullptr, uint32_t n_zero = 0) {
+                 int status_mode, uint32_t* zero = nullptr, uint32_t n_zero = 0, const uint32_t* copy_src = nullptr,
+                 uint32_t* copy_dst = nullptr, uint32_t copy_n = 0) {
     if (t->stage_pending) {
         TN_HIP(hipEventSynchronize(t->stage_ev));
         t->stage_pending = false;
@@ -631,7 +630,7 @@ int upload_slots(SparseTable* t, SlotDesc* dst_descs, uint32_t* dst_lbase, DevSt
     TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)std::max<size_t>((db + lb) / 4, n_zero), 256, 64)), dim3(256),
               run_on, reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(dst_descs),
               (uint32_t)(db / 4), dst_lbase, (uint32_t)(lb / 4), ds, status_mode, zero, n_zero,
-              (const DevStatus*)t->dplan);
+              (const DevStatus*)t->dplan, copy_src, copy_dst, copy_n);
     TN_HIP(hipEventRecord(t->stage_ev, run_on));
     t->stage_pending = true;
     return TN_OK;
@@ -853,6 +852,22 @@ int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* d
         case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
         default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
     }
+}
+
+// Bytes of dynamic LDS a workgroup of `kernel` may have on this device (128 KB at most), after telling the
+// runtime that the kernel wants them.
+size_t big_lds_bytes_for(const void* kernel) {
+    int dev = 0, most = 0;
+    size_t bytes = 48 * 1024;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&most, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && most > 2048)
+        bytes = std::min<size_t>((size_t)most - 2048, 128 * 1024);  // (room for the kernel's static arrays)
+    if (bytes > 48 * 1024 &&
+        hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        bytes = 48 * 1024;
+    }
+    return bytes;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -1573,37 +1588,51 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     // to one row per distinct sign: stable sort of (distinct index, position) pairs, then one
     // ordered sum per distinct index.
     PushSrc src{};
+    const uint32_t* pub_ubase = nullptr;  // a push on the pull's plan publishes its own copy of the distinct counts
     auto prepare_src = [&]() -> int {
         src = op_source(p, grad_dim, pd);
         if (!pooled) return TN_OK;
-        int bits = 1;
-        while (bits < 32 && (1ull << bits) < L) bits++;
-        size_t temp_bytes = 0;
-        TN_TRY(sort_pairs_temp_bytes(L, bits, &temp_bytes));
+        if (!t->place_lds) {
+            t->place_lds = big_lds_bytes_for(reinterpret_cast<const void*>(k_place_lookups));
+            t->huge_lds = big_lds_bytes_for(reinterpret_cast<const void*>(k_order_huge));
+        }
+        const bool huge_in_lds = (size_t)batch * sizeof(uint32_t) <= t->huge_lds;
+        const int huge_grid = huge_in_lds ? GRID_CAP : 64;
         Carver c{nullptr};
-        uint32_t *long_list, *long_count, *keys, *skeys, *seg_off;
-        uint64_t *vals, *svals;
+        uint32_t *long_list, *long_count, *gcur, *seg_off, *tkey, *mid_list, *huge_list, *gcnt;
+        uint64_t *vals, *svals, *tval;
         float* flat;
-        char* temp;
         auto carve = [&](Carver& cv) {
-            long_count = cv.take<uint32_t>(1);
+            long_count = cv.take<uint32_t>(4);  // lists of k_reduce_pooled, k_place_lookups (mid, huge)
             long_list = cv.take<uint32_t>(L / LONG_SEGMENT + 1);
-            keys = cv.take<uint32_t>(L);
-            skeys = cv.take<uint32_t>(L);
+            mid_list = cv.take<uint32_t>(L / ORDER_MID + 1);
+            huge_list = cv.take<uint32_t>(L / ORDER_HUGE + 1);
+            gcur = cv.take<uint32_t>(L);
+            tkey = cv.take<uint32_t>(L);
             vals = cv.take<uint64_t>(L);
+            tval = cv.take<uint64_t>(L);
             svals = cv.take<uint64_t>(L);
             seg_off = cv.take<uint32_t>(L + 1);
             flat = cv.take<float>(L * (size_t)grad_dim);
-            temp = cv.take<char>(temp_bytes);
+            gcnt = cv.take<uint32_t>(huge_in_lds ? 0 : (size_t)huge_grid * (size_t)batch);
         };
         carve(c);
         TN_TRY(t->pooled_ws.ensure(align_up(c.off, 256)));
         Carver c2{(char*)t->pooled_ws.p};
         carve(c2);
-        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, pd, p.lbase, N, (uint32_t)L, p.u_of_gi, batch, keys,
-                  vals, ds, long_count);
-        TN_TRY(sort_pairs_u32_u64(temp, temp_bytes, keys, skeys, vals, svals, L, bits, st));
-        TN_LAUNCH(k_segment_starts, dim3(lblocks), dim3(256), st, skeys, (uint32_t)L, ds, seg_off);
+        TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, pd, p.lbase, N, (uint32_t)L, batch, vals, ds, long_count);
+        // The lookups of every distinct sign side by side, ascending by example (= by position): into their
+        // sign's segment first, then ordered inside it.
+        const uint32_t place_cap = (uint32_t)(t->place_lds / sizeof(uint32_t));
+        TN_LAUNCH_LDS(k_place_lookups, dim3(N), dim3(PLACE_THREADS), t->place_lds, st, p.lbase, p.ubase, N, (uint32_t)L,
+                      p.u_of_gi, vals, tkey, tval, seg_off, gcur, place_cap, mid_list, huge_list, long_count, ds);
+        TN_LAUNCH(k_rank_short, dim3(launch_grid(L, 256, GRID_CAP * 4)), dim3(256), st, (uint32_t)L, tkey, tval, seg_off,
+                  svals, ds);
+        TN_LAUNCH(k_rank_mid, dim3(launch_grid((int64_t)L / ORDER_MID + 1, 1, GRID_CAP * 2)), dim3(256), st, mid_list,
+                  long_count, seg_off, tval, svals, ds);
+        TN_LAUNCH_LDS(k_order_huge, dim3(launch_grid((int64_t)L / ORDER_HUGE + 1, 1, huge_grid)), dim3(256),
+                      huge_in_lds ? (size_t)batch * sizeof(uint32_t) : 0, st, huge_list, long_count, seg_off, tval, svals,
+                      (uint32_t)batch, huge_in_lds ? 1 : 0, gcnt, ds);
         // signs with LONG_SEGMENT lookups or more get a workgroup each instead of one thread group
         const int chunks = vec ? grad_dim / 4 : grad_dim;
         const uint32_t long_min = chunks <= 256 ? LONG_SEGMENT : 0xFFFFFFFFu;
@@ -1632,7 +1661,9 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // that gather (the plan's counts are final from ready_ev on)
         const bool hoist = behind_pull && !t->one_stream;
         if (hoist) TN_HIP(hipStreamWaitEvent(t->aux, t->ready_ev, 0));
-        TN_TRY(upload_slots(t, p.push_descs, nullptr, ds, descs, lbase, hoist ? t->aux : st, STATUS_REUSE_PLAN));
+        TN_TRY(upload_slots(t, p.push_descs, nullptr, ds, descs, lbase, hoist ? t->aux : st, STATUS_REUSE_PLAN, nullptr, 0,
+                            p.ubase, p.push_ubase, (uint32_t)(N + 1)));
+        pub_ubase = p.push_ubase;
         if (hoist) TN_HIP(hipStreamWaitEvent(st, t->stage_ev, 0));
         // On a plan with show counts the verify pass also sums the clicks; they start at zero
         // after the pull, a further push on the same plan clears them first.
@@ -1672,6 +1703,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // (its status cannot be waited for, a push only enqueues)
         t->plan_valid = false;
         ds = t->dplan;
+        pub_ubase = nullptr;
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
         carve_plan((char*)t->plan_buf.p, p, N, L);
         pd = p.descs;
@@ -1691,12 +1723,14 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         TN_HIP(hipEventRecord(t->apply_ev, st));
         TN_HIP(hipStreamWaitEvent(t->side, t->apply_ev, 0));
     }
-    TN_LAUNCH(k_publish, dim3(1), dim3(256), pub_on_side ? t->side : st, ds, p.ubase, (uint32_t)(N + 1),
-              reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr);
+    TN_LAUNCH(k_publish, dim3(1), dim3(256), pub_on_side ? t->side : st, ds, pub_ubase ? pub_ubase : p.ubase,
+              (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr);
     t->push_pending = true;
     t->push_pub_on_side = pub_on_side;
     t->push_slots = N;
-    if (reuse) {
+    // (the reduction of pooled gradients reads the plan's slot layout until the end of the call: nothing of the
+    // next pull may run beside it)
+    if (reuse && !pooled) {
         t->flow = FLOW_PUSH;
         t->flow_stream = st;
     }
@@ -1782,7 +1816,7 @@ int tn_sparse_table_combine_op(uint32_t table_handle, int N, const int64_t* cons
         TN_LAUNCH(k_stage_in, dim3(launch_grid((int64_t)(db + lb) / 4, 256, 64)), dim3(256), st,
                   reinterpret_cast<const uint32_t*>(t->hstage), reinterpret_cast<uint32_t*>(ddescs), (uint32_t)(db / 4),
                   dlbase, (uint32_t)(lb / 4), t->dstatus, (int)STATUS_NEW_PLAN, (uint32_t*)nullptr, 0u,
-                  (const DevStatus*)t->dstatus);
+                  (const DevStatus*)t->dstatus, (const uint32_t*)nullptr, (uint32_t*)nullptr, 0u);
         TN_HIP(hipEventRecord(t->stage_ev, st));
         t->stage_pending = true;
         // where the lookups of every example start, then one thread group per (slot, example)

@@ -33,3 +33,30 @@ def tn():
     import tensornet_amd.ops  # noqa: F401
 
     return tensornet_amd
+
+
+@pytest.fixture(autouse=True)
+def _free_sparse_tables(request):
+    """A sparse table keeps its HBM until the process ends (as the reference's tables keep their host
+    memory); with the default size that is 17 GB per table, and one test needs 176 GB for its own.  So
+    every GPU test gives back what the tables it created hold."""
+    if request.node.get_closest_marker("gpu") is None:
+        yield
+        return
+    import tensornet_amd.core as core
+
+    created = []
+    real = core.create_sparse_table
+
+    def tracking(*args, **kwargs):
+        h = real(*args, **kwargs)
+        created.append(h)
+        return h
+
+    core.create_sparse_table = tracking
+    try:
+        yield
+    finally:
+        core.create_sparse_table = real
+        for h in created:
+            core.clear_sparse_table(h)
