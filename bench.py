@@ -27,31 +27,29 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-# HBM bytes per launch (read + written) of the cfg3 kernels at 5e8 resident keys, from the rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs summarised in profiles/cfg3_adagrad_dim16_pull_push.md (FETCH_SIZE x 2.0 and
-# WRITE_SIZE x 1.0: the factors that make the counters reproduce the known traffic of the dense Adam stream).
-# Counters cannot be read from inside this script; the figures are refreshed together with that summary.
-MEASURED_TRAFFIC = {
-    "k_show_decay": 85646700000,
-    "k_reduce_pooled": 393500000,
-    "k_gather_vars": 372900000,
-    "k_combine_fwd": 356200000,
-    "k_apply_single": 341500000,
-    "k_reduce_long": 236600000,
-    "k_lds_dedup": 226800000,
-    "k_verify_values": 207500000,
-    "k_group_emit": 204200000,
-    "k_probe_recs": 191000000,
-    "k_lds_scatter": 165500000,
-    "k_lookup_keys": 123300000,
-    "k_apply_vec": 121300000,
-    "k_lds_hist": 100900000,
-    "k_apply_big": 91800000,
-    "k_lds_mapped": 86800000,
-    "k_group_count": 49000000,
-    "k_lds_flags": 20700000,
-    "k_lds_assign": 1100000,
-}
+# HBM bytes per launch (read + written) of the cfg3 kernels at 5e8 resident keys come from the rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs that `python3 -m tensornet_amd.profile_summary` condenses into this file beside
+# profiles/cfg3_adagrad_dim16_pull_push.md (counters cannot be read from inside this script).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "cfg3_traffic.json")
+# launched by a step, a few microseconds each, no traffic worth counting
+SMALL_STEP_KERNELS = ("k_stage_in", "k_publish", "k_lds_offsets", "k_init_new_recs", "k_group_offsets", "k_scan_tiles")
+
+
+def measured_traffic(step_kernels):
+    """{kernel: HBM bytes per launch} of the committed profile, its provenance, and a loud failure if a kernel the
+    step launches is not in it (the profile is older than the kernels: refresh it)."""
+    if not os.path.exists(TRAFFIC_FILE):
+        raise SystemExit("bench.py: %s is missing (python3 -m tensornet_amd.profile_summary writes it)" % TRAFFIC_FILE)
+    with open(TRAFFIC_FILE) as f:
+        t = json.load(f)
+    per_launch = t["bytes_per_launch"]
+    missing = sorted(k.split("<")[0] for k in step_kernels
+                     if k.split("<")[0] not in per_launch and not k.startswith(SMALL_STEP_KERNELS))
+    if missing:
+        raise SystemExit("bench.py: the step launches %s, which %s does not cover: refresh the profile "
+                         "(python3 -m tensornet_amd.profile_summary)" % (", ".join(missing), TRAFFIC_FILE))
+    return per_launch, {"file": os.path.relpath(TRAFFIC_FILE, ROOT), "profiled_at_commit": t.get("commit"),
+                        "fetch_factor": t.get("fetch_factor"), "write_factor": t.get("write_factor")}
 
 
 def state_bytes(opt, dim):
@@ -313,6 +311,10 @@ def main():
         log("  %-28s %5.1f launches/step %9.3f ms/step" % (k, c, ms))
     log("  sum of kernel time %.3f ms/step" % kernel_ms)
 
+    # measured HBM traffic of the dominant kernel: from the committed profile of this workload (none of the others)
+    traffic, traffic_source = (measured_traffic(per_step.keys()) if args.config == "cfg3" and resident == cfg["resident"]
+                               else (None, None))
+
     out = {
         "metric": "sparse pull+push keys/sec (dim16 AdaGrad); achieved HBM GB/s vs ~8 TB/s peak",
         "value": value,
@@ -331,6 +333,8 @@ def main():
                         "feature labels 1 on %.0f %% of the lookups"
                         % (args.config, cfg["batch"], cfg["slots"], cfg["lens"], cfg["zipf_s"], cfg["vocab"], dim,
                            opt_name, resident, 100 * synth.CLICK_RATE),
+            "optimizer": opt_name,
+            "dim": dim,
             "lookups_per_step": mean_L,
             "distinct_rows_per_step": mean_U,
             "globally_distinct_keys_of_a_batch": G0,
@@ -347,7 +351,8 @@ def main():
             "peak": HBM_PEAK / 1e9,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK,
-            "traffic": MEASURED_TRAFFIC.get(dname.split("<")[0]) if args.config == "cfg3" else None,
+            "traffic": traffic.get(dname.split("<")[0]) if traffic else None,
+            "traffic_source": traffic_source,
             "avg_launch_us": avg_launch_s * 1e6,
             "algorithmic_bytes_per_launch": dbytes,
         },
