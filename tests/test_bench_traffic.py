@@ -15,7 +15,7 @@ SHAPE = dict(L=5000000, U=2000000, G=1080000, G1=917000, Rm=550000, Gm=149000, R
 # side measurements of bench.py (combiner, ShowDecay, dense): profiled in the same runs, not part of the step
 SIDE = ("k_show_decay", "k_reduce_pooled", "k_reduce_long", "k_combine_fwd", "k_lookup_keys", "k_example_rowptr",
         "k_place_lookups", "k_rank_short", "k_rank_mid", "k_order_huge", "k_dense_adam_v4", "k_dense_adagrad_v4",
-        "k_probe", "k_load_rows", "k_export_rows", "k_finish_insert", "k_reset_status", "k_zero_f32")
+        "k_probe", "k_load_rows", "k_export_rows", "k_finish_insert", "k_reset_status", "k_zero_f32", "k_fill_f32")
 
 
 def test_traffic_file_names_known_kernels():
