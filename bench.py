@@ -188,6 +188,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
     ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
+    ap.add_argument("--no-fallback", action="store_true", help="skip the side measurement of a pull whose buckets overflow")
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -363,6 +364,49 @@ def main():
         "side_stream_kernels": [k for k in per_step if k.startswith(SIDE_STREAM_KERNELS)],
         "batch_shape": mean_shape,
     }
+
+    # ---- side measurement: a batch that overflows the buckets sized from the recent pulls ----------
+    # The second-level buckets follow the share of distinct records of the recent pulls.  A dozen pulls of a
+    # batch that repeats a thousand signs shrink them; the next ordinary batch then overflows, and its pull is
+    # repeated with buckets sized for a batch of distinct signs only.
+    if not args.no_fallback:
+        few = synth.splitmix64(np.arange(1, 1001, dtype=np.uint64)).view(np.int64)
+        frng = np.random.default_rng(5)
+        rep_values = [torch.from_numpy(few[frng.integers(0, len(few), v.numel())]).cuda() for v in batches[0][0]]
+        rep_vars = [torch.zeros((v.numel() + 1, dim), device="cuda") for v in rep_values]
+        rep_pull = tn.ops.BoundSparseTablePull(rep_vars, rep_values, h)
+        fresh = []
+        for b in (nb, nb + 1):
+            hb = synth.make_batch(cfg, b)
+            values = [torch.from_numpy(v).cuda() for v in hb]
+            labels = [torch.from_numpy(l).cuda() for l in synth.make_labels(hb, b)]
+            grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
+            vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
+            fresh.append((tn.ops.BoundSparseTablePull(vars_, values, h),
+                          tn.ops.BoundSparseTablePush(values, grads, labels, h)))
+        for _ in range(12):
+            rep_pull()
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        times = []
+        for pull, push in fresh:  # the first overflows and is redone, the second runs on worst-case buckets
+            t0 = time.perf_counter()
+            pull()
+            t1 = time.perf_counter()
+            push()
+            tn.ops.sparse_table_sync(h)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+            log("  pull %.3f ms, push %.3f ms" % ((t1 - t0) * 1e3, (time.perf_counter() - t1) * 1e3))
+        out["fallback_step"] = {
+            "what": "pull + push of an ordinary batch right after 12 pulls of a batch that repeats 1000 signs (buckets "
+                    "sized for those overflow; the pull is redone with buckets sized for distinct signs only), and of "
+                    "the batch after it; single steps, host waits included",
+            "overflowing_step_ms": times[0],
+            "step_after_ms": times[1],
+            "ordinary_step_ms": ms_per_step,
+        }
+        log("fallback: overflowing step %.3f ms, the step after %.3f ms (ordinary %.3f ms)" % (times[0], times[1], ms_per_step))
 
     # ---- side measurement: the combiner around the ops on the device ---------------
     # pull -> embedding_lookup_sparse (mean) -> push of the pooled gradients, same batches

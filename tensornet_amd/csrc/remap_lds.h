@@ -63,6 +63,12 @@ constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
 static_assert((uint64_t)LDS_MAX_SUB * LDS_BUCKET_TARGET <= 0xFFFFFFull && GRP_SLOTS <= 256,
               "a record's word holds the occurrences of a sign in its slot and the slot");
 
+// Raises DEV_ERR_REMAP_OVERFLOW.  A batch that overflows does so in a million places at once: atomics on the one
+// word would queue up for milliseconds, so only those that do not see the flag yet set it.
+__device__ __forceinline__ void flag_overflow(DevStatus* status) {
+    if (!(ld_relaxed(&status->err) & DEV_ERR_REMAP_OVERFLOW)) atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+}
+
 // A distinct (slot, sign) record on its way to the grouping.
 struct GroupRec {
     uint64_t sign;
@@ -151,7 +157,7 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
             if (local < span)
                 atomicAdd(&hist[local], 1u);
             else
-                atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+                flag_overflow(status);
         });
         __syncthreads();
         for (uint32_t i = threadIdx.x; i < span; i += 256)
@@ -309,7 +315,7 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                         h = (h + 1) & (LDS_TABLE - 1);
                     }
                     if (tries == LDS_TABLE) {  // table full: keep indices in bounds, let the host fall back
-                        atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+                        flag_overflow(status);
                         continue;
                     }
                 }
@@ -367,7 +373,7 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                 if (at < (uint32_t)GRP_CAP)
                     recs[(size_t)c * GRP_CAP + at] = r;
                 else
-                    atomicOr(&status->err, DEV_ERR_REMAP_OVERFLOW);
+                    flag_overflow(status);
             }
         }
         __syncthreads();

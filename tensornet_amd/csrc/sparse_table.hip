@@ -516,15 +516,19 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         // distinct records plus a quarter (GRP_CAP is the room of a bucket)
         const double expected = std::min(1.0, distinct_est * 1.25) * (double)L;
         w.nb2 = (uint32_t)std::max<size_t>(1, ((size_t)expected + GRP_TARGET - 1) / GRP_TARGET);
-        w.bcount = c.take<uint32_t>(dt_entries + 1 + w.nb2);  // zeroed together
+        // room for the buckets of a batch of distinct signs only: a call that overflows is repeated with that
+        // many, and must not pay for a larger buffer then (freeing and allocating waits for the whole device)
+        const size_t nb2_room = std::max<size_t>(w.nb2, (L + GRP_TARGET - 1) / GRP_TARGET);
+        const size_t nb1_room = std::max<size_t>(dt_entries, L / LDS_BUCKET_TARGET + MAX_SLOTS + 1);
+        w.bcount = c.take<uint32_t>(nb1_room + 1 + nb2_room);  // (the part in use is zeroed together)
         w.cursor2 = w.bcount + dt_entries + 1;
-        w.recs = c.take<GroupRec>((size_t)w.nb2 * GRP_CAP);
-        w.aux = c.take<uint2>((size_t)w.nb2 * GRP_CAP);
-        w.rrow = c.take<uint32_t>((size_t)w.nb2 * GRP_CAP);
-        w.bcounts = c.take<uint4>(w.nb2);
-        w.bbase = c.take<uint4>(w.nb2);
-        w.bstart = c.take<uint32_t>(dt_entries + 1);
-        w.bcursor = c.take<uint32_t>(dt_entries + 1);
+        w.recs = c.take<GroupRec>(nb2_room * GRP_CAP);
+        w.aux = c.take<uint2>(nb2_room * GRP_CAP);
+        w.rrow = c.take<uint32_t>(nb2_room * GRP_CAP);
+        w.bcounts = c.take<uint4>(nb2_room);
+        w.bbase = c.take<uint4>(nb2_room);
+        w.bstart = c.take<uint32_t>(nb1_room + 1);
+        w.bcursor = c.take<uint32_t>(nb1_room + 1);
         w.prec = c.take<ulonglong2>(L);
         w.first_of = c.take<uint32_t>(L);
         w.cnt_at = c.take<uint32_t>(L);
@@ -1408,7 +1412,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     // The remap through LDS needs the call's status on the host to fall back if a
     // bucket overflowed, so it is only used when the pull waits for its stream anyway.
     bool use_lds = !t->async_pull;
-    for (int attempt = 0; attempt < 2; attempt++) {
+    for (int attempt = 0; attempt < 3; attempt++) {
+        const double est_used = t->distinct_est;  // what this attempt's buckets are sized from
         std::vector<SlotDesc> descs;
         std::vector<uint32_t> lbase;
         size_t L = 0, dt_entries = 0;
@@ -1494,10 +1499,15 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             // rows the failed attempt inserted belong to signs of this batch; keep them counted
             t->hpull->st.err &= ~DEV_ERR_REMAP_OVERFLOW;
             harvest(t);
-            t->distinct_est = 1.0;  // the batch had more distinct records than the buckets were sized for
+            // The batch had more distinct records than the buckets were sized for (the share of the recent pulls
+            // plus a quarter).  Sized for a batch of distinct signs only, a bucket cannot overflow short of an
+            // adversarial hash (first level: 768 lookups for 2048 entries; second level: 1024 records expected
+            // in room for 1536), so the call is repeated through LDS once more -- at the cost of a pull, not of
+            // the global-table path, which remains for the batch that overflows even then.
+            if (est_used >= 1.0) use_lds = false;
+            t->distinct_est = 1.0;
             t->latched = TN_OK;
             t->latched_msg.clear();
-            use_lds = false;
             continue;
         }
         if (early) {
@@ -1509,7 +1519,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         }
         return sync_table(t, st);
     }
-    return fail(TN_ERR_HIP, "SparseTablePull: remap fell back twice");
+    return fail(TN_ERR_HIP, "SparseTablePull: remap fell back three times");
 }
 
 }  // extern "C"
