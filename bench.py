@@ -188,6 +188,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense Adam side measurement")
     ap.add_argument("--no-combiner", action="store_true", help="skip the combiner side measurement")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="leave roofline.traffic out (development runs on kernels newer than the committed profile)")
     ap.add_argument("--no-fallback", action="store_true", help="skip the side measurement of a pull whose buckets overflow")
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
     args = ap.parse_args()
@@ -313,7 +315,8 @@ def main():
     log("  sum of kernel time %.3f ms/step" % kernel_ms)
 
     # measured HBM traffic of the dominant kernel: from the committed profile of this workload (none of the others)
-    traffic, traffic_source = (measured_traffic(per_step.keys()) if args.config == "cfg3" and resident == cfg["resident"]
+    traffic, traffic_source = (measured_traffic(per_step.keys())
+                               if args.config == "cfg3" and resident == cfg["resident"] and not args.no_traffic
                                else (None, None))
 
     out = {
