@@ -795,6 +795,10 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
 // the arrays is first put together in LDS and then copied out in order; only where_u, indexed
 // by the distinct index of the record, stays a scattered store.  where_u[u] = {place in the member
 // list, table row of the record's sign (rrow, from k_probe_recs)}; the groups get the rows too.
+//
+// SLOT_RANKS: a record carries its rank in its slot instead of the position of its first occurrence
+// (the pull of a small batch); its distinct index is the slot's base plus that rank.
+template <bool SLOT_RANKS>
 __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6, 8))) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
@@ -806,7 +810,8 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                                                     uint32_t* __restrict__ big_list, Member* __restrict__ list,
                                                     uint2* __restrict__ where_u,
                                                     const uint32_t* __restrict__ rrow,
-                                                    uint32_t* __restrict__ grp_row, DevStatus* status) {
+                                                    uint32_t* __restrict__ grp_row, DevStatus* status,
+                                                    const uint32_t* __restrict__ ubase) {
     // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
     // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
     __shared__ Member s_list[GRP_CAP];
@@ -867,7 +872,8 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
         const uint32_t top = ids_cap - 1 - bb.z;         // member place of local member 0 of the several-record groups
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++)
-            if (j * EMIT_THREADS + threadIdx.x < n) us[j] = rank_of(flag8, wordpre, rs[j].gi);
+            if (j * EMIT_THREADS + threadIdx.x < n)
+                us[j] = SLOT_RANKS ? ubase[rs[j].cnt >> 24] + rs[j].gi : rank_of(flag8, wordpre, rs[j].gi);
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
             if (j * EMIT_THREADS + threadIdx.x >= n) continue;

@@ -1,0 +1,432 @@
+// Pull and push of a small batch (every slot fits one workgroup's LDS table): the same plan as the
+// path through two levels of buckets leaves, from far fewer launches.  A batch of a few thousand
+// lookups spends its time in the dependent launches of that path (about 3 us each, whatever the
+// kernel does), not in its kernels, so here
+//
+//   pull  k_small_slots   one workgroup per slot: per-slot first-occurrence remap in LDS
+//                         (sparse_table_ops.cc:115-137), lookup-or-insert of every distinct sign
+//                         (sparse_table.cc:52-66), its record handed to its second-level bucket;
+//                         the workgroup that finishes last adds up the slots' counts and publishes
+//                         the call's status to the host, which returns as soon as it sees it
+//         k_small_finish  rows into the variables (sparse_table_ops.cc:244-265), distinct indices
+//                         made global
+//         k_group_count, k_group_emit<true>   the groups of equal signs over all slots, as ever
+//   push  k_small_verify  slot descriptors in, comparison with the plan's signs, click sums
+//         k_apply_big (16 slots or more), k_small_apply   every group by one launch; its last
+//                         workgroup publishes the status
+//
+// Workgroups of one launch never wait for each other: a workgroup that needs the others' results is
+// the one that finishes last (a ticket counter tells), or runs in the next launch.
+#ifndef TN_SMALL_BATCH_H_
+#define TN_SMALL_BATCH_H_
+
+#include "remap_lds.h"
+
+namespace tn {
+
+constexpr int SMALL_THREADS = 1024;
+constexpr int SMALL_ITEMS = 4;                               // lookups per thread of k_small_slots
+constexpr int SMALL_SLOT_MAX = SMALL_THREADS * SMALL_ITEMS;  // lookups of a slot at most
+constexpr int SMALL_SLOTS = GRP_SLOTS;                       // slots at most (the grouping's slot masks)
+constexpr int SMALL_NB2_MAX = 512;                           // second-level buckets at most
+constexpr int SMALL_TILE = 1024;                             // lookups per workgroup of k_small_verify
+
+// What a slot's workgroup leaves for the one that finishes last.
+struct SlotOut {
+    uint32_t n_unique, n_new, err, pad;
+};
+
+// Persistent device state of the small path (zero when allocated).  A call uses one of the two sets of
+// bucket cursors and clears the other for the call after it; the ticket counters are set back to zero by
+// the workgroup that draws the last ticket.
+struct SmallState {
+    uint32_t cursor2[2][SMALL_NB2_MAX];
+    uint32_t done_pull, done_verify, done_apply, pad;
+    SlotOut slot_out[SMALL_SLOTS];
+};
+
+// Bytes of dynamic LDS of k_small_slots for a table of `entries` entries and nb2 second-level buckets.
+inline size_t small_slots_lds(uint32_t entries, uint32_t nb2) {
+    return ((size_t)entries + 1) * 16 + (size_t)nb2 * sizeof(uint32_t);
+}
+
+__device__ __forceinline__ void host_store(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// True in every thread of the workgroup that draws the last of `n` tickets.  Every thread of every workgroup of
+// the launch calls it once.  No fence: a release fence writes back the whole L2, which with a fence per
+// workgroup took several times as long as the kernels' work.  What the last workgroup reads of the others is
+// therefore written with device-scope atomics (they meet in memory, whatever the XCD) by the thread that draws
+// the ticket, which waits for them before it draws; a thread that raises an error flag elsewhere fences itself.
+__device__ __forceinline__ bool last_workgroup(uint32_t* counter, uint32_t n, uint32_t* sh_flag) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __builtin_amdgcn_s_waitcnt(0);  // this thread's atomics are done
+        const uint32_t ticket = atomicAdd(counter, 1u);
+        *sh_flag = ticket == n - 1 ? 1u : 0u;
+        if (ticket == n - 1) atomicExch(counter, 0u);  // nobody draws after the last
+    }
+    __syncthreads();
+    return *sh_flag != 0;
+}
+
+__device__ __forceinline__ void publish_word(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
+    const SlotDesc* host_descs, SlotDesc* descs, uint32_t* lbase, uint32_t* ubase, int N, uint32_t L, uint32_t entries,
+    Store s, OptDev o, uint64_t seed, uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ u_of_gi,
+    uint32_t* __restrict__ prow, uint32_t nb2, uint32_t* cursor2, uint32_t* cursor2_next, GroupRec* __restrict__ recs,
+    uint32_t* __restrict__ rrow, SmallState* state, DevStatus* status, uint32_t* host_dst, uint32_t* host_seq,
+    uint32_t seq) {
+    extern __shared__ unsigned long long smem64[];
+    unsigned long long* keys = smem64;  // entry `entries`: the sign EMPTY_KEY itself
+    uint32_t* minpos = reinterpret_cast<uint32_t*>(keys + entries + 1);
+    uint32_t* cnts = minpos + entries + 1;
+    uint32_t* hist2 = cnts + entries + 1;
+    __shared__ SlotDesc sd;
+    __shared__ uint32_t wsum[SMALL_THREADS / 64];
+    __shared__ uint32_t sh_new, sh_err, sh_last, sh_total;
+    const int sl = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+    // the slot's descriptor comes straight out of the host's staging buffer (one round trip over the bus,
+    // in flight while the tables are cleared)
+    if (tid < sizeof(SlotDesc) / 4)
+        reinterpret_cast<uint32_t*>(&sd)[tid] = reinterpret_cast<const uint32_t*>(host_descs + sl)[tid];
+    for (uint32_t i = tid; i <= entries; i += SMALL_THREADS) {
+        keys[i] = EMPTY_KEY;
+        minpos[i] = 0xFFFFFFFFu;
+        cnts[i] = 0;
+    }
+    for (uint32_t i = tid; i < nb2; i += SMALL_THREADS) hist2[i] = 0;
+    if (sl == 0)
+        for (uint32_t i = tid; i < (uint32_t)SMALL_NB2_MAX; i += SMALL_THREADS) cursor2_next[i] = 0;
+    if (tid == 0) {
+        sh_new = 0;
+        sh_err = 0;
+    }
+    __syncthreads();
+    const SlotDesc d = sd;
+    if (tid == 0) {
+        descs[sl] = d;
+        lbase[sl] = d.lbase;
+        if (sl == N - 1) lbase[N] = L;
+    }
+    const uint32_t n = d.len;
+    // a thread's lookups are consecutive: the ranks of its first occurrences are, too
+    uint64_t sg[SMALL_ITEMS];
+    uint32_t h[SMALL_ITEMS];
+    const uint32_t p0 = tid * SMALL_ITEMS;
+#pragma unroll
+    for (int j = 0; j < SMALL_ITEMS; j++) sg[j] = p0 + j < n ? (uint64_t)d.values[p0 + j] : 0;
+#pragma unroll
+    for (int j = 0; j < SMALL_ITEMS; j++) {
+        h[j] = entries;
+        if (p0 + j >= n) continue;
+        const uint64_t sign = sg[j];
+        if (sign != EMPTY_KEY) {
+            uint32_t e = (uint32_t)(mix64(sign) >> 7) & (entries - 1);
+            for (;;) {  // entries >= 2 n: a free entry exists
+                unsigned long long old = keys[e];
+                if (old == EMPTY_KEY) old = atomicCAS(&keys[e], (unsigned long long)EMPTY_KEY, sign);
+                if (old == EMPTY_KEY || old == sign) break;
+                e = (e + 1) & (entries - 1);
+            }
+            h[j] = e;
+        }
+        atomicMin(&minpos[h[j]], p0 + j);
+        atomicAdd(&cnts[h[j]], 1u);
+    }
+    __syncthreads();
+    uint32_t firsts = 0;
+#pragma unroll
+    for (int j = 0; j < SMALL_ITEMS; j++)
+        if (p0 + j < n && minpos[h[j]] == p0 + j) firsts |= 1u << j;
+    uint32_t total = 0;
+    uint32_t rank0 = block_excl_scan<uint32_t, SMALL_THREADS / 64>(__popc(firsts), wsum, &total);  // (barriers inside)
+    // the entry of a distinct sign now takes its rank in place of the position (every thread has read the positions)
+    uint32_t shows[SMALL_ITEMS];
+    {
+        uint32_t r = rank0;
+#pragma unroll
+        for (int j = 0; j < SMALL_ITEMS; j++) {
+            shows[j] = 0;
+            if (firsts & (1u << j)) {
+                shows[j] = cnts[h[j]];  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+                minpos[h[j]] = r++;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SMALL_ITEMS; j++) {
+        if (p0 + j >= n) continue;
+        const uint32_t r = minpos[h[j]];
+        d.mapped[p0 + j] = (int64_t)r;
+        vals_copy[d.lbase + p0 + j] = sg[j];
+        u_of_gi[d.lbase + p0 + j] = r | ((firsts & (1u << j)) ? FIRST_BIT : 0u);  // relative to the slot until k_small_finish
+    }
+    // lookup-or-insert of the distinct signs (optimizer_kernel.h:299-308); the thread that claims a free slot of
+    // the table fills the row.  The rows are read by the next launch only: another slot's workgroup may be
+    // filling the row of a sign that this one finds claimed.
+    uint32_t rows[SMALL_ITEMS], place[SMALL_ITEMS], bucket[SMALL_ITEMS];
+    uint32_t n_new = 0, err = 0;
+    {
+        uint32_t r = rank0;
+#pragma unroll
+        for (int j = 0; j < SMALL_ITEMS; j++) {
+            if (!(firsts & (1u << j))) continue;
+            bool is_new = false;
+            const uint32_t row = probe_slot<true>(s, sg[j], is_new);
+            if (row == NO_ROW) {
+                err |= DEV_ERR_TABLE_FULL;
+            } else if (is_new) {
+                init_row(s, o, seed, sg[j], row);
+                n_new++;
+            }
+            rows[j] = row;
+            prow[d.lbase + r] = row;
+            bucket[j] = group_bucket(sg[j], nb2);
+            place[j] = atomicAdd(&hist2[bucket[j]], 1u);
+            r++;
+        }
+    }
+    __syncthreads();
+    for (uint32_t b = tid; b < nb2; b += SMALL_THREADS) {
+        const uint32_t c = hist2[b];
+        hist2[b] = c ? atomicAdd(&cursor2[b], c) : 0u;  // this slot's slice of the bucket
+    }
+    __syncthreads();
+    {
+        uint32_t r = rank0;
+#pragma unroll
+        for (int j = 0; j < SMALL_ITEMS; j++) {
+            if (!(firsts & (1u << j))) continue;
+            const uint32_t at = hist2[bucket[j]] + place[j];
+            if (at < (uint32_t)GRP_CAP) {
+                GroupRec rec;
+                rec.sign = sg[j];
+                rec.gi = r;  // the record's rank in its slot (k_group_emit<true> adds the slot's base)
+                rec.cnt = shows[j] | ((uint32_t)sl << 24);
+                recs[(size_t)bucket[j] * GRP_CAP + at] = rec;
+                rrow[(size_t)bucket[j] * GRP_CAP + at] = rows[j];
+            } else {
+                err |= DEV_ERR_REMAP_OVERFLOW;  // the host repeats the call with more buckets
+            }
+            r++;
+        }
+    }
+    if (n_new) atomicAdd(&sh_new, n_new);
+    if (err) atomicOr(&sh_err, err);
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t* out = reinterpret_cast<uint32_t*>(&state->slot_out[sl]);
+        publish_word(out, total);
+        publish_word(out + 1, sh_new);
+        publish_word(out + 2, sh_err);
+    }
+    if (!last_workgroup(&state->done_pull, (uint32_t)N, &sh_last)) return;
+    // the last workgroup: bases of the slots' distinct indices, the call's status, both to the host
+    uint32_t mine = 0;
+    if (tid == 0) {
+        sh_new = 0;
+        sh_err = 0;
+    }
+    __syncthreads();
+    if (tid < (uint32_t)N) {
+        const uint32_t* so = reinterpret_cast<const uint32_t*>(&state->slot_out[tid]);
+        mine = ld_relaxed(so);
+        const uint32_t nn = ld_relaxed(so + 1), ee = ld_relaxed(so + 2);
+        if (nn) atomicAdd(&sh_new, nn);
+        if (ee) atomicOr(&sh_err, ee);
+    }
+    const uint32_t base = block_excl_scan<uint32_t, SMALL_THREADS / 64>(mine, wsum, &sh_total);
+    const uint32_t sw = sizeof(DevStatus) / 4;
+    if (tid < (uint32_t)N) {
+        ubase[tid] = base;
+        host_store(host_dst + sw + tid, base);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t U = sh_total;
+        ubase[N] = U;
+        host_store(host_dst + sw + N, U);
+        DevStatus st{};
+        st.err = sh_err;
+        st.n_unique = U;
+        st.n_new = sh_new;
+        st.gcap = U + U / 2 < 16 ? 16 : U + U / 2;
+        *status = st;
+        *s.count += sh_new;
+        const uint32_t* sp = reinterpret_cast<const uint32_t*>(&st);
+        for (uint32_t i = 0; i < sw; i++) host_store(host_dst + i, sp[i]);
+    }
+    __threadfence_system();
+    __syncthreads();
+    if (tid == 0) host_store(host_seq, seq);
+}
+
+// Second launch of a small pull: vars[slot][rank, :] = table row of the slot's distinct sign of that rank
+// (PopulatePulledVariable_, sparse_table_ops.cc:244-265), and the distinct indices of the lookups made
+// global (rank in the slot + base of the slot).  The ranks of a slot occupy the first positions of its
+// window of lookup positions.
+template <int VEC>
+__global__ __launch_bounds__(256) void k_small_finish(Store s, const SlotDesc* __restrict__ descs,
+                                                      const uint32_t* __restrict__ lbase,
+                                                      const uint32_t* __restrict__ ubase, int N, uint32_t L,
+                                                      const uint32_t* __restrict__ prow, uint32_t* __restrict__ u_of_gi) {
+    extern __shared__ uint32_t lb[];  // lb[N + 1], ub[N + 1]
+    uint32_t* ub = lb + N + 1;
+    for (int i = threadIdx.x; i <= N; i += 256) {
+        lb[i] = lbase[i];
+        ub[i] = ubase[i];
+    }
+    __syncthreads();
+    // one thread per (position, part of the row): few rows per thread would leave the rows' round trips in a queue
+    const uint32_t chunks = (uint32_t)(s.wdim / VEC);
+    const uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (uint64_t)L * chunks) return;
+    const uint32_t gi = (uint32_t)(t / chunks);
+    const uint32_t c = (uint32_t)(t - (uint64_t)gi * chunks);
+    const int sl = find_slot(lb, N, gi);
+    if (c == 0) u_of_gi[gi] += ub[sl];
+    const uint32_t r = gi - lb[sl];
+    if (r >= ub[sl + 1] - ub[sl]) return;  // beyond the slot's distinct signs
+    const SlotDesc& d = descs[sl];
+    if ((int64_t)r >= d.rows) return;      // the host reports the variable as too small
+    const uint32_t row = prow[gi];
+    if (row > s.cap) return;  // NO_ROW (table full): never address the table with it
+    if (VEC == 4) {
+        const float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);
+        *reinterpret_cast<float4*>(d.var + (uint64_t)r * s.wdim + c * 4) = v;
+    } else {
+        d.var[(uint64_t)r * s.wdim + c] = s.w[(uint64_t)row * s.wstride + c];
+    }
+}
+
+// First launch of a small push on the last pull's plan: the slot descriptors come in from the host's staging
+// buffer (every workgroup reads them into LDS, the first also leaves them in device memory for the
+// update kernels), the signs are compared with the plan's copy, and with CLICKS the non-zero labels are added to
+// the click sums of the member lists (sparse_table_ops.cc:283-296; a few thousand lookups do not queue up on
+// any entry).  The workgroup that finishes last tells the host that the comparison is done.
+template <bool CLICKS>
+__global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs, SlotDesc* push_descs,
+                                                      const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                      const uint64_t* __restrict__ vals_copy, DevStatus* status,
+                                                      const uint32_t* __restrict__ u_of_gi,
+                                                      const uint2* __restrict__ where_u, Member* list,
+                                                      SmallState* state, uint32_t* host_mismatch, uint32_t* host_seq,
+                                                      uint32_t seq) {
+    extern __shared__ unsigned long long vsm64[];  // the descriptors, then lb[N + 1]
+    uint32_t* vsm = reinterpret_cast<uint32_t*>(vsm64);
+    SlotDesc* sd = reinterpret_cast<SlotDesc*>(vsm64);
+    uint32_t* lb = vsm + (size_t)N * (sizeof(SlotDesc) / 4);
+    __shared__ uint32_t sh_last;
+    const uint32_t words = (uint32_t)N * (sizeof(SlotDesc) / 4);
+    for (uint32_t i = threadIdx.x; i < words; i += 256) vsm[i] = reinterpret_cast<const uint32_t*>(host_descs)[i];
+    for (int i = threadIdx.x; i <= N; i += 256) lb[i] = lbase[i];
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        status->err = 0;  // what the pull reported is on the host; the update kernels start from a clean slate
+        status->abort = 0;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0)
+        for (uint32_t i = threadIdx.x; i < words; i += 256) reinterpret_cast<uint32_t*>(push_descs)[i] = vsm[i];
+    const uint32_t g0 = blockIdx.x * SMALL_TILE;
+    const uint32_t g1 = min(L, g0 + (uint32_t)SMALL_TILE);
+    bool bad = false;
+    constexpr int PER = SMALL_TILE / 256;
+    uint64_t now[PER], then[PER];
+    int label[PER];
+    uint32_t u[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t gi = g0 + j * 256 + threadIdx.x;
+        now[j] = then[j] = 0;
+        label[j] = 0;
+        u[j] = 0;
+        if (gi < g1) {
+            const int sl = find_slot(lb, N, gi);
+            now[j] = (uint64_t)sd[sl].values[gi - lb[sl]];
+            then[j] = vals_copy[gi];
+            if (CLICKS) {
+                label[j] = (int)sd[sl].labels[gi - lb[sl]];
+                u[j] = u_of_gi[gi] & ~FIRST_BIT;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        bad |= now[j] != then[j];
+        if (CLICKS && label[j] != 0) atomicAdd(&list[where_u[u[j]].x].click, label[j]);
+    }
+    if (bad) {
+        atomicOr(&status->mismatch, 1u);
+        host_store(host_mismatch, 1u);
+        __threadfence_system();
+    }
+    if (!last_workgroup(&state->done_verify, gridDim.x, &sh_last)) return;
+    if (threadIdx.x == 0) host_store(host_seq, seq);
+}
+
+// What the update kernel of a small push does when its last workgroup is done: the call's status and the
+// slots' distinct bases to the host, the flags of the plan's status block back to zero (a further push on
+// the same plan starts from them).
+struct SmallPublish {
+    SmallState* state;
+    const uint32_t* ubase;
+    uint32_t n_ubase;
+    uint32_t* host_dst;
+    uint32_t* host_seq;
+    uint32_t seq;
+};
+
+__device__ __forceinline__ void small_publish(const SmallPublish& pub, DevStatus* status, uint32_t* sh_flag) {
+    if (!last_workgroup(&pub.state->done_apply, gridDim.x, sh_flag)) return;
+    const uint32_t sw = sizeof(DevStatus) / 4;
+    const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
+    for (uint32_t i = threadIdx.x; i < sw + pub.n_ubase; i += blockDim.x)
+        host_store(pub.host_dst + i, i < sw ? ld_relaxed(sp + i) : pub.ubase[i - sw]);
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        status->mismatch = 0;
+        status->err = 0;
+        host_store(pub.host_seq, pub.seq);
+    }
+}
+
+// Every group of the plan that k_apply_big does not take, one record or several, by one launch (the
+// lane groups of k_apply_vec); the last workgroup publishes the call's status.
+template <int KIND, int LPG>
+__global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                     const uint32_t* __restrict__ grp_row,
+                                                     const uint32_t* __restrict__ grp_off,
+                                                     const uint32_t* __restrict__ grp_cnt,
+                                                     const Member* __restrict__ list, uint32_t big_k,
+                                                     uint32_t ids_cap, SmallPublish pub) {
+    __shared__ uint32_t sh_flag;
+    // (a plan that turned out not to be this batch's: nothing to do but to say so)
+    if (!(status->mismatch | status->abort)) {
+        const uint32_t n_single = status->n_single, n_multi = status->n_multi;
+        const int sub = threadIdx.x % LPG;
+        const int lane0 = (int)__lane_id() - sub;
+        const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+        const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+        for (uint32_t t = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
+            const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
+            const uint32_t row = grp_row[g];
+            if (row == NO_ROW) continue;
+            const uint32_t k = grp_cnt[g];
+            if (is_big(k, big_k)) continue;
+            apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g], nullptr, sub, lane0, c1, c2);
+        }
+    }
+    small_publish(pub, status, &sh_flag);
+}
+
+}  // namespace tn
+
+#endif  // TN_SMALL_BATCH_H_

@@ -1459,29 +1459,11 @@ __global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc
 // per-element array; the next record's gradient is fetched while the current
 // one is applied.  Groups with big_k records or more are left to k_apply_big.
 template <int KIND, int LPG>
-__global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc src, DevStatus* status,
-                                                   const uint32_t* __restrict__ grp_row,
-                                                   const uint32_t* __restrict__ grp_off,
-                                                   const uint32_t* __restrict__ grp_cnt,
-                                                   const Member* __restrict__ list, uint32_t big_k,
-                                                   uint32_t ids_cap, const float* const* __restrict__ gaddr) {
-    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
-    if (status->mismatch | status->abort) return;
-    const uint32_t n_multi = status->n_multi;
+__device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o, const PushSrc& src, DevStatus* status,
+                                                uint32_t row, uint32_t k, const Member* mem, const float* const* ga,
+                                                int sub, int lane0, float c1, float c2) {
     const int D = s.D;
-    const int sub = threadIdx.x % LPG;                       // my float4 inside the row
-    const int lane = (int)__lane_id();
-    const int lane0 = lane - sub;                            // first lane of my group in the wavefront
-    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
-    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
-    for (uint32_t gi = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; gi < n_multi; gi += gstride) {
-        const uint32_t g = ids_cap - n_multi + gi;  // groups with several records sit at the top of the id space
-        const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
-        const uint32_t k = grp_cnt[g];
-        if (is_big(k, big_k)) continue;
-        const Member* mem = list + grp_off[g];
-        const float* const* ga = gaddr ? gaddr + grp_off[g] : nullptr;
+    {
         float* wp = s.w + (uint64_t)row * s.wstride;
         float* sp = s.st + (uint64_t)row * s.sstride;
         float4 w = reinterpret_cast<float4*>(wp)[sub];
@@ -1513,7 +1495,10 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                 if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
             }
             if (!ok) {
-                if (sub == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+                if (sub == 0) {
+                    atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+                    __threadfence();  // (k_small_apply publishes the status when its last workgroup is done)
+                }
                 continue;
             }
             any = true;
@@ -1551,7 +1536,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
                 ftrl_elem(o, gr.w, w.w, a.w, b.w);
             }
         }
-        if (!any) continue;
+        if (!any) return;
         reinterpret_cast<float4*>(wp)[sub] = w;
         if (KIND == OPT_ADAGRAD) {
             if (sub == 0) {
@@ -1566,6 +1551,31 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
             reinterpret_cast<float4*>(sp + D)[sub] = b;
             if (sub == 0) sp[2 * D + 1] = __int_as_float(delta_show);
         }
+    }
+}
+
+template <int KIND, int LPG>
+__global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                   const uint32_t* __restrict__ grp_row,
+                                                   const uint32_t* __restrict__ grp_off,
+                                                   const uint32_t* __restrict__ grp_cnt,
+                                                   const Member* __restrict__ list, uint32_t big_k,
+                                                   uint32_t ids_cap, const float* const* __restrict__ gaddr) {
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
+    const uint32_t n_multi = status->n_multi;
+    const int sub = threadIdx.x % LPG;                       // my float4 inside the row
+    const int lane0 = (int)__lane_id() - sub;                // first lane of my group in the wavefront
+    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+    for (uint32_t gi = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; gi < n_multi; gi += gstride) {
+        const uint32_t g = ids_cap - n_multi + gi;  // groups with several records sit at the top of the id space
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
+        const uint32_t k = grp_cnt[g];
+        if (is_big(k, big_k)) continue;
+        apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g], gaddr ? gaddr + grp_off[g] : nullptr, sub,
+                                   lane0, c1, c2);
     }
 }
 

@@ -3,8 +3,10 @@
 // and at operator level (core/kernels/sparse_table_ops.cc:170-265,317-368).
 #include "combine_kernels.h"
 #include "remap_lds.h"
+#include "small_batch.h"
 
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 
 // Device memory of tn_sparse_table_pull_static, the one entry point that allocates nothing: the call's
@@ -34,6 +36,10 @@ constexpr size_t ONE_STREAM_LOOKUPS = 3u << 20;
 constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to which no scan kernel runs between its launches
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
 constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS wins: it also takes fewer launches (cfg1, 8 k lookups: 0.154 -> 0.136 ms)
+
+// Up to this many lookups a batch whose slots each fit one workgroup (SMALL_SLOT_MAX lookups, SMALL_SLOTS slots)
+// takes the path of few launches (small_batch.h).
+constexpr size_t SMALL_MAX_LOOKUPS = 1u << 18;
 
 enum { FLOW_NONE = 0, FLOW_PULL = 1, FLOW_PUSH = 2 };
 
@@ -76,6 +82,15 @@ struct SparseTable {
     DevBuf comb_buf;                // slot descriptors of a combine op
     DevBuf pooled_ws;               // scratch of a push of pooled gradients (ordered lookups, reduced rows)
     size_t place_lds = 0, huge_lds = 0;  // dynamic LDS of k_place_lookups / k_order_huge on this device (0: not asked yet)
+    // The path of few launches for small batches: its device state, the words in pinned memory its kernels
+    // report through ([0] a pull's status is on the host, [1] a push's signs are compared, [2] a push's status
+    // is on the host) with the numbers the host expects there next, the dynamic LDS k_small_slots may have.
+    SmallState* small_state = nullptr;
+    uint32_t* hseq = nullptr;
+    uint32_t seq_pull = 0, seq_verify = 0, seq_apply = 0;
+    uint32_t small_calls = 0;  // (its parity: which set of bucket cursors the next small pull uses)
+    size_t small_lds = 0;
+    bool plan_small = false;   // the plan was left by a small pull: a push may take the small path, too
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     // The slot descriptors of a call reach the device here while the caller's stream still runs the tail of the
@@ -234,6 +249,10 @@ int ensure_side_buffers(SparseTable* t) {
     std::memset(t->hpull, 0, sizeof(HostStatus));
     std::memset(t->hpush, 0, sizeof(HostStatus));
     TN_HIP(hipHostMalloc((void**)&t->hcount, 64, hipHostMallocDefault));
+    TN_HIP(hipHostMalloc((void**)&t->hseq, 64, hipHostMallocDefault));
+    std::memset(t->hseq, 0, 64);
+    TN_HIP(hipMalloc((void**)&t->small_state, sizeof(SmallState)));
+    TN_HIP(hipMemset(t->small_state, 0, sizeof(SmallState)));
     t->hstage_bytes = (size_t)MAX_SLOTS * sizeof(SlotDesc) + (MAX_SLOTS + 1) * sizeof(uint32_t);
     TN_HIP(hipHostMalloc((void**)&t->hstage, t->hstage_bytes, hipHostMallocDefault));
     TN_HIP(hipEventCreateWithFlags(&t->stage_ev, hipEventDisableTiming));
@@ -523,15 +542,19 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     return align_up(c.off, 256);
 }
 
+// Second-level buckets of a batch of L lookups: GRP_TARGET records each on average if the batch has the
+// expected share of distinct records plus a quarter (GRP_CAP is the room of a bucket).
+uint32_t second_level_buckets(size_t L, double distinct_est) {
+    const double expected = std::min(1.0, distinct_est * 1.25) * (double)L;
+    return (uint32_t)std::max<size_t>(1, ((size_t)expected + GRP_TARGET - 1) / GRP_TARGET);
+}
+
 // dt_entries: entries of the global dedup table, or (use_lds) the number of buckets.
 size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds, double distinct_est = 1.0) {
     Carver c{base};
     if (use_lds) {
         w.nbuckets = (uint32_t)dt_entries;
-        // second-level buckets: GRP_TARGET records each on average if the batch has the expected share of
-        // distinct records plus a quarter (GRP_CAP is the room of a bucket)
-        const double expected = std::min(1.0, distinct_est * 1.25) * (double)L;
-        w.nb2 = (uint32_t)std::max<size_t>(1, ((size_t)expected + GRP_TARGET - 1) / GRP_TARGET);
+        w.nb2 = second_level_buckets(L, distinct_est);
         // room for the buckets of a batch of distinct signs only: a call that overflows is repeated with that
         // many, and must not pay for a larger buffer then (freeing and allocating waits for the whole device)
         const size_t nb2_room = std::max<size_t>(w.nb2, (L + GRP_TARGET - 1) / GRP_TARGET);
@@ -786,9 +809,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
             TN_HIP(hipStreamWaitEvent(st, t->join2_ev, 0));
         }
-        TN_LAUNCH(k_group_emit, dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
+        TN_LAUNCH((k_group_emit<false>), dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
                   own_offsets ? nullptr : w.bbase, w.bcounts, w.flag8, w.wordpre, L, big_threshold(s),
-                  p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds);
+                  p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds,
+                  (const uint32_t*)nullptr);
         return TN_OK;  // the rows were found beside the grouping
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
@@ -856,17 +880,20 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
     return TN_OK;
 }
 
+// Lanes that share a row in the update kernels (a float4 each), 0 if the rows cannot be handled that way.
+int lanes_per_group(const Store& s, bool vec_ok) {
+    if (!vec_ok || s.D % 4 != 0) return 0;
+    const int q = s.D / 4;
+    return (q >= 1 && q <= 32 && (q & (q - 1)) == 0) ? q : 0;
+}
+
 // Applies the grouped records; n_upper bounds the number of records.
 // addr_ready: p.gaddr already holds the gradient addresses of the multi-record groups' records.
 int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
                  hipStream_t st, bool addr_ready = false) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
-    int lpg = 0;
-    if (vec_ok && s.D % 4 == 0) {
-        int q = s.D / 4;
-        if (q >= 1 && q <= 32 && (q & (q - 1)) == 0) lpg = q;
-    }
+    const int lpg = lanes_per_group(s, vec_ok);
     switch (o.kind) {
         case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
         case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
@@ -874,14 +901,51 @@ int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* d
     }
 }
 
+// The updates of a small push: the signs with many records by k_apply_big (a sign has at most one record per
+// slot, so there are none below BIG_GROUP slots), every other group by one launch of k_small_apply, whose last
+// workgroup publishes the call's status.
+template <int KIND>
+int launch_small_apply_kind(SparseTable* t, int lpg, int N, const OptDev& o, const PushSrc& src, DevStatus* ds,
+                            const Plan& p, int64_t n_upper, hipStream_t st, const SmallPublish& pub) {
+    const Store& s = t->store;
+    const uint32_t big_k = big_threshold(s);
+    if (big_k != 0xFFFFFFFFu && (uint32_t)N >= big_k)
+        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
+                      big_lds_bytes(s.D), st, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list,
+                      big_gbuf_floats(s.D), (const float* const*)nullptr);
+#define TN_LAUNCH_SMALL(LPG)                                                                                          \
+    TN_LAUNCH((k_small_apply<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, o, src, \
+              ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, (uint32_t)n_upper, pub)
+    switch (lpg) {
+        case 1: TN_LAUNCH_SMALL(1); break;
+        case 2: TN_LAUNCH_SMALL(2); break;
+        case 4: TN_LAUNCH_SMALL(4); break;
+        case 8: TN_LAUNCH_SMALL(8); break;
+        case 16: TN_LAUNCH_SMALL(16); break;
+        default: TN_LAUNCH_SMALL(32); break;
+    }
+#undef TN_LAUNCH_SMALL
+    return TN_OK;
+}
+
+int launch_small_apply(SparseTable* t, int lpg, int N, const PushSrc& src, DevStatus* ds, const Plan& p, int64_t n_upper,
+                       hipStream_t st, const SmallPublish& pub) {
+    const OptDev o = make_optdev(t);
+    switch (o.kind) {
+        case OPT_ADAGRAD: return launch_small_apply_kind<OPT_ADAGRAD>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
+        case OPT_ADAM: return launch_small_apply_kind<OPT_ADAM>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
+        default: return launch_small_apply_kind<OPT_FTRL>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
+    }
+}
+
 // Bytes of dynamic LDS a workgroup of `kernel` may have on this device (128 KB at most), after telling the
 // runtime that the kernel wants them.
-size_t big_lds_bytes_for(const void* kernel) {
+size_t big_lds_bytes_for(const void* kernel, size_t cap = 128 * 1024) {
     int dev = 0, most = 0;
     size_t bytes = 48 * 1024;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&most, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && most > 2048)
-        bytes = std::min<size_t>((size_t)most - 2048, 128 * 1024);  // (room for the kernel's static arrays)
+        bytes = std::min<size_t>((size_t)most - 2048, cap);  // (room for the kernel's static arrays)
     if (bytes > 48 * 1024 &&
         hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -891,6 +955,43 @@ size_t big_lds_bytes_for(const void* kernel) {
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Entries of the LDS table of k_small_slots for slots of at most max_len lookups (load <= 0.5).
+uint32_t small_entries(size_t max_len) {
+    uint32_t e = 64;
+    while ((size_t)e < 2 * max_len) e *= 2;
+    return e;
+}
+
+// Does the batch qualify for the path of few launches?  (nb2: its second-level buckets.)
+bool small_batch_fits(SparseTable* t, int N, const int64_t* lens, size_t L, uint32_t nb2) {
+    if (t->async_pull || N > SMALL_SLOTS || L == 0 || L > SMALL_MAX_LOOKUPS || nb2 > (uint32_t)SMALL_NB2_MAX) return false;
+    size_t max_len = 0;
+    for (int s = 0; s < N; s++) max_len = std::max<size_t>(max_len, (size_t)lens[s]);
+    if (max_len > (size_t)SMALL_SLOT_MAX) return false;
+    if (!t->small_lds)
+        t->small_lds = big_lds_bytes_for(reinterpret_cast<const void*>(k_small_slots),
+                                         small_slots_lds(small_entries(SMALL_SLOT_MAX), SMALL_NB2_MAX));
+    return small_slots_lds(small_entries(max_len), nb2) <= t->small_lds;
+}
+
+// Waits for a kernel of the small path to report through pinned memory: *flag == want.  The word is polled for a
+// while (it arrives a few microseconds after the kernel's end, well before a wait on the stream or on an event
+// returns), then the stream is waited for, which also brings a failed launch to light.
+int wait_reported(const uint32_t* flag, uint32_t want, hipStream_t st, const char* what) {
+    const volatile uint32_t* f = flag;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+        for (int i = 0; i < 256; i++) {
+            if (*f == want) return TN_OK;
+            __builtin_ia32_pause();
+        }
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) break;
+    }
+    TN_HIP(hipStreamSynchronize(st));
+    if (*f != want) return fail(TN_ERR_HIP, std::string(what) + ": the device did not report");
+    return TN_OK;
+}
 
 }  // namespace
 }  // namespace tn
@@ -1428,6 +1529,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     // The remap through LDS needs the call's status on the host to fall back if a
     // bucket overflowed, so it is only used when the pull waits for its stream anyway.
     bool use_lds = !t->async_pull;
+    bool small_allowed = true;
     for (int attempt = 0; attempt < 3; attempt++) {
         const double est_used = t->distinct_est;  // what this attempt's buckets are sized from
         std::vector<SlotDesc> descs;
@@ -1452,14 +1554,84 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         }
         t->one_stream = L < ONE_STREAM_LOOKUPS;
         TN_TRY(ensure_room(t, (uint64_t)L, st));
+        // a batch whose slots each fit one workgroup takes the path of few launches (small_batch.h)
+        const bool small = small_allowed && small_batch_fits(t, N, value_lens, L, second_level_buckets(L, t->distinct_est));
+        const bool lds_scratch = use_lds || small;
+        if (small) dt_entries = 1;  // no first-level buckets
         Plan p{};
         Scratch w{};
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
         carve_plan((char*)t->plan_buf.p, p, N, L);
-        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, use_lds, t->distinct_est)));
-        carve_scratch((char*)t->ws.p, w, L, dt_entries, use_lds, t->distinct_est);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, lds_scratch, t->distinct_est)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries, lds_scratch, t->distinct_est);
         w.span_cap = span_cap;
         t->plan_valid = false;
+        if (small) {
+            if (t->stage_pending) {
+                TN_HIP(hipEventSynchronize(t->stage_ev));
+                t->stage_pending = false;
+            }
+            std::memcpy(t->hstage, descs.data(), descs.size() * sizeof(SlotDesc));
+            size_t max_len = 0;
+            for (int s = 0; s < N; s++) max_len = std::max<size_t>(max_len, (size_t)value_lens[s]);
+            const uint32_t entries = small_entries(max_len);
+            const uint32_t set = t->small_calls++ & 1u;
+            uint32_t* cur = t->small_state->cursor2[set];
+            uint32_t* next = t->small_state->cursor2[set ^ 1u];
+            const uint32_t seq = ++t->seq_pull;
+            const Store& s = t->store;
+            DevStatus* ds = t->dplan;
+            uint32_t* prow = w.first_of;  // row of the slot's distinct sign of rank r at [first lookup of the slot + r]
+            TN_LAUNCH_LDS(k_small_slots, dim3(N), dim3(SMALL_THREADS), small_slots_lds(entries, w.nb2), st,
+                          reinterpret_cast<const SlotDesc*>(t->hstage), p.descs, p.lbase, p.ubase, N, (uint32_t)L, entries, s,
+                          make_optdev(t), t->seed, p.vals_copy, p.u_of_gi, prow, w.nb2, cur, next, w.recs, w.rrow,
+                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
+            const size_t base_lds = 2 * ((size_t)N + 1) * sizeof(uint32_t);
+            const int tiles = (int)(((uint64_t)L * (uint64_t)(vec ? wdim / 4 : wdim) + 255) / 256);
+            if (vec)
+                TN_LAUNCH_LDS((k_small_finish<4>), dim3(tiles), dim3(256), base_lds, st, s, p.descs, p.lbase, p.ubase, N,
+                              (uint32_t)L, prow, p.u_of_gi);
+            else
+                TN_LAUNCH_LDS((k_small_finish<1>), dim3(tiles), dim3(256), base_lds, st, s, p.descs, p.lbase, p.ubase, N,
+                              (uint32_t)L, prow, p.u_of_gi);
+            const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
+            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs, big_threshold(s), w.aux,
+                      w.bcounts);
+            TN_LAUNCH((k_group_emit<true>), dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
+                      (const uint4*)nullptr, w.bcounts, (const uint8_t*)nullptr, (const uint32_t*)nullptr, (uint32_t)L,
+                      big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
+                      p.grp_row, ds, p.ubase);
+            TN_HIP(hipGetLastError());
+            // the call returns when the first launch has reported: what follows it is complete in stream order
+            TN_HIP(hipEventRecord(t->tail_ev, st));
+            t->tail_recorded = true;
+            t->pull_pending = true;
+            t->pull_slots = N;
+            t->pull_lookups = (uint64_t)L;
+            t->pending_rows.assign(var_rows, var_rows + N);
+            t->plan_valid = true;
+            t->plan_small = true;
+            t->plan_clicks_dirty = false;
+            t->plan_has_show = true;
+            t->plan_N = N;
+            t->plan_lens.assign(value_lens, value_lens + N);
+            t->plan_epoch = t->epoch;
+            TN_TRY(wait_reported(t->hseq + 0, seq, st, "SparseTablePull"));
+            if (t->hpull->st.err & DEV_ERR_REMAP_OVERFLOW) {
+                // a second-level bucket overflowed (more distinct records than the recent pulls had): once more
+                // with buckets for a batch of distinct signs only, then on the other paths
+                t->hpull->st.err &= ~DEV_ERR_REMAP_OVERFLOW;
+                harvest(t);
+                if (est_used >= 1.0) small_allowed = false;
+                t->distinct_est = 1.0;
+                t->latched = TN_OK;
+                t->latched_msg.clear();
+                continue;
+            }
+            harvest(t);
+            return take_latched(t);
+        }
+        t->plan_small = false;
         // Behind a push of the training loop the descriptors go in on the auxiliary stream, beside that push's
         // updates: those read the push's own descriptors and status block, and nothing of the scratch buffer.
         // (Same slot count: the arrays at the head of the plan buffer keep their places.)
@@ -1680,7 +1852,56 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         src.flat = flat;
         return TN_OK;
     };
-    if (reuse) {
+    const int small_lpg = lanes_per_group(t->store, vec && t->store.wstride % 4 == 0);
+    if (reuse && t->plan_small && !pooled && small_lpg != 0 && N <= SMALL_SLOTS) {
+        // A small batch on the plan of its small pull: slot descriptors, comparison of the signs and click sums by
+        // one launch, the updates by one or two more, which also publish the status (small_batch.h).  The call's
+        // status block is the plan's: nothing of the next call runs beside this one.
+        carve_plan((char*)t->plan_buf.p, p, N, L);
+        pd = p.push_descs;
+        ds = t->dplan;
+        if (t->stage_pending) {
+            TN_HIP(hipEventSynchronize(t->stage_ev));
+            t->stage_pending = false;
+        }
+        std::memcpy(t->hstage, descs.data(), descs.size() * sizeof(SlotDesc));
+        t->hpush->st.mismatch = 0;
+        const bool clicks = with_click;  // (a small pull's plan has the show counts)
+        if (clicks) {
+            if (t->plan_clicks_dirty)
+                TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
+            t->plan_clicks_dirty = true;
+        }
+        const uint32_t seq_v = ++t->seq_verify, seq_a = ++t->seq_apply;
+        const int tiles = (int)((L + SMALL_TILE - 1) / SMALL_TILE);
+        const size_t vlds = (size_t)N * sizeof(SlotDesc) + ((size_t)N + 1) * sizeof(uint32_t);
+        if (clicks)
+            TN_LAUNCH_LDS((k_small_verify<true>), dim3(tiles), dim3(256), vlds, st,
+                          reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
+                          ds, p.u_of_gi, p.where_u, p.list, t->small_state, &t->hpush->st.mismatch, t->hseq + 1, seq_v);
+        else
+            TN_LAUNCH_LDS((k_small_verify<false>), dim3(tiles), dim3(256), vlds, st,
+                          reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
+                          ds, p.u_of_gi, p.where_u, p.list, t->small_state, &t->hpush->st.mismatch, t->hseq + 1, seq_v);
+        SmallPublish pub{};
+        pub.state = t->small_state;
+        pub.ubase = p.ubase;
+        pub.n_ubase = (uint32_t)(N + 1);
+        pub.host_dst = reinterpret_cast<uint32_t*>(t->hpush);
+        pub.host_seq = t->hseq + 2;
+        pub.seq = seq_a;
+        TN_TRY(launch_small_apply(t, small_lpg, N, op_source(p, grad_dim, pd), ds, p, (int64_t)L, st, pub));
+        TN_HIP(hipGetLastError());
+        // the outcome of the comparison: the updates are queued behind it and do nothing on a mismatch
+        TN_TRY(wait_reported(t->hseq + 1, seq_v, st, "SparseTablePush"));
+        if (t->hpush->st.mismatch == 0) {
+            t->push_pending = true;
+            t->push_pub_on_side = false;
+            t->push_slots = N;
+            return TN_OK;
+        }
+        reuse = false;  // another batch than the last pull's: analysed below
+    } else if (reuse) {
         carve_plan((char*)t->plan_buf.p, p, N, L);
         pd = p.push_descs;
         // behind a pull that returned before its gather the descriptors go in on the auxiliary stream, beside
