@@ -751,8 +751,27 @@ __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t
     }
 }
 
-// Fills the rows k_probe_recs inserted (the row initialiser of init_row): one lane per pair of elements, the
-// first lane of a row also its padding columns and optimizer state.
+// Elements 2 q and 2 q + 1 of a new row (the row initialiser of init_row, spread over lanes); with q == 0 also
+// the row's padding columns and optimizer state.
+__device__ __forceinline__ void init_row_pair(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row,
+                                              uint32_t q, float stddev) {
+    float* w = s.w + row * s.wstride;
+    const int c = 2 * (int)q;
+    float2 z = make_float2(0.f, 0.f);
+    if (!o.zero_init) {
+        z = normal_pair(rnd64(seed, sign, (uint64_t)q));
+        z.x = (z.x * stddev) * o.initial_scale;
+        z.y = (z.y * stddev) * o.initial_scale;
+    }
+    w[c] = z.x;
+    if (c + 1 < s.D) w[c + 1] = z.y;
+    if (q == 0) {
+        for (int e = s.D; e < s.wlen; e++) w[e] = 0.f;  // cvm columns / padding
+        init_state(s, o, s.st + row * s.sstride);
+    }
+}
+
+// Fills the rows k_probe_recs inserted: one lane per pair of elements.
 __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64_t seed,
                                                        const GroupRec* __restrict__ recs,
                                                        const uint32_t* __restrict__ rrow,
@@ -765,22 +784,7 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
     for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
         const uint32_t j = (uint32_t)(t / pairs), q = (uint32_t)(t - (uint64_t)j * pairs);
         const uint32_t i = newlist[j];
-        const uint64_t sign = recs[i].sign;
-        const uint64_t row = rrow[i];
-        float* w = s.w + row * s.wstride;
-        const int c = 2 * (int)q;
-        float2 z = make_float2(0.f, 0.f);
-        if (!o.zero_init) {
-            z = normal_pair(rnd64(seed, sign, (uint64_t)q));
-            z.x = (z.x * stddev) * o.initial_scale;
-            z.y = (z.y * stddev) * o.initial_scale;
-        }
-        w[c] = z.x;
-        if (c + 1 < s.D) w[c + 1] = z.y;
-        if (q == 0) {
-            for (int e = s.D; e < s.wlen; e++) w[e] = 0.f;  // cvm columns / padding
-            init_state(s, o, s.st + row * s.sstride);
-        }
+        init_row_pair(s, o, seed, recs[i].sign, rrow[i], q, stddev);
     }
 }
 

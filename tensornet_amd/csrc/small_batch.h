@@ -121,23 +121,40 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     const uint32_t p0 = tid * SMALL_ITEMS;
 #pragma unroll
     for (int j = 0; j < SMALL_ITEMS; j++) sg[j] = p0 + j < n ? (uint64_t)d.values[p0 + j] : 0;
+    const int lane = (int)(tid & 63);
 #pragma unroll
     for (int j = 0; j < SMALL_ITEMS; j++) {
         h[j] = entries;
-        if (p0 + j >= n) continue;
+        const bool valid = p0 + j < n;
         const uint64_t sign = sg[j];
-        if (sign != EMPTY_KEY) {
-            uint32_t e = (uint32_t)(mix64(sign) >> 7) & (entries - 1);
-            for (;;) {  // entries >= 2 n: a free entry exists
-                unsigned long long old = keys[e];
-                if (old == EMPTY_KEY) old = atomicCAS(&keys[e], (unsigned long long)EMPTY_KEY, sign);
-                if (old == EMPTY_KEY || old == sign) break;
-                e = (e + 1) & (entries - 1);
+        // A frequent sign fills whole wavefronts: the lanes that hold the same sign as the first valid lane let
+        // that lane (the lowest position among them) enter it with their number, instead of queueing up on
+        // one LDS address, and take its entry from it.
+        const unsigned long long vmask = __ballot(valid);
+        if (vmask == 0) continue;
+        const int leader = __ffsll((long long)vmask) - 1;
+        const uint64_t lead_sign = ((uint64_t)(uint32_t)__shfl((int)(sign >> 32), leader) << 32) |
+                                   (uint32_t)__shfl((int)(uint32_t)sign, leader);
+        const bool same = valid && sign == lead_sign;
+        const unsigned long long smask = __ballot(same);
+        const bool pooled = __popcll(smask) >= 8;
+        const bool follower = pooled && same && lane != leader;
+        if (valid && !follower) {
+            if (sign != EMPTY_KEY) {
+                uint32_t e = (uint32_t)(mix64(sign) >> 7) & (entries - 1);
+                for (;;) {  // entries >= 2 n: a free entry exists
+                    unsigned long long old = keys[e];
+                    if (old == EMPTY_KEY) old = atomicCAS(&keys[e], (unsigned long long)EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                    e = (e + 1) & (entries - 1);
+                }
+                h[j] = e;
             }
-            h[j] = e;
+            atomicMin(&minpos[h[j]], p0 + j);
+            atomicAdd(&cnts[h[j]], pooled && lane == leader ? (uint32_t)__popcll(smask) : 1u);
         }
-        atomicMin(&minpos[h[j]], p0 + j);
-        atomicAdd(&cnts[h[j]], 1u);
+        const uint32_t lead_h = (uint32_t)__shfl((int)h[j], leader);
+        if (follower) h[j] = lead_h;
     }
     __syncthreads();
     uint32_t firsts = 0;
@@ -168,23 +185,41 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
         vals_copy[d.lbase + p0 + j] = sg[j];
         u_of_gi[d.lbase + p0 + j] = r | ((firsts & (1u << j)) ? FIRST_BIT : 0u);  // relative to the slot until k_small_finish
     }
-    // lookup-or-insert of the distinct signs (optimizer_kernel.h:299-308); the thread that claims a free slot of
-    // the table fills the row.  The rows are read by the next launch only: another slot's workgroup may be
+    // lookup-or-insert of the distinct signs (optimizer_kernel.h:299-308), the first key groups of a thread's
+    // signs in flight together.  A row this workgroup inserts is listed in LDS (the key table is dead) and filled
+    // further down by all threads: one lane of a wavefront drawing the normal deviates of a row would hold up
+    // the other sixty-three.  The rows are read by the next launch only: another slot's workgroup may be
     // filling the row of a sign that this one finds claimed.
+    unsigned long long* new_sign = keys;                                   // [n] at most
+    uint32_t* new_row = reinterpret_cast<uint32_t*>(keys + n);            // (the table has 2 n + 1 entries or more)
     uint32_t rows[SMALL_ITEMS], place[SMALL_ITEMS], bucket[SMALL_ITEMS];
-    uint32_t n_new = 0, err = 0;
+    uint32_t err = 0;
     {
+        uint64_t at[SMALL_ITEMS];
+        ulonglong2 q[SMALL_ITEMS][4];
+#pragma unroll
+        for (int j = 0; j < SMALL_ITEMS; j++) {
+            at[j] = 0;
+            if ((firsts & (1u << j)) && sg[j] != EMPTY_KEY) {
+                at[j] = home_group(sg[j], s.cap);
+                const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + at[j]);
+                q[j][0] = g[0], q[j][1] = g[1], q[j][2] = g[2], q[j][3] = g[3];
+            }
+        }
         uint32_t r = rank0;
 #pragma unroll
         for (int j = 0; j < SMALL_ITEMS; j++) {
             if (!(firsts & (1u << j))) continue;
             bool is_new = false;
-            const uint32_t row = probe_slot<true>(s, sg[j], is_new);
+            const uint32_t row = sg[j] == EMPTY_KEY
+                                     ? probe_slot<true>(s, sg[j], is_new)
+                                     : probe_from<true>(s, sg[j], at[j], q[j][0], q[j][1], q[j][2], q[j][3], is_new);
             if (row == NO_ROW) {
                 err |= DEV_ERR_TABLE_FULL;
             } else if (is_new) {
-                init_row(s, o, seed, sg[j], row);
-                n_new++;
+                const uint32_t k = atomicAdd(&sh_new, 1u);
+                new_sign[k] = sg[j];
+                new_row[k] = row;
             }
             rows[j] = row;
             prow[d.lbase + r] = row;
@@ -197,6 +232,16 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     for (uint32_t b = tid; b < nb2; b += SMALL_THREADS) {
         const uint32_t c = hist2[b];
         hist2[b] = c ? atomicAdd(&cursor2[b], c) : 0u;  // this slot's slice of the bucket
+    }
+    {
+        // the new rows (row initialiser of init_row): a thread per pair of elements
+        const uint32_t pairs = (uint32_t)(s.D + 1) / 2;
+        const uint32_t work = sh_new * pairs;
+        const float stddev = (float)(1.0 / sqrt((double)s.D));
+        for (uint32_t t = tid; t < work; t += SMALL_THREADS) {
+            const uint32_t k = t / pairs;
+            init_row_pair(s, o, seed, (uint64_t)new_sign[k], new_row[k], t - k * pairs, stddev);
+        }
     }
     __syncthreads();
     {
@@ -218,7 +263,6 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
             r++;
         }
     }
-    if (n_new) atomicAdd(&sh_new, n_new);
     if (err) atomicOr(&sh_err, err);
     __syncthreads();
     if (tid == 0) {
@@ -243,14 +287,17 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
         if (ee) atomicOr(&sh_err, ee);
     }
     const uint32_t base = block_excl_scan<uint32_t, SMALL_THREADS / 64>(mine, wsum, &sh_total);
-    const uint32_t sw = sizeof(DevStatus) / 4;
+    uint32_t* ub_sh = reinterpret_cast<uint32_t*>(keys);  // (the tables are dead; 64 entries hold SMALL_SLOTS words)
     if (tid < (uint32_t)N) {
         ubase[tid] = base;
-        host_store(host_dst + sw + tid, base);
+        ub_sh[tid] = base;
     }
     __syncthreads();
+    if (tid >= 64) return;  // one wavefront writes to the host: its fence is the only one
+    const uint32_t sw = sizeof(DevStatus) / 4;
+    const uint32_t U = sh_total;
+    for (uint32_t i = tid; i < (uint32_t)N; i += 64) host_store(host_dst + sw + i, ub_sh[i]);
     if (tid == 0) {
-        const uint32_t U = sh_total;
         ubase[N] = U;
         host_store(host_dst + sw + N, U);
         DevStatus st{};
@@ -264,7 +311,6 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
         for (uint32_t i = 0; i < sw; i++) host_store(host_dst + i, sp[i]);
     }
     __threadfence_system();
-    __syncthreads();
     if (tid == 0) host_store(host_seq, seq);
 }
 
@@ -307,8 +353,8 @@ __global__ __launch_bounds__(256) void k_small_finish(Store s, const SlotDesc* _
 }
 
 // First launch of a small push on the last pull's plan: the slot descriptors come in from the host's staging
-// buffer (every workgroup reads them into LDS, the first also leaves them in device memory for the
-// update kernels), the signs are compared with the plan's copy, and with CLICKS the non-zero labels are added to
+// buffer (a workgroup reads those of its tile's slots into LDS, the first also copies all of them to device
+// memory for the update kernels), the signs are compared with the plan's copy, and with CLICKS the non-zero labels are added to
 // the click sums of the member lists (sparse_table_ops.cc:283-296; a few thousand lookups do not queue up on
 // any entry).  The workgroup that finishes last tells the host that the comparison is done.
 template <bool CLICKS>
@@ -319,21 +365,29 @@ __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs
                                                       const uint2* __restrict__ where_u, Member* list,
                                                       SmallState* state, uint32_t* host_mismatch, uint32_t* host_seq,
                                                       uint32_t seq) {
-    extern __shared__ unsigned long long vsm64[];  // the descriptors, then lb[N + 1]
-    uint32_t* vsm = reinterpret_cast<uint32_t*>(vsm64);
-    SlotDesc* sd = reinterpret_cast<SlotDesc*>(vsm64);
-    uint32_t* lb = vsm + (size_t)N * (sizeof(SlotDesc) / 4);
+    extern __shared__ uint32_t lb[];      // lb[N + 1]
+    __shared__ SlotDesc sd[SMALL_SLOTS];  // the descriptors of the slots the tile touches: sd[0] is slot s0's
     __shared__ uint32_t sh_last;
-    const uint32_t words = (uint32_t)N * (sizeof(SlotDesc) / 4);
-    for (uint32_t i = threadIdx.x; i < words; i += 256) vsm[i] = reinterpret_cast<const uint32_t*>(host_descs)[i];
     for (int i = threadIdx.x; i <= N; i += 256) lb[i] = lbase[i];
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         status->err = 0;  // what the pull reported is on the host; the update kernels start from a clean slate
         status->abort = 0;
     }
     __syncthreads();
-    if (blockIdx.x == 0)
-        for (uint32_t i = threadIdx.x; i < words; i += 256) reinterpret_cast<uint32_t*>(push_descs)[i] = vsm[i];
+    constexpr uint32_t DW = sizeof(SlotDesc) / 4;
+    const int s0 = find_slot(lb, N, blockIdx.x * SMALL_TILE);
+    const int s1 = find_slot(lb, N, min(L, (blockIdx.x + 1) * (uint32_t)SMALL_TILE) - 1);
+    {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(host_descs + s0);
+        const uint32_t words = (uint32_t)(s1 - s0 + 1) * DW;
+        for (uint32_t i = threadIdx.x; i < words; i += 256) reinterpret_cast<uint32_t*>(sd)[i] = src[i];
+    }
+    if (blockIdx.x == 0) {  // all of them into device memory, for the update kernels
+        const uint32_t words = (uint32_t)N * DW;
+        for (uint32_t i = threadIdx.x; i < words; i += 256)
+            reinterpret_cast<uint32_t*>(push_descs)[i] = reinterpret_cast<const uint32_t*>(host_descs)[i];
+    }
+    __syncthreads();
     const uint32_t g0 = blockIdx.x * SMALL_TILE;
     const uint32_t g1 = min(L, g0 + (uint32_t)SMALL_TILE);
     bool bad = false;
@@ -349,10 +403,10 @@ __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs
         u[j] = 0;
         if (gi < g1) {
             const int sl = find_slot(lb, N, gi);
-            now[j] = (uint64_t)sd[sl].values[gi - lb[sl]];
+            now[j] = (uint64_t)sd[sl - s0].values[gi - lb[sl]];
             then[j] = vals_copy[gi];
             if (CLICKS) {
-                label[j] = (int)sd[sl].labels[gi - lb[sl]];
+                label[j] = (int)sd[sl - s0].labels[gi - lb[sl]];
                 u[j] = u_of_gi[gi] & ~FIRST_BIT;
             }
         }
@@ -385,12 +439,12 @@ struct SmallPublish {
 
 __device__ __forceinline__ void small_publish(const SmallPublish& pub, DevStatus* status, uint32_t* sh_flag) {
     if (!last_workgroup(&pub.state->done_apply, gridDim.x, sh_flag)) return;
+    if (threadIdx.x >= 64) return;  // one wavefront: its fence is the only one
     const uint32_t sw = sizeof(DevStatus) / 4;
     const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
-    for (uint32_t i = threadIdx.x; i < sw + pub.n_ubase; i += blockDim.x)
+    for (uint32_t i = threadIdx.x; i < sw + pub.n_ubase; i += 64)
         host_store(pub.host_dst + i, i < sw ? ld_relaxed(sp + i) : pub.ubase[i - sw]);
     __threadfence_system();
-    __syncthreads();
     if (threadIdx.x == 0) {
         status->mismatch = 0;
         status->err = 0;
@@ -408,6 +462,19 @@ __global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc 
                                                      const Member* __restrict__ list, uint32_t big_k,
                                                      uint32_t ids_cap, SmallPublish pub) {
     __shared__ uint32_t sh_flag;
+    // the slots' gradient matrices and bases from LDS: one round trip less in every record's chain of loads
+    __shared__ SlotDesc sd[SMALL_SLOTS];
+    __shared__ uint32_t ub[SMALL_SLOTS + 1];
+    {
+        const uint32_t n_slots = pub.n_ubase - 1;
+        const uint32_t words = n_slots * (uint32_t)(sizeof(SlotDesc) / 4);
+        for (uint32_t i = threadIdx.x; i < words; i += 256)
+            reinterpret_cast<uint32_t*>(sd)[i] = reinterpret_cast<const uint32_t*>(src.descs)[i];
+        for (uint32_t i = threadIdx.x; i <= n_slots; i += 256) ub[i] = src.ubase[i];
+        __syncthreads();
+        src.descs = sd;
+        src.ubase = ub;
+    }
     // (a plan that turned out not to be this batch's: nothing to do but to say so)
     if (!(status->mismatch | status->abort)) {
         const uint32_t n_single = status->n_single, n_multi = status->n_multi;

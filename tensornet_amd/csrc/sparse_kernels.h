@@ -208,28 +208,21 @@ __device__ __forceinline__ uint64_t home_group(uint64_t sign, uint64_t cap) {
 
 __device__ __forceinline__ void init_row(const Store& s, const OptDev& o, uint64_t seed, uint64_t sign, uint64_t row);
 
-// Slot of `sign` in the table, NO_ROW if absent (or, with INSERT, if the table
-// is full).  With INSERT an absent sign claims the first free slot of its probe
-// sequence and is_new tells whether this call made the claim.
+// The probe sequence of `sign` from the group at idx on, whose eight keys the caller has loaded
+// already (q0..q3): several probes of a thread can have their first groups in flight together.
 template <bool INSERT>
-__device__ __forceinline__ uint32_t probe_slot(const Store& s, uint64_t sign, bool& is_new) {
-    is_new = false;
-    if (sign == EMPTY_KEY) {
-        if (INSERT) {
-            is_new = atomicCAS(s.special, 0u, 1u) == 0u;
-            return (uint32_t)s.cap;
-        }
-        return ld_relaxed(s.special) ? (uint32_t)s.cap : NO_ROW;
-    }
+__device__ __forceinline__ uint32_t probe_from(const Store& s, uint64_t sign, uint64_t idx, ulonglong2 q0, ulonglong2 q1,
+                                               ulonglong2 q2, ulonglong2 q3, bool& is_new) {
     // Linear probing in aligned groups of PROBE_WIDTH slots, starting at the group of the home
     // slot (the capacity is a multiple of PROBE_WIDTH): a group is one 64-byte granule, read
     // with four 16-byte loads in one round trip, and at a load of 0.75 few probes need a second
     // group.  Unaligned windows straddle granule boundaries and were measured at half the rate.
-    uint64_t idx = home_group(sign, s.cap);
     for (uint64_t p = 0; p < s.cap; p += PROBE_WIDTH) {
-        // plain loads: a key never changes once set, and a stale free slot is settled by the compare-and-swap
-        const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + idx);
-        const ulonglong2 q0 = g[0], q1 = g[1], q2 = g[2], q3 = g[3];
+        if (p != 0) {
+            // plain loads: a key never changes once set, and a stale free slot is settled by the compare-and-swap
+            const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + idx);
+            q0 = g[0], q1 = g[1], q2 = g[2], q3 = g[3];
+        }
         const uint64_t k[PROBE_WIDTH] = {q0.x, q0.y, q1.x, q1.y, q2.x, q2.y, q3.x, q3.y};
 #pragma unroll
         for (int j = 0; j < PROBE_WIDTH; j++) {
@@ -246,6 +239,24 @@ __device__ __forceinline__ uint32_t probe_slot(const Store& s, uint64_t sign, bo
         idx = idx + PROBE_WIDTH >= s.cap ? 0 : idx + PROBE_WIDTH;
     }
     return NO_ROW;
+}
+
+// Slot of `sign` in the table, NO_ROW if absent (or, with INSERT, if the table
+// is full).  With INSERT an absent sign claims the first free slot of its probe
+// sequence and is_new tells whether this call made the claim.
+template <bool INSERT>
+__device__ __forceinline__ uint32_t probe_slot(const Store& s, uint64_t sign, bool& is_new) {
+    is_new = false;
+    if (sign == EMPTY_KEY) {
+        if (INSERT) {
+            is_new = atomicCAS(s.special, 0u, 1u) == 0u;
+            return (uint32_t)s.cap;
+        }
+        return ld_relaxed(s.special) ? (uint32_t)s.cap : NO_ROW;
+    }
+    const uint64_t idx = home_group(sign, s.cap);
+    const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + idx);
+    return probe_from<INSERT>(s, sign, idx, g[0], g[1], g[2], g[3], is_new);
 }
 
 // With groups_of != nullptr the signs are those of its groups (ids_cap = size of the id space).

@@ -1874,7 +1874,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         }
         const uint32_t seq_v = ++t->seq_verify, seq_a = ++t->seq_apply;
         const int tiles = (int)((L + SMALL_TILE - 1) / SMALL_TILE);
-        const size_t vlds = (size_t)N * sizeof(SlotDesc) + ((size_t)N + 1) * sizeof(uint32_t);
+        const size_t vlds = ((size_t)N + 1) * sizeof(uint32_t);
         if (clicks)
             TN_LAUNCH_LDS((k_small_verify<true>), dim3(tiles), dim3(256), vlds, st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
