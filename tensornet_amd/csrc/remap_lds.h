@@ -558,104 +558,121 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
 //   y: bits 0-15 records of the bucket's earlier several-record groups, 16-23 place, 24-31 slot
 // and per bucket the number of groups with one record, with several, the
 // records of the latter, and the big groups.  At most GRP_SLOTS slots.
-__global__ __launch_bounds__(GRP_THREADS) void k_group_count(uint32_t nb2, const uint32_t* __restrict__ cursor2,
-                                                     const GroupRec* __restrict__ recs, uint32_t big_k,
-                                                     uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
-    __shared__ unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
-    __shared__ unsigned long long mlo[GRP_TABLE + 1], mhi[GRP_TABLE + 1];
+// LDS of a workgroup that groups second-level buckets (group_count_bucket).
+struct GroupCountLds {
+    unsigned long long keys[GRP_TABLE + 1];  // entry GRP_TABLE: the sign EMPTY_KEY itself
+    unsigned long long mlo[GRP_TABLE + 1], mhi[GRP_TABLE + 1];
+    uint16_t rech[GRP_CAP];
+    unsigned long long sh[GRP_THREADS / 64];
+};
+
+// One second-level bucket, by a workgroup of GRP_THREADS threads (the caller puts a barrier between two buckets).
+__device__ __forceinline__ void group_count_bucket(uint32_t c, GroupCountLds& lds, const uint32_t* __restrict__ cursor2,
+                                                   const GroupRec* __restrict__ recs, uint32_t big_k,
+                                                   uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
+    unsigned long long* const keys = lds.keys;
+    unsigned long long* const mlo = lds.mlo;
+    unsigned long long* const mhi = lds.mhi;
+    uint16_t* const rech = lds.rech;
+    unsigned long long* const sh = lds.sh;
     // Once every record knows its entry (rech) the keys are dead: the entries' group numbers and offsets
     // take their place, which lets three workgroups instead of two share a CU's LDS.
     uint2* const einfo = reinterpret_cast<uint2*>(keys);  // x: info word, y: records before the group
-    __shared__ uint16_t rech[GRP_CAP];
-    __shared__ unsigned long long sh[GRP_THREADS / 64];
+    const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
+    if (n == 0) {
+        if (threadIdx.x == 0) bcounts[c] = make_uint4(0, 0, 0, 0);
+        return;
+    }
+    const size_t first = (size_t)c * GRP_CAP;
+    // all records of the bucket sit in registers (GRP_CAP = GRP_THREADS x GRP_RECS), loaded together
+    // and in flight while the table is cleared
+    uint64_t sg[GRP_RECS];
+    uint32_t sl[GRP_RECS];  // slot of the record, 0xFFFFFFFF = no record
+#pragma unroll
+    for (int j = 0; j < GRP_RECS; j++) {
+        const uint32_t i = j * GRP_THREADS + threadIdx.x;
+        sg[j] = 0;
+        sl[j] = 0xFFFFFFFFu;
+        if (i < n) {
+            const GroupRec r = recs[first + i];
+            sg[j] = r.sign;
+            sl[j] = r.cnt >> 24;
+        }
+    }
+    for (int i = threadIdx.x; i <= GRP_TABLE; i += GRP_THREADS) {
+        keys[i] = EMPTY_KEY;
+        mlo[i] = 0;
+        mhi[i] = 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < GRP_RECS; j++) {
+        if (sl[j] == 0xFFFFFFFFu) continue;
+        const uint64_t sign = sg[j];
+        uint32_t h = GRP_TABLE;
+        if (sign != EMPTY_KEY) {
+            h = (uint32_t)(mix64(sign) >> 9) & (GRP_TABLE - 1);
+            for (;;) {  // n <= GRP_CAP < GRP_TABLE: a free entry exists
+                unsigned long long old = keys[h];
+                if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
+                if (old == EMPTY_KEY || old == sign) break;
+                h = (h + 1) & (GRP_TABLE - 1);
+            }
+        }
+        atomicOr(sl[j] < 64 ? &mlo[h] : &mhi[h], 1ull << (sl[j] & 63));
+        rech[j * GRP_THREADS + threadIdx.x] = (uint16_t)h;
+    }
+    __syncthreads();
+    uint32_t ks[GRP_ITEMS];
+    unsigned long long v = 0;  // 16-bit fields: groups of one record, of several, records of those, big groups
+    for (int j = 0; j < GRP_ITEMS; j++) {
+        const uint32_t e = j * GRP_THREADS + threadIdx.x;
+        const uint32_t k = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
+        ks[j] = k;
+        if (k == 1) v += 1ull;
+        if (k > 1) v += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
+    }
+    unsigned long long total;
+    unsigned long long ex = block_excl_scan<unsigned long long, GRP_THREADS / 64>(v, sh, &total);
+    if (threadIdx.x == 0)
+        bcounts[c] = make_uint4((uint32_t)(total & 0xFFFF), (uint32_t)((total >> 16) & 0xFFFF),
+                                (uint32_t)((total >> 32) & 0xFFFF), (uint32_t)(total >> 48));
+    for (int j = 0; j < GRP_ITEMS; j++) {
+        const uint32_t k = ks[j];
+        if (k == 0) continue;
+        const uint32_t e = j * GRP_THREADS + threadIdx.x;
+        if (k == 1) {
+            einfo[e] = make_uint2((uint32_t)(ex & 0xFFFF) | (1u << 24), 0u);
+            ex += 1ull;
+        } else {
+            einfo[e] = make_uint2((uint32_t)((ex >> 16) & 0xFFFF) | ((uint32_t)(ex >> 48) << 12) | (k << 24),
+                                  (uint32_t)((ex >> 32) & 0xFFFF));
+            ex += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < GRP_RECS; j++) {
+        const uint32_t s1 = sl[j];
+        if (s1 == 0xFFFFFFFFu) continue;
+        const uint32_t i = j * GRP_THREADS + threadIdx.x;
+        const uint32_t h = rech[i];
+        uint32_t place;
+        if (s1 < 64)
+            place = (uint32_t)__popcll(mlo[h] & ((1ull << s1) - 1ull));
+        else
+            place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (s1 - 64)) - 1ull));
+        const uint2 ei = einfo[h];
+        aux[first + i] = make_uint2(ei.x, ei.y | (place << 16) | (s1 << 24));
+    }
+}
+
+__global__ __launch_bounds__(GRP_THREADS) void k_group_count(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+                                                     const GroupRec* __restrict__ recs, uint32_t big_k,
+                                                     uint2* __restrict__ aux, uint4* __restrict__ bcounts) {
+    __shared__ GroupCountLds lds;
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
-        const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
-        if (n == 0) {
-            if (threadIdx.x == 0) bcounts[c] = make_uint4(0, 0, 0, 0);
-            continue;
-        }
-        const size_t first = (size_t)c * GRP_CAP;
-        // all records of the bucket sit in registers (GRP_CAP = GRP_THREADS x GRP_RECS), loaded together
-        // and in flight while the table is cleared
-        uint64_t sg[GRP_RECS];
-        uint32_t sl[GRP_RECS];  // slot of the record, 0xFFFFFFFF = no record
-#pragma unroll
-        for (int j = 0; j < GRP_RECS; j++) {
-            const uint32_t i = j * GRP_THREADS + threadIdx.x;
-            sg[j] = 0;
-            sl[j] = 0xFFFFFFFFu;
-            if (i < n) {
-                const GroupRec r = recs[first + i];
-                sg[j] = r.sign;
-                sl[j] = r.cnt >> 24;
-            }
-        }
-        for (int i = threadIdx.x; i <= GRP_TABLE; i += GRP_THREADS) {
-            keys[i] = EMPTY_KEY;
-            mlo[i] = 0;
-            mhi[i] = 0;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < GRP_RECS; j++) {
-            if (sl[j] == 0xFFFFFFFFu) continue;
-            const uint64_t sign = sg[j];
-            uint32_t h = GRP_TABLE;
-            if (sign != EMPTY_KEY) {
-                h = (uint32_t)(mix64(sign) >> 9) & (GRP_TABLE - 1);
-                for (;;) {  // n <= GRP_CAP < GRP_TABLE: a free entry exists
-                    unsigned long long old = keys[h];
-                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
-                    if (old == EMPTY_KEY || old == sign) break;
-                    h = (h + 1) & (GRP_TABLE - 1);
-                }
-            }
-            atomicOr(sl[j] < 64 ? &mlo[h] : &mhi[h], 1ull << (sl[j] & 63));
-            rech[j * GRP_THREADS + threadIdx.x] = (uint16_t)h;
-        }
-        __syncthreads();
-        uint32_t ks[GRP_ITEMS];
-        unsigned long long v = 0;  // 16-bit fields: groups of one record, of several, records of those, big groups
-        for (int j = 0; j < GRP_ITEMS; j++) {
-            const uint32_t e = j * GRP_THREADS + threadIdx.x;
-            const uint32_t k = (e <= GRP_TABLE) ? (uint32_t)(__popcll(mlo[e]) + __popcll(mhi[e])) : 0;
-            ks[j] = k;
-            if (k == 1) v += 1ull;
-            if (k > 1) v += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
-        }
-        unsigned long long total;
-        unsigned long long ex = block_excl_scan<unsigned long long, GRP_THREADS / 64>(v, sh, &total);
-        if (threadIdx.x == 0)
-            bcounts[c] = make_uint4((uint32_t)(total & 0xFFFF), (uint32_t)((total >> 16) & 0xFFFF),
-                                    (uint32_t)((total >> 32) & 0xFFFF), (uint32_t)(total >> 48));
-        for (int j = 0; j < GRP_ITEMS; j++) {
-            const uint32_t k = ks[j];
-            if (k == 0) continue;
-            const uint32_t e = j * GRP_THREADS + threadIdx.x;
-            if (k == 1) {
-                einfo[e] = make_uint2((uint32_t)(ex & 0xFFFF) | (1u << 24), 0u);
-                ex += 1ull;
-            } else {
-                einfo[e] = make_uint2((uint32_t)((ex >> 16) & 0xFFFF) | ((uint32_t)(ex >> 48) << 12) | (k << 24),
-                                      (uint32_t)((ex >> 32) & 0xFFFF));
-                ex += (1ull << 16) + ((unsigned long long)k << 32) + (is_big(k, big_k) ? 1ull << 48 : 0ull);
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < GRP_RECS; j++) {
-            const uint32_t s1 = sl[j];
-            if (s1 == 0xFFFFFFFFu) continue;
-            const uint32_t i = j * GRP_THREADS + threadIdx.x;
-            const uint32_t h = rech[i];
-            uint32_t place;
-            if (s1 < 64)
-                place = (uint32_t)__popcll(mlo[h] & ((1ull << s1) - 1ull));
-            else
-                place = (uint32_t)__popcll(mlo[h]) + (uint32_t)__popcll(mhi[h] & ((1ull << (s1 - 64)) - 1ull));
-            const uint2 ei = einfo[h];
-            aux[first + i] = make_uint2(ei.x, ei.y | (place << 16) | (s1 << 24));
-        }
+        group_count_bucket(c, lds, cursor2, recs, big_k, aux, bcounts);
         __syncthreads();
     }
 }

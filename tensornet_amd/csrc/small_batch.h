@@ -3,20 +3,20 @@
 // lookups spends its time in the dependent launches of that path (about 3 us each, whatever the
 // kernel does), not in its kernels, so here
 //
-//   pull  k_small_slots   one workgroup per slot: per-slot first-occurrence remap in LDS
-//                         (sparse_table_ops.cc:115-137), lookup-or-insert of every distinct sign
-//                         (sparse_table.cc:52-66), its record handed to its second-level bucket;
-//                         the workgroup that finishes last adds up the slots' counts and publishes
-//                         the call's status to the host, which returns as soon as it sees it
-//         k_small_finish  rows into the variables (sparse_table_ops.cc:244-265), distinct indices
-//                         made global
-//         k_group_count, k_group_emit<true>   the groups of equal signs over all slots, as ever
-//   push  k_small_verify  slot descriptors in, comparison with the plan's signs, click sums
-//         k_apply_big (16 slots or more), k_small_apply   every group by one launch; its last
-//                         workgroup publishes the status
+//   pull  k_small_slots          one workgroup per slot: per-slot first-occurrence remap in LDS
+//                                (sparse_table_ops.cc:115-137), lookup-or-insert of every distinct sign
+//                                (sparse_table.cc:52-66), its record handed to its second-level bucket
+//         k_small_group_finish   the first pass of the grouping (what k_group_count does) beside: the slots'
+//                                counts added up, the call's status published to the host (which returns as
+//                                soon as it sees it), rows into the variables (sparse_table_ops.cc:244-265),
+//                                distinct indices made global
+//         k_group_emit<true>     the groups of equal signs over all slots, as ever
+//   push  k_small_verify         slot descriptors in, comparison with the plan's signs, click sums
+//         k_small_apply          every group by one launch (tells the host that the comparison is complete)
+//         k_apply_big            with more than 12 slots: the signs with 5 records or more
 //
-// Workgroups of one launch never wait for each other: a workgroup that needs the others' results is
-// the one that finishes last (a ticket counter tells), or runs in the next launch.
+// Workgroups of one launch never wait for each other, and none needs another's results: what needs them runs
+// in the next launch.
 #ifndef TN_SMALL_BATCH_H_
 #define TN_SMALL_BATCH_H_
 
@@ -37,11 +37,9 @@ struct SlotOut {
 };
 
 // Persistent device state of the small path (zero when allocated).  A call uses one of the two sets of
-// bucket cursors and clears the other for the call after it; the ticket counters are set back to zero by
-// the workgroup that draws the last ticket.
+// bucket cursors and clears the other for the call after it.
 struct SmallState {
     uint32_t cursor2[2][SMALL_NB2_MAX];
-    uint32_t done_pull, done_verify, done_apply, pad;
     SlotOut slot_out[SMALL_SLOTS];
 };
 
@@ -54,33 +52,11 @@ __device__ __forceinline__ void host_store(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// True in every thread of the workgroup that draws the last of `n` tickets.  Every thread of every workgroup of
-// the launch calls it once.  No fence: a release fence writes back the whole L2, which with a fence per
-// workgroup took several times as long as the kernels' work.  What the last workgroup reads of the others is
-// therefore written with device-scope atomics (they meet in memory, whatever the XCD) by the thread that draws
-// the ticket, which waits for them before it draws; a thread that raises an error flag elsewhere fences itself.
-__device__ __forceinline__ bool last_workgroup(uint32_t* counter, uint32_t n, uint32_t* sh_flag) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __builtin_amdgcn_s_waitcnt(0);  // this thread's atomics are done
-        const uint32_t ticket = atomicAdd(counter, 1u);
-        *sh_flag = ticket == n - 1 ? 1u : 0u;
-        if (ticket == n - 1) atomicExch(counter, 0u);  // nobody draws after the last
-    }
-    __syncthreads();
-    return *sh_flag != 0;
-}
-
-__device__ __forceinline__ void publish_word(uint32_t* p, uint32_t v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
-    const SlotDesc* host_descs, SlotDesc* descs, uint32_t* lbase, uint32_t* ubase, int N, uint32_t L, uint32_t entries,
+    const SlotDesc* host_descs, SlotDesc* descs, uint32_t* lbase, int N, uint32_t L, uint32_t entries,
     Store s, OptDev o, uint64_t seed, uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ u_of_gi,
     uint32_t* __restrict__ prow, uint32_t nb2, uint32_t* cursor2, uint32_t* cursor2_next, GroupRec* __restrict__ recs,
-    uint32_t* __restrict__ rrow, SmallState* state, DevStatus* status, uint32_t* host_dst, uint32_t* host_seq,
-    uint32_t seq) {
+    uint32_t* __restrict__ rrow, SmallState* state) {
     extern __shared__ unsigned long long smem64[];
     unsigned long long* keys = smem64;  // entry `entries`: the sign EMPTY_KEY itself
     uint32_t* minpos = reinterpret_cast<uint32_t*>(keys + entries + 1);
@@ -88,7 +64,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     uint32_t* hist2 = cnts + entries + 1;
     __shared__ SlotDesc sd;
     __shared__ uint32_t wsum[SMALL_THREADS / 64];
-    __shared__ uint32_t sh_new, sh_err, sh_last, sh_total;
+    __shared__ uint32_t sh_new, sh_err;
     const int sl = blockIdx.x;
     const uint32_t tid = threadIdx.x;
     // the slot's descriptor comes straight out of the host's staging buffer (one round trip over the bus,
@@ -265,74 +241,85 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     }
     if (err) atomicOr(&sh_err, err);
     __syncthreads();
-    if (tid == 0) {
-        uint32_t* out = reinterpret_cast<uint32_t*>(&state->slot_out[sl]);
-        publish_word(out, total);
-        publish_word(out + 1, sh_new);
-        publish_word(out + 2, sh_err);
+    if (tid == 0) {  // for the next launch, which adds up the slots' counts and publishes the call's status
+        SlotOut out;
+        out.n_unique = total;
+        out.n_new = sh_new;
+        out.err = sh_err;
+        out.pad = 0;
+        state->slot_out[sl] = out;
     }
-    if (!last_workgroup(&state->done_pull, (uint32_t)N, &sh_last)) return;
-    // the last workgroup: bases of the slots' distinct indices, the call's status, both to the host
-    uint32_t mine = 0;
-    if (tid == 0) {
-        sh_new = 0;
-        sh_err = 0;
-    }
-    __syncthreads();
-    if (tid < (uint32_t)N) {
-        const uint32_t* so = reinterpret_cast<const uint32_t*>(&state->slot_out[tid]);
-        mine = ld_relaxed(so);
-        const uint32_t nn = ld_relaxed(so + 1), ee = ld_relaxed(so + 2);
-        if (nn) atomicAdd(&sh_new, nn);
-        if (ee) atomicOr(&sh_err, ee);
-    }
-    const uint32_t base = block_excl_scan<uint32_t, SMALL_THREADS / 64>(mine, wsum, &sh_total);
-    uint32_t* ub_sh = reinterpret_cast<uint32_t*>(keys);  // (the tables are dead; 64 entries hold SMALL_SLOTS words)
-    if (tid < (uint32_t)N) {
-        ubase[tid] = base;
-        ub_sh[tid] = base;
-    }
-    __syncthreads();
-    if (tid >= 64) return;  // one wavefront writes to the host: its fence is the only one
-    const uint32_t sw = sizeof(DevStatus) / 4;
-    const uint32_t U = sh_total;
-    for (uint32_t i = tid; i < (uint32_t)N; i += 64) host_store(host_dst + sw + i, ub_sh[i]);
-    if (tid == 0) {
-        ubase[N] = U;
-        host_store(host_dst + sw + N, U);
-        DevStatus st{};
-        st.err = sh_err;
-        st.n_unique = U;
-        st.n_new = sh_new;
-        st.gcap = U + U / 2 < 16 ? 16 : U + U / 2;
-        *status = st;
-        *s.count += sh_new;
-        const uint32_t* sp = reinterpret_cast<const uint32_t*>(&st);
-        for (uint32_t i = 0; i < sw; i++) host_store(host_dst + i, sp[i]);
-    }
-    __threadfence_system();
-    if (tid == 0) host_store(host_seq, seq);
 }
 
-// Second launch of a small pull: vars[slot][rank, :] = table row of the slot's distinct sign of that rank
-// (PopulatePulledVariable_, sparse_table_ops.cc:244-265), and the distinct indices of the lookups made
-// global (rank in the slot + base of the slot).  The ranks of a slot occupy the first positions of its
-// window of lookup positions.
+// Second launch of a small pull, two kinds of workgroups.  The first nb2 group the second-level buckets
+// (group_count_bucket: what k_group_count does).  The others finish what the slots' workgroups began:
+// vars[slot][rank, :] = table row of the slot's distinct sign of that rank (PopulatePulledVariable_,
+// sparse_table_ops.cc:244-265), and the distinct indices of the lookups made global (rank in the slot + base
+// of the slot; the ranks of a slot occupy the first positions of its window of lookup positions).  Each of them
+// adds up the slots' counts itself; the first also leaves the bases and the call's status in device memory and
+// publishes them to the host, which returns from the call when it sees them.
 template <int VEC>
-__global__ __launch_bounds__(256) void k_small_finish(Store s, const SlotDesc* __restrict__ descs,
-                                                      const uint32_t* __restrict__ lbase,
-                                                      const uint32_t* __restrict__ ubase, int N, uint32_t L,
-                                                      const uint32_t* __restrict__ prow, uint32_t* __restrict__ u_of_gi) {
-    extern __shared__ uint32_t lb[];  // lb[N + 1], ub[N + 1]
-    uint32_t* ub = lb + N + 1;
-    for (int i = threadIdx.x; i <= N; i += 256) {
-        lb[i] = lbase[i];
-        ub[i] = ubase[i];
+__global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
+    uint32_t nb2, const uint32_t* __restrict__ cursor2, const GroupRec* __restrict__ recs, uint32_t big_k,
+    uint2* __restrict__ aux, uint4* __restrict__ bcounts, Store s, const SlotDesc* __restrict__ descs,
+    const uint32_t* __restrict__ lbase, uint32_t* ubase, int N, uint32_t L, const uint32_t* __restrict__ prow,
+    uint32_t* __restrict__ u_of_gi, const SmallState* __restrict__ state, DevStatus* status, uint32_t* host_dst,
+    uint32_t* host_seq, uint32_t seq) {
+    __shared__ GroupCountLds lds;
+    if (blockIdx.x < nb2) {
+        group_count_bucket(blockIdx.x, lds, cursor2, recs, big_k, aux, bcounts);
+        return;
+    }
+    // (the grouping's LDS is free here)
+    uint32_t* lb = reinterpret_cast<uint32_t*>(lds.mlo);  // lb[N + 1]
+    uint32_t* ub = reinterpret_cast<uint32_t*>(lds.mhi);  // ub[N + 1]
+    uint32_t* wsum = reinterpret_cast<uint32_t*>(lds.sh);
+    uint32_t* misc = reinterpret_cast<uint32_t*>(lds.rech);  // [0] new rows, [1] error flags, [2] distinct signs
+    const uint32_t tid = threadIdx.x;
+    const bool publisher = blockIdx.x == nb2;
+    uint32_t mine = 0, nn = 0, ee = 0;
+    if (tid < (uint32_t)N) {
+        const SlotOut so = state->slot_out[tid];
+        mine = so.n_unique;
+        nn = so.n_new;
+        ee = so.err;
+    }
+    for (uint32_t i = tid; i <= (uint32_t)N; i += GRP_THREADS) lb[i] = lbase[i];
+    if (tid < 2) misc[tid] = 0;
+    const uint32_t base = block_excl_scan<uint32_t, GRP_THREADS / 64>(mine, wsum, &misc[2]);  // (barriers inside)
+    if (tid < (uint32_t)N) ub[tid] = base;
+    if (publisher) {
+        if (nn) atomicAdd(&misc[0], nn);
+        if (ee) atomicOr(&misc[1], ee);
+    }
+    __syncthreads();
+    const uint32_t U = misc[2];
+    if (tid == 0) ub[N] = U;
+    if (publisher && tid < 64) {  // one wavefront: device copies, then the host's, then the word the host polls
+        const uint32_t sw = sizeof(DevStatus) / 4;
+        for (uint32_t i = tid; i <= (uint32_t)N; i += 64) {
+            const uint32_t v = i < (uint32_t)N ? ub[i] : U;
+            ubase[i] = v;
+            host_store(host_dst + sw + i, v);
+        }
+        if (tid == 0) {
+            DevStatus st{};
+            st.err = misc[1];
+            st.n_unique = U;
+            st.n_new = misc[0];
+            st.gcap = U + U / 2 < 16 ? 16 : U + U / 2;
+            *status = st;
+            *s.count += misc[0];
+            const uint32_t* sp = reinterpret_cast<const uint32_t*>(&st);
+            for (uint32_t i = 0; i < sw; i++) host_store(host_dst + i, sp[i]);
+        }
+        __threadfence_system();
+        if (tid == 0) host_store(host_seq, seq);
     }
     __syncthreads();
     // one thread per (position, part of the row): few rows per thread would leave the rows' round trips in a queue
     const uint32_t chunks = (uint32_t)(s.wdim / VEC);
-    const uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t t = (uint64_t)(blockIdx.x - nb2) * GRP_THREADS + tid;
     if (t >= (uint64_t)L * chunks) return;
     const uint32_t gi = (uint32_t)(t / chunks);
     const uint32_t c = (uint32_t)(t - (uint64_t)gi * chunks);
@@ -356,18 +343,17 @@ __global__ __launch_bounds__(256) void k_small_finish(Store s, const SlotDesc* _
 // buffer (a workgroup reads those of its tile's slots into LDS, the first also copies all of them to device
 // memory for the update kernels), the signs are compared with the plan's copy, and with CLICKS the non-zero labels are added to
 // the click sums of the member lists (sparse_table_ops.cc:283-296; a few thousand lookups do not queue up on
-// any entry).  The workgroup that finishes last tells the host that the comparison is done.
+// any entry).  A mismatch also goes to the host (pinned memory); that the comparison is complete, the kernel
+// launched next tells it.
 template <bool CLICKS>
 __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs, SlotDesc* push_descs,
                                                       const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                       const uint64_t* __restrict__ vals_copy, DevStatus* status,
                                                       const uint32_t* __restrict__ u_of_gi,
                                                       const uint2* __restrict__ where_u, Member* list,
-                                                      SmallState* state, uint32_t* host_mismatch, uint32_t* host_seq,
-                                                      uint32_t seq) {
+                                                      uint32_t* host_mismatch) {
     extern __shared__ uint32_t lb[];      // lb[N + 1]
     __shared__ SlotDesc sd[SMALL_SLOTS];  // the descriptors of the slots the tile touches: sd[0] is slot s0's
-    __shared__ uint32_t sh_last;
     for (int i = threadIdx.x; i <= N; i += 256) lb[i] = lbase[i];
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         status->err = 0;  // what the pull reported is on the host; the update kernels start from a clean slate
@@ -419,79 +405,48 @@ __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs
     if (bad) {
         atomicOr(&status->mismatch, 1u);
         host_store(host_mismatch, 1u);
-        __threadfence_system();
-    }
-    if (!last_workgroup(&state->done_verify, gridDim.x, &sh_last)) return;
-    if (threadIdx.x == 0) host_store(host_seq, seq);
-}
-
-// What the update kernel of a small push does when its last workgroup is done: the call's status and the
-// slots' distinct bases to the host, the flags of the plan's status block back to zero (a further push on
-// the same plan starts from them).
-struct SmallPublish {
-    SmallState* state;
-    const uint32_t* ubase;
-    uint32_t n_ubase;
-    uint32_t* host_dst;
-    uint32_t* host_seq;
-    uint32_t seq;
-};
-
-__device__ __forceinline__ void small_publish(const SmallPublish& pub, DevStatus* status, uint32_t* sh_flag) {
-    if (!last_workgroup(&pub.state->done_apply, gridDim.x, sh_flag)) return;
-    if (threadIdx.x >= 64) return;  // one wavefront: its fence is the only one
-    const uint32_t sw = sizeof(DevStatus) / 4;
-    const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
-    for (uint32_t i = threadIdx.x; i < sw + pub.n_ubase; i += 64)
-        host_store(pub.host_dst + i, i < sw ? ld_relaxed(sp + i) : pub.ubase[i - sw]);
-    __threadfence_system();
-    if (threadIdx.x == 0) {
-        status->mismatch = 0;
-        status->err = 0;
-        host_store(pub.host_seq, pub.seq);
     }
 }
 
 // Every group of the plan that k_apply_big does not take, one record or several, by one launch (the
-// lane groups of k_apply_vec); the last workgroup publishes the call's status.
+// lane groups of k_apply_vec, the records of a sign four at a time).  Nothing is reported to the host: on
+// the plan of the last pull every sign has its row, and the host has compared the slots' distinct counts with
+// the rows of the gradient matrices itself.
 template <int KIND, int LPG>
-__global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc src, DevStatus* status,
+__global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc src, int N, DevStatus* status,
                                                      const uint32_t* __restrict__ grp_row,
                                                      const uint32_t* __restrict__ grp_off,
                                                      const uint32_t* __restrict__ grp_cnt,
                                                      const Member* __restrict__ list, uint32_t big_k,
-                                                     uint32_t ids_cap, SmallPublish pub) {
-    __shared__ uint32_t sh_flag;
+                                                     uint32_t ids_cap, uint32_t* host_seq, uint32_t seq) {
+    // this kernel runs: the comparison of the signs, launched before it, is complete
+    if (blockIdx.x == 0 && threadIdx.x == 0) host_store(host_seq, seq);
     // the slots' gradient matrices and bases from LDS: one round trip less in every record's chain of loads
     __shared__ SlotDesc sd[SMALL_SLOTS];
     __shared__ uint32_t ub[SMALL_SLOTS + 1];
-    {
-        const uint32_t n_slots = pub.n_ubase - 1;
-        const uint32_t words = n_slots * (uint32_t)(sizeof(SlotDesc) / 4);
-        for (uint32_t i = threadIdx.x; i < words; i += 256)
-            reinterpret_cast<uint32_t*>(sd)[i] = reinterpret_cast<const uint32_t*>(src.descs)[i];
-        for (uint32_t i = threadIdx.x; i <= n_slots; i += 256) ub[i] = src.ubase[i];
-        __syncthreads();
-        src.descs = sd;
-        src.ubase = ub;
+    const uint32_t words = (uint32_t)N * (uint32_t)(sizeof(SlotDesc) / 4);
+    for (uint32_t i = threadIdx.x; i < words; i += 256)
+        reinterpret_cast<uint32_t*>(sd)[i] = reinterpret_cast<const uint32_t*>(src.descs)[i];
+    for (uint32_t i = threadIdx.x; i <= (uint32_t)N; i += 256) ub[i] = src.ubase[i];
+    // a plan that turned out not to be this batch's: nothing to do (the host analyses the batch itself)
+    const uint32_t stop = status->mismatch | status->abort;
+    const uint32_t n_single = status->n_single, n_multi = status->n_multi;
+    __syncthreads();
+    if (stop) return;
+    src.descs = sd;
+    src.ubase = ub;
+    const int sub = threadIdx.x % LPG;
+    const int lane0 = (int)__lane_id() - sub;
+    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
+    for (uint32_t t = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
+        const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
+        const uint32_t row = grp_row[g];
+        if (row == NO_ROW) continue;
+        const uint32_t k = grp_cnt[g];
+        if (is_big(k, big_k)) continue;
+        apply_group_vec<KIND, LPG, 4>(s, o, src, status, row, k, list + grp_off[g], nullptr, sub, lane0, c1, c2);
     }
-    // (a plan that turned out not to be this batch's: nothing to do but to say so)
-    if (!(status->mismatch | status->abort)) {
-        const uint32_t n_single = status->n_single, n_multi = status->n_multi;
-        const int sub = threadIdx.x % LPG;
-        const int lane0 = (int)__lane_id() - sub;
-        const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
-        const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
-        for (uint32_t t = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
-            const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
-            const uint32_t row = grp_row[g];
-            if (row == NO_ROW) continue;
-            const uint32_t k = grp_cnt[g];
-            if (is_big(k, big_k)) continue;
-            apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g], nullptr, sub, lane0, c1, c2);
-        }
-    }
-    small_publish(pub, status, &sh_flag);
 }
 
 }  // namespace tn

@@ -1469,29 +1469,74 @@ __global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc
 // is sorted) and stores the row once.  Each lane holds one float4 of every
 // per-element array; the next record's gradient is fetched while the current
 // one is applied.  Groups with big_k records or more are left to k_apply_big.
-template <int KIND, int LPG>
+// AHEAD = 1: the next record's gradient is fetched while the current one is applied (what keeps the most
+// wavefronts on a CU: the kernels of a large batch).  AHEAD > 1: records are taken AHEAD at a time, the gradients
+// of the next AHEAD and the member entries of the AHEAD after those in flight meanwhile: a chain of k records
+// costs k / AHEAD round trips instead of 2 k, which is what a small batch, whose kernels are as long as their
+// longest chain, is after.
+template <int KIND, int LPG, int AHEAD = 1>
 __device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o, const PushSrc& src, DevStatus* status,
                                                 uint32_t row, uint32_t k, const Member* mem, const float* const* ga,
                                                 int sub, int lane0, float c1, float c2) {
     const int D = s.D;
-    {
-        float* wp = s.w + (uint64_t)row * s.wstride;
-        float* sp = s.st + (uint64_t)row * s.sstride;
-        float4 w = reinterpret_cast<float4*>(wp)[sub];
-        float4 a, b;          // Adam m,v / Ftrl z,n
-        float g2sum = 0.f, show = 0.f, click = 0.f;
-        int delta_show = 0;
+    float* wp = s.w + (uint64_t)row * s.wstride;
+    float* sp = s.st + (uint64_t)row * s.sstride;
+    float4 w = reinterpret_cast<float4*>(wp)[sub];
+    float4 a, b;          // Adam m,v / Ftrl z,n
+    float g2sum = 0.f, show = 0.f, click = 0.f;
+    int delta_show = 0;
+    if (KIND == OPT_ADAGRAD) {
+        float4 h = *reinterpret_cast<const float4*>(sp);
+        g2sum = h.x;
+        show = h.y;
+        click = h.z;
+    } else {
+        a = reinterpret_cast<float4*>(sp)[sub];
+        b = reinterpret_cast<float4*>(sp + D)[sub];
+        delta_show = __float_as_int(sp[2 * D + 1]);
+    }
+    bool any = false;
+    // one record applied to the row held in registers
+    auto step = [&](const float4 gr, const int bshow, const int bclick) {
+        any = true;
         if (KIND == OPT_ADAGRAD) {
-            float4 h = *reinterpret_cast<const float4*>(sp);
-            g2sum = h.x;
-            show = h.y;
-            click = h.z;
+            show += (float)bshow;
+            click += (float)bclick;
+            const float p0 = gr.x * gr.x, p1 = gr.y * gr.y, p2 = gr.z * gr.z, p3 = gr.w * gr.w;
+            // add_g2sum: double accumulator over the float products, element order 0..D-1
+            double tot = 0.0;
+            for (int l = 0; l < LPG; l++) {
+                double cand = tot;
+                cand += (double)p0;
+                cand += (double)p1;
+                cand += (double)p2;
+                cand += (double)p3;
+                tot = __shfl(cand, lane0 + l);
+            }
+            g2sum = (float)((double)g2sum + tot / (double)D);
+            const float den = o.eps + sqrtf(g2sum);
+            w.x -= o.lr * gr.x / den;
+            w.y -= o.lr * gr.y / den;
+            w.z -= o.lr * gr.z / den;
+            w.w -= o.lr * gr.w / den;
+        } else if (KIND == OPT_ADAM) {
+            delta_show += bshow;
+            adam_elem(o, c1, c2, gr.x, w.x, a.x, b.x);
+            adam_elem(o, c1, c2, gr.y, w.y, a.y, b.y);
+            adam_elem(o, c1, c2, gr.z, w.z, a.z, b.z);
+            adam_elem(o, c1, c2, gr.w, w.w, a.w, b.w);
         } else {
-            a = reinterpret_cast<float4*>(sp)[sub];
-            b = reinterpret_cast<float4*>(sp + D)[sub];
-            delta_show = __float_as_int(sp[2 * D + 1]);
+            delta_show += bshow;
+            ftrl_elem(o, gr.x, w.x, a.x, b.x);
+            ftrl_elem(o, gr.y, w.y, a.y, b.y);
+            ftrl_elem(o, gr.z, w.z, a.z, b.z);
+            ftrl_elem(o, gr.w, w.w, a.w, b.w);
         }
-        bool any = false;
+    };
+    auto no_gradient = [&]() {
+        if (sub == 0) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+    };
+    if (AHEAD == 1) {
         const float* gp;
         int nshow = 0, nclick = 0;
         bool nok = record_at(src, mem, ga, 0, gp, nshow, nclick);
@@ -1506,62 +1551,73 @@ __device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o,
                 if (nok) gnext = reinterpret_cast<const float4*>(gp)[sub];
             }
             if (!ok) {
-                if (sub == 0) {
-                    atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-                    __threadfence();  // (k_small_apply publishes the status when its last workgroup is done)
-                }
+                no_gradient();
                 continue;
             }
-            any = true;
-            if (KIND == OPT_ADAGRAD) {
-                show += (float)bshow;
-                click += (float)bclick;
-                const float p0 = gr.x * gr.x, p1 = gr.y * gr.y, p2 = gr.z * gr.z, p3 = gr.w * gr.w;
-                // add_g2sum: double accumulator over the float products, element order 0..D-1
-                double tot = 0.0;
-                for (int l = 0; l < LPG; l++) {
-                    double cand = tot;
-                    cand += (double)p0;
-                    cand += (double)p1;
-                    cand += (double)p2;
-                    cand += (double)p3;
-                    tot = __shfl(cand, lane0 + l);
+            step(gr, bshow, bclick);
+        }
+    } else {
+        // chunk c: applied; chunk c + 1: gradients in flight; chunk c + 2: member entries in flight.  Every load is
+        // issued whether its record exists or not (past the end: the group's last member again, the row in place of
+        // a gradient): a load under a condition makes the compiler wait for all loads where the branches join.
+        Member m1[AHEAD], m2[AHEAD];
+        float4 g0[AHEAD], g1[AHEAD];
+        int sh0[AHEAD], ck0[AHEAD], sh1[AHEAD], ck1[AHEAD];
+        bool ok0[AHEAD], ok1[AHEAD];
+        auto fetch = [&](const Member (&m)[AHEAD], uint32_t first, float4 (&g)[AHEAD], int (&sh)[AHEAD], int (&ck)[AHEAD],
+                         bool (&ok)[AHEAD]) {
+#pragma unroll
+            for (int q = 0; q < AHEAD; q++) {
+                const float* gp = nullptr;
+                ok[q] = src_record(src, m[q], gp, sh[q], ck[q]) && first + q < k;
+                g[q] = reinterpret_cast<const float4*>(ok[q] ? gp : wp)[sub];
+            }
+        };
+#pragma unroll
+        for (int q = 0; q < AHEAD; q++) {
+            m1[q] = mem[min((uint32_t)q, k - 1)];
+            m2[q] = mem[min((uint32_t)(AHEAD + q), k - 1)];
+        }
+        fetch(m1, 0, g0, sh0, ck0, ok0);
+#pragma unroll
+        for (int q = 0; q < AHEAD; q++) m1[q] = m2[q];
+        for (uint32_t c0 = 0; c0 < k; c0 += AHEAD) {
+#pragma unroll
+            for (int q = 0; q < AHEAD; q++) m2[q] = mem[min(c0 + 2 * AHEAD + q, k - 1)];
+            fetch(m1, c0 + AHEAD, g1, sh1, ck1, ok1);
+#pragma unroll
+            for (int q = 0; q < AHEAD; q++) {
+                if (c0 + q >= k) break;
+                if (!ok0[q]) {
+                    no_gradient();
+                    continue;
                 }
-                g2sum = (float)((double)g2sum + tot / (double)D);
-                const float den = o.eps + sqrtf(g2sum);
-                w.x -= o.lr * gr.x / den;
-                w.y -= o.lr * gr.y / den;
-                w.z -= o.lr * gr.z / den;
-                w.w -= o.lr * gr.w / den;
-            } else if (KIND == OPT_ADAM) {
-                delta_show += bshow;
-                adam_elem(o, c1, c2, gr.x, w.x, a.x, b.x);
-                adam_elem(o, c1, c2, gr.y, w.y, a.y, b.y);
-                adam_elem(o, c1, c2, gr.z, w.z, a.z, b.z);
-                adam_elem(o, c1, c2, gr.w, w.w, a.w, b.w);
-            } else {
-                delta_show += bshow;
-                ftrl_elem(o, gr.x, w.x, a.x, b.x);
-                ftrl_elem(o, gr.y, w.y, a.y, b.y);
-                ftrl_elem(o, gr.z, w.z, a.z, b.z);
-                ftrl_elem(o, gr.w, w.w, a.w, b.w);
+                step(g0[q], sh0[q], ck0[q]);
+            }
+#pragma unroll
+            for (int q = 0; q < AHEAD; q++) {
+                g0[q] = g1[q];
+                sh0[q] = sh1[q];
+                ck0[q] = ck1[q];
+                ok0[q] = ok1[q];
+                m1[q] = m2[q];
             }
         }
-        if (!any) return;
-        reinterpret_cast<float4*>(wp)[sub] = w;
-        if (KIND == OPT_ADAGRAD) {
-            if (sub == 0) {
-                *reinterpret_cast<float4*>(sp) = make_float4(g2sum, show, click, 0.f);  // no_show_days = 0
-                if (o.use_cvm) {
-                    wp[D] = show;
-                    wp[D + 1] = logf(click + 1) - logf(show + 1);
-                }
+    }
+    if (!any) return;
+    reinterpret_cast<float4*>(wp)[sub] = w;
+    if (KIND == OPT_ADAGRAD) {
+        if (sub == 0) {
+            *reinterpret_cast<float4*>(sp) = make_float4(g2sum, show, click, 0.f);  // no_show_days = 0
+            if (o.use_cvm) {
+                wp[D] = show;
+                wp[D + 1] = logf(click + 1) - logf(show + 1);
             }
-        } else {
-            reinterpret_cast<float4*>(sp)[sub] = a;
-            reinterpret_cast<float4*>(sp + D)[sub] = b;
-            if (sub == 0) sp[2 * D + 1] = __int_as_float(delta_show);
         }
+    } else {
+        reinterpret_cast<float4*>(sp)[sub] = a;
+        reinterpret_cast<float4*>(sp + D)[sub] = b;
+        if (sub == 0) sp[2 * D + 1] = __int_as_float(delta_show);
     }
 }
 

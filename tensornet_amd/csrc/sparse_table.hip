@@ -41,6 +41,16 @@ constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS 
 // takes the path of few launches (small_batch.h).
 constexpr size_t SMALL_MAX_LOOKUPS = 1u << 18;
 
+// A small batch of at most this many slots leaves every sign to the lane groups of k_small_apply: no launch of
+// k_apply_big.  With more slots a sign with SMALL_BIG_GROUP records or more goes to k_apply_big: a small batch's
+// kernels are as long as their longest chain, and the records of a sign applied one after the other by a lane
+// group (four elements per lane) take four times as long as by a wavefront (measured, 4096 x 26 slots, Adam:
+// the updates take 0.040 ms with every sign left to the lane groups, 0.017 + 0.015 ms with the threshold at 5,
+// 0.017 + 0.026 ms at 16; 1024 x 8 slots: 0.012 ms without k_apply_big, 0.009 + 0.009 ms with it).
+constexpr int SMALL_NO_BIG_SLOTS = 12;
+constexpr uint32_t SMALL_BIG_GROUP = 5;
+constexpr uint32_t BIG_GROUP_DEFAULT = 16;
+
 enum { FLOW_NONE = 0, FLOW_PULL = 1, FLOW_PUSH = 2 };
 
 struct HostStatus {
@@ -83,14 +93,16 @@ struct SparseTable {
     DevBuf pooled_ws;               // scratch of a push of pooled gradients (ordered lookups, reduced rows)
     size_t place_lds = 0, huge_lds = 0;  // dynamic LDS of k_place_lookups / k_order_huge on this device (0: not asked yet)
     // The path of few launches for small batches: its device state, the words in pinned memory its kernels
-    // report through ([0] a pull's status is on the host, [1] a push's signs are compared, [2] a push's status
-    // is on the host) with the numbers the host expects there next, the dynamic LDS k_small_slots may have.
+    // report through ([0] a pull's status is on the host, [1] a push's signs are compared) with the numbers the
+    // host expects there next, the dynamic LDS k_small_slots may have.
     SmallState* small_state = nullptr;
     uint32_t* hseq = nullptr;
-    uint32_t seq_pull = 0, seq_verify = 0, seq_apply = 0;
+    uint32_t seq_pull = 0, seq_verify = 0;
+    std::vector<int64_t> plan_counts;  // distinct signs per slot of the small pull that left the plan
     uint32_t small_calls = 0;  // (its parity: which set of bucket cursors the next small pull uses)
     size_t small_lds = 0;
     bool plan_small = false;   // the plan was left by a small pull: a push may take the small path, too
+    uint32_t plan_big_k = BIG_GROUP_DEFAULT;  // records from which the plan lists a sign as one for k_apply_big
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     // The slot descriptors of a call reach the device here while the caller's stream still runs the tail of the
@@ -504,7 +516,7 @@ size_t group_cap(size_t n) { return std::max<size_t>(16, n + n / 2); }
 
 // Signs with this many records or more are applied by one wavefront each
 // (k_apply_big); rows too wide for its LDS staging stay with the lane groups.
-constexpr uint32_t BIG_GROUP = 16;
+constexpr uint32_t BIG_GROUP = BIG_GROUP_DEFAULT;
 uint32_t big_threshold(const Store& s) { return s.D <= BIG_DIM_MAX ? BIG_GROUP : 0xFFFFFFFFu; }
 
 void carve_groups(Carver& c, Plan& p, size_t n) {
@@ -514,7 +526,7 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_cnt = c.take<uint32_t>(n);
     p.list = c.take<Member>(n);
     p.where_u = c.take<uint2>(n);
-    p.big_list = c.take<uint32_t>(n / BIG_GROUP + 64);
+    p.big_list = c.take<uint32_t>(n / std::min<uint32_t>(BIG_GROUP, SMALL_BIG_GROUP) + 64);  // (the lowest threshold a plan may use)
     p.newlist = c.take<uint32_t>(n);
     p.gaddr = c.take<const float*>(n);
 }
@@ -833,8 +845,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
 // stream beside it, forked from and joined back into the caller's stream by events.
 template <int KIND>
 int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
-                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready) {
-    const uint32_t big_k = big_threshold(s);
+                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready, uint32_t big_k) {
     const uint32_t ids_cap = (uint32_t)n_upper;
     const bool with_big = big_k != 0xFFFFFFFFu;
     const float* const* gaddr = (with_big && !src.infos && !src.flat) ? p.gaddr : nullptr;
@@ -889,33 +900,31 @@ int lanes_per_group(const Store& s, bool vec_ok) {
 
 // Applies the grouped records; n_upper bounds the number of records.
 // addr_ready: p.gaddr already holds the gradient addresses of the multi-record groups' records.
+// big_k: the number of records from which the plan's grouping listed a sign for k_apply_big (0: the table's default).
 int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
-                 hipStream_t st, bool addr_ready = false) {
+                 hipStream_t st, bool addr_ready = false, uint32_t big_k = 0) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     const int lpg = lanes_per_group(s, vec_ok);
+    if (big_k == 0) big_k = big_threshold(s);
     switch (o.kind) {
-        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
-        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
-        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready);
+        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
+        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
+        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
     }
 }
 
-// The updates of a small push: the signs with many records by k_apply_big (a sign has at most one record per
-// slot, so there are none below BIG_GROUP slots), every other group by one launch of k_small_apply, whose last
-// workgroup publishes the call's status.
+// The updates of a small push: every group by one launch of k_small_apply (which also tells the host that the
+// comparison launched before it is complete), but the signs with many records, if the plan lists any, by
+// k_apply_big after it.
 template <int KIND>
 int launch_small_apply_kind(SparseTable* t, int lpg, int N, const OptDev& o, const PushSrc& src, DevStatus* ds,
-                            const Plan& p, int64_t n_upper, hipStream_t st, const SmallPublish& pub) {
+                            const Plan& p, int64_t n_upper, hipStream_t st, uint32_t* host_seq, uint32_t seq) {
     const Store& s = t->store;
-    const uint32_t big_k = big_threshold(s);
-    if (big_k != 0xFFFFFFFFu && (uint32_t)N >= big_k)
-        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
-                      big_lds_bytes(s.D), st, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list,
-                      big_gbuf_floats(s.D), (const float* const*)nullptr);
+    const uint32_t big_k = t->plan_big_k;
 #define TN_LAUNCH_SMALL(LPG)                                                                                          \
     TN_LAUNCH((k_small_apply<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, o, src, \
-              ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, (uint32_t)n_upper, pub)
+              N, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, (uint32_t)n_upper, host_seq, seq)
     switch (lpg) {
         case 1: TN_LAUNCH_SMALL(1); break;
         case 2: TN_LAUNCH_SMALL(2); break;
@@ -925,16 +934,20 @@ int launch_small_apply_kind(SparseTable* t, int lpg, int N, const OptDev& o, con
         default: TN_LAUNCH_SMALL(32); break;
     }
 #undef TN_LAUNCH_SMALL
+    if (big_k != 0xFFFFFFFFu && (uint32_t)N >= big_k)
+        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / big_k + 1, 1, 16384)), dim3(64),
+                      big_lds_bytes(s.D), st, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list,
+                      big_gbuf_floats(s.D), (const float* const*)nullptr);
     return TN_OK;
 }
 
 int launch_small_apply(SparseTable* t, int lpg, int N, const PushSrc& src, DevStatus* ds, const Plan& p, int64_t n_upper,
-                       hipStream_t st, const SmallPublish& pub) {
+                       hipStream_t st, uint32_t* host_seq, uint32_t seq) {
     const OptDev o = make_optdev(t);
     switch (o.kind) {
-        case OPT_ADAGRAD: return launch_small_apply_kind<OPT_ADAGRAD>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
-        case OPT_ADAM: return launch_small_apply_kind<OPT_ADAM>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
-        default: return launch_small_apply_kind<OPT_FTRL>(t, lpg, N, o, src, ds, p, n_upper, st, pub);
+        case OPT_ADAGRAD: return launch_small_apply_kind<OPT_ADAGRAD>(t, lpg, N, o, src, ds, p, n_upper, st, host_seq, seq);
+        case OPT_ADAM: return launch_small_apply_kind<OPT_ADAM>(t, lpg, N, o, src, ds, p, n_upper, st, host_seq, seq);
+        default: return launch_small_apply_kind<OPT_FTRL>(t, lpg, N, o, src, ds, p, n_upper, st, host_seq, seq);
     }
 }
 
@@ -1583,26 +1596,28 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             DevStatus* ds = t->dplan;
             uint32_t* prow = w.first_of;  // row of the slot's distinct sign of rank r at [first lookup of the slot + r]
             TN_LAUNCH_LDS(k_small_slots, dim3(N), dim3(SMALL_THREADS), small_slots_lds(entries, w.nb2), st,
-                          reinterpret_cast<const SlotDesc*>(t->hstage), p.descs, p.lbase, p.ubase, N, (uint32_t)L, entries, s,
+                          reinterpret_cast<const SlotDesc*>(t->hstage), p.descs, p.lbase, N, (uint32_t)L, entries, s,
                           make_optdev(t), t->seed, p.vals_copy, p.u_of_gi, prow, w.nb2, cur, next, w.recs, w.rrow,
-                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
-            const size_t base_lds = 2 * ((size_t)N + 1) * sizeof(uint32_t);
-            const int tiles = (int)(((uint64_t)L * (uint64_t)(vec ? wdim / 4 : wdim) + 255) / 256);
+                          t->small_state);
+            const uint32_t big_k = N <= SMALL_NO_BIG_SLOTS || big_threshold(s) == 0xFFFFFFFFu ? 0xFFFFFFFFu : SMALL_BIG_GROUP;
+            t->plan_big_k = big_k;
+            // the grouping's first pass (one workgroup per second-level bucket) and, beside it, a thread per
+            // (lookup position, part of a row) for the variables
+            const int finish_blocks = (int)(((uint64_t)L * (uint64_t)(vec ? wdim / 4 : wdim) + GRP_THREADS - 1) / GRP_THREADS);
             if (vec)
-                TN_LAUNCH_LDS((k_small_finish<4>), dim3(tiles), dim3(256), base_lds, st, s, p.descs, p.lbase, p.ubase, N,
-                              (uint32_t)L, prow, p.u_of_gi);
+                TN_LAUNCH((k_small_group_finish<4>), dim3(w.nb2 + finish_blocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs,
+                          big_k, w.aux, w.bcounts, s, p.descs, p.lbase, p.ubase, N, (uint32_t)L, prow, p.u_of_gi,
+                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
             else
-                TN_LAUNCH_LDS((k_small_finish<1>), dim3(tiles), dim3(256), base_lds, st, s, p.descs, p.lbase, p.ubase, N,
-                              (uint32_t)L, prow, p.u_of_gi);
-            const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
-            TN_LAUNCH(k_group_count, dim3(bblocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs, big_threshold(s), w.aux,
-                      w.bcounts);
-            TN_LAUNCH((k_group_emit<true>), dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
+                TN_LAUNCH((k_small_group_finish<1>), dim3(w.nb2 + finish_blocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs,
+                          big_k, w.aux, w.bcounts, s, p.descs, p.lbase, p.ubase, N, (uint32_t)L, prow, p.u_of_gi,
+                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
+            TN_LAUNCH((k_group_emit<true>), dim3(w.nb2), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
                       (const uint4*)nullptr, w.bcounts, (const uint8_t*)nullptr, (const uint32_t*)nullptr, (uint32_t)L,
-                      big_threshold(s), p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
+                      big_k, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
                       p.grp_row, ds, p.ubase);
             TN_HIP(hipGetLastError());
-            // the call returns when the first launch has reported: what follows it is complete in stream order
+            // the call returns when the second launch has reported: what follows is complete in stream order
             TN_HIP(hipEventRecord(t->tail_ev, st));
             t->tail_recorded = true;
             t->pull_pending = true;
@@ -1629,9 +1644,11 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                 continue;
             }
             harvest(t);
+            t->plan_counts = t->last_counts;
             return take_latched(t);
         }
         t->plan_small = false;
+        t->plan_big_k = big_threshold(t->store);
         // Behind a push of the training loop the descriptors go in on the auxiliary stream, beside that push's
         // updates: those read the push's own descriptors and status block, and nothing of the scratch buffer.
         // (Same slot count: the arrays at the head of the plan buffer keep their places.)
@@ -1855,8 +1872,9 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     const int small_lpg = lanes_per_group(t->store, vec && t->store.wstride % 4 == 0);
     if (reuse && t->plan_small && !pooled && small_lpg != 0 && N <= SMALL_SLOTS) {
         // A small batch on the plan of its small pull: slot descriptors, comparison of the signs and click sums by
-        // one launch, the updates by one or two more, which also publish the status (small_batch.h).  The call's
-        // status block is the plan's: nothing of the next call runs beside this one.
+        // one launch, the updates by one or two more (small_batch.h).  The call's status block is the plan's:
+        // nothing of the next call runs beside this one.  The device has nothing to report: every sign of the plan
+        // has its row, and whether a gradient matrix has a row for every distinct sign of its slot is known here.
         carve_plan((char*)t->plan_buf.p, p, N, L);
         pd = p.push_descs;
         ds = t->dplan;
@@ -1872,32 +1890,28 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
         }
-        const uint32_t seq_v = ++t->seq_verify, seq_a = ++t->seq_apply;
+        const uint32_t seq_v = ++t->seq_verify;
         const int tiles = (int)((L + SMALL_TILE - 1) / SMALL_TILE);
         const size_t vlds = ((size_t)N + 1) * sizeof(uint32_t);
         if (clicks)
             TN_LAUNCH_LDS((k_small_verify<true>), dim3(tiles), dim3(256), vlds, st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
-                          ds, p.u_of_gi, p.where_u, p.list, t->small_state, &t->hpush->st.mismatch, t->hseq + 1, seq_v);
+                          ds, p.u_of_gi, p.where_u, p.list, &t->hpush->st.mismatch);
         else
             TN_LAUNCH_LDS((k_small_verify<false>), dim3(tiles), dim3(256), vlds, st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
-                          ds, p.u_of_gi, p.where_u, p.list, t->small_state, &t->hpush->st.mismatch, t->hseq + 1, seq_v);
-        SmallPublish pub{};
-        pub.state = t->small_state;
-        pub.ubase = p.ubase;
-        pub.n_ubase = (uint32_t)(N + 1);
-        pub.host_dst = reinterpret_cast<uint32_t*>(t->hpush);
-        pub.host_seq = t->hseq + 2;
-        pub.seq = seq_a;
-        TN_TRY(launch_small_apply(t, small_lpg, N, op_source(p, grad_dim, pd), ds, p, (int64_t)L, st, pub));
+                          ds, p.u_of_gi, p.where_u, p.list, &t->hpush->st.mismatch);
+        TN_TRY(launch_small_apply(t, small_lpg, N, op_source(p, grad_dim, pd), ds, p, (int64_t)L, st, t->hseq + 1, seq_v));
         TN_HIP(hipGetLastError());
         // the outcome of the comparison: the updates are queued behind it and do nothing on a mismatch
         TN_TRY(wait_reported(t->hseq + 1, seq_v, st, "SparseTablePush"));
         if (t->hpush->st.mismatch == 0) {
-            t->push_pending = true;
-            t->push_pub_on_side = false;
-            t->push_slots = N;
+            t->last_counts = t->plan_counts;
+            // (the records without a gradient row were left out by the update kernel, as on the other paths)
+            for (int s = 0; s < N; s++)
+                if (grad_rows[s] < t->plan_counts[s])
+                    return fail(TN_ERR_INVALID_ARGUMENT, std::string("sparse push: ") + dev_err_text(DEV_ERR_GRAD_ROWS) +
+                                                             " (slot " + std::to_string(s) + ")");
             return TN_OK;
         }
         reuse = false;  // another batch than the last pull's: analysed below
@@ -1923,7 +1937,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // op-level gradients (not pooled): the verify pass also works out the gradient addresses of the records
         // of the groups with several records (see k_member_grads)
         const PushSrc vsrc = op_source(p, grad_dim, pd);
-        const bool addr_in_verify = !pooled && big_threshold(t->store) != 0xFFFFFFFFu;
+        const bool addr_in_verify = !pooled && t->plan_big_k != 0xFFFFFFFFu;
         const float** vgaddr = addr_in_verify ? p.gaddr : nullptr;
         if (clicks) {
             if (t->plan_clicks_dirty)
@@ -1941,7 +1955,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // return at once when the mismatch flag is set.  The device never waits for the host.
         if (!t->plan_has_show) TN_TRY(launch_counts());
         TN_TRY(prepare_src());
-        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify));
+        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify, t->plan_big_k));
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
     }
