@@ -29,6 +29,7 @@ constexpr int SMALL_ITEMS = 4;                               // lookups per thre
 constexpr int SMALL_SLOT_MAX = SMALL_THREADS * SMALL_ITEMS;  // lookups of a slot at most
 constexpr int SMALL_SLOTS = GRP_SLOTS;                       // slots at most (the grouping's slot masks)
 constexpr int SMALL_NB2_MAX = 512;                           // second-level buckets at most
+constexpr int SMALL_PARTS_MAX = 4;                           // workgroups of k_small_slots per slot at most
 constexpr int SMALL_TILE = 1024;                             // lookups per workgroup of k_small_verify
 
 // What a slot's workgroup leaves for the one that finishes last.
@@ -40,7 +41,7 @@ struct SlotOut {
 // bucket cursors and clears the other for the call after it.
 struct SmallState {
     uint32_t cursor2[2][SMALL_NB2_MAX];
-    SlotOut slot_out[SMALL_SLOTS];
+    SlotOut slot_out[SMALL_SLOTS * SMALL_PARTS_MAX];  // one per workgroup of k_small_slots
 };
 
 // Bytes of dynamic LDS of k_small_slots for a table of `entries` entries and nb2 second-level buckets.
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     const SlotDesc* host_descs, SlotDesc* descs, uint32_t* lbase, int N, uint32_t L, uint32_t entries,
     Store s, OptDev o, uint64_t seed, uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ u_of_gi,
     uint32_t* __restrict__ prow, uint32_t nb2, uint32_t* cursor2, uint32_t* cursor2_next, GroupRec* __restrict__ recs,
-    uint32_t* __restrict__ rrow, SmallState* state) {
+    uint32_t* __restrict__ rrow, SmallState* state, uint32_t parts) {
     extern __shared__ unsigned long long smem64[];
     unsigned long long* keys = smem64;  // entry `entries`: the sign EMPTY_KEY itself
     uint32_t* minpos = reinterpret_cast<uint32_t*>(keys + entries + 1);
@@ -65,7 +66,12 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     __shared__ SlotDesc sd;
     __shared__ uint32_t wsum[SMALL_THREADS / 64];
     __shared__ uint32_t sh_new, sh_err;
-    const int sl = blockIdx.x;
+    // `parts` workgroups per slot: each of them works out the whole remap of the slot (in LDS, the same in all),
+    // then takes every parts-th distinct sign through the table and every parts-th wavefront's lookups to the
+    // outputs.  A CU sustains about 0.2 random 64-byte reads per nanosecond: the 2600 probes of a slot of 4096
+    // lookups keep one CU busy for 13 us, while most of the device has nothing to do.
+    const int sl = blockIdx.x / parts;
+    const uint32_t part = blockIdx.x % parts;
     const uint32_t tid = threadIdx.x;
     // the slot's descriptor comes straight out of the host's staging buffer (one round trip over the bus,
     // in flight while the tables are cleared)
@@ -77,7 +83,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
         cnts[i] = 0;
     }
     for (uint32_t i = tid; i < nb2; i += SMALL_THREADS) hist2[i] = 0;
-    if (sl == 0)
+    if (blockIdx.x == 0)
         for (uint32_t i = tid; i < (uint32_t)SMALL_NB2_MAX; i += SMALL_THREADS) cursor2_next[i] = 0;
     if (tid == 0) {
         sh_new = 0;
@@ -85,7 +91,7 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     }
     __syncthreads();
     const SlotDesc d = sd;
-    if (tid == 0) {
+    if (tid == 0 && part == 0) {
         descs[sl] = d;
         lbase[sl] = d.lbase;
         if (sl == N - 1) lbase[N] = L;
@@ -140,67 +146,109 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     uint32_t total = 0;
     uint32_t rank0 = block_excl_scan<uint32_t, SMALL_THREADS / 64>(__popc(firsts), wsum, &total);  // (barriers inside)
     // the entry of a distinct sign now takes its rank in place of the position (every thread has read the positions)
-    uint32_t shows[SMALL_ITEMS];
+    uint32_t mine = 0;  // the distinct signs this workgroup takes through the table
     {
         uint32_t r = rank0;
 #pragma unroll
-        for (int j = 0; j < SMALL_ITEMS; j++) {
-            shows[j] = 0;
+        for (int j = 0; j < SMALL_ITEMS; j++)
             if (firsts & (1u << j)) {
-                shows[j] = cnts[h[j]];  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+                if (r % parts == part) mine |= 1u << j;
                 minpos[h[j]] = r++;
             }
-        }
     }
     __syncthreads();
-#pragma unroll
-    for (int j = 0; j < SMALL_ITEMS; j++) {
-        if (p0 + j >= n) continue;
-        const uint32_t r = minpos[h[j]];
-        d.mapped[p0 + j] = (int64_t)r;
-        vals_copy[d.lbase + p0 + j] = sg[j];
-        u_of_gi[d.lbase + p0 + j] = r | ((firsts & (1u << j)) ? FIRST_BIT : 0u);  // relative to the slot until k_small_finish
-    }
-    // lookup-or-insert of the distinct signs (optimizer_kernel.h:299-308), the first key groups of a thread's
-    // signs in flight together.  A row this workgroup inserts is listed in LDS (the key table is dead) and filled
-    // further down by all threads: one lane of a wavefront drawing the normal deviates of a row would hold up
-    // the other sixty-three.  The rows are read by the next launch only: another slot's workgroup may be
-    // filling the row of a sign that this one finds claimed.
+    // lookup-or-insert of the distinct signs (optimizer_kernel.h:299-308; the probe sequence of probe_slot).  A
+    // thread's signs go through their sequences side by side: the key groups of all of them are read in one round
+    // trip, the compare-and-swaps of those that found a free slot go out together, and so on round by round --
+    // one after the other, a wavefront would spend a round trip on every sign that needs a second group or
+    // claims a slot, in every one of its four places.  A row this workgroup inserts is listed in LDS (the key
+    // table is dead) and filled further down by all threads: one lane of a wavefront drawing the normal deviates
+    // of a row would hold up the other sixty-three.  The rows are read by the next launch only: another slot's
+    // workgroup may be filling the row of a sign that this one finds claimed.
     unsigned long long* new_sign = keys;                                   // [n] at most
     uint32_t* new_row = reinterpret_cast<uint32_t*>(keys + n);            // (the table has 2 n + 1 entries or more)
-    uint32_t rows[SMALL_ITEMS], place[SMALL_ITEMS], bucket[SMALL_ITEMS];
-    uint32_t err = 0;
+    uint32_t rows[SMALL_ITEMS], place[SMALL_ITEMS];
+    uint32_t err = 0, fresh = 0;
     {
         uint64_t at[SMALL_ITEMS];
-        ulonglong2 q[SMALL_ITEMS][4];
+        uint32_t live = 0;
 #pragma unroll
         for (int j = 0; j < SMALL_ITEMS; j++) {
+            rows[j] = NO_ROW;
             at[j] = 0;
-            if ((firsts & (1u << j)) && sg[j] != EMPTY_KEY) {
+            if (!(mine & (1u << j))) continue;
+            if (sg[j] == EMPTY_KEY) {
+                bool is_new = false;
+                rows[j] = probe_slot<true>(s, sg[j], is_new);
+                if (is_new) fresh |= 1u << j;
+            } else {
                 at[j] = home_group(sg[j], s.cap);
+                live |= 1u << j;
+            }
+        }
+        const uint64_t groups = s.cap / PROBE_WIDTH;
+        for (uint64_t round = 0; live != 0 && round < 2 * groups + 64; round++) {
+            ulonglong2 q[SMALL_ITEMS][4];
+#pragma unroll
+            for (int j = 0; j < SMALL_ITEMS; j++) {
+                if (!(live & (1u << j))) continue;
                 const ulonglong2* g = reinterpret_cast<const ulonglong2*>(s.keys + at[j]);
                 q[j][0] = g[0], q[j][1] = g[1], q[j][2] = g[2], q[j][3] = g[3];
+            }
+            uint32_t claim = 0, where[SMALL_ITEMS];
+#pragma unroll
+            for (int j = 0; j < SMALL_ITEMS; j++) {
+                where[j] = PROBE_WIDTH;
+                if (!(live & (1u << j))) continue;
+                const uint64_t k[PROBE_WIDTH] = {q[j][0].x, q[j][0].y, q[j][1].x, q[j][1].y,
+                                                 q[j][2].x, q[j][2].y, q[j][3].x, q[j][3].y};
+                bool free_slot = false;
+#pragma unroll
+                for (int e = PROBE_WIDTH - 1; e >= 0; e--)  // the first slot of the group that holds the sign or is free
+                    if (k[e] == sg[j] || k[e] == EMPTY_KEY) {
+                        where[j] = (uint32_t)e;
+                        free_slot = k[e] == EMPTY_KEY;
+                    }
+                if (where[j] == PROBE_WIDTH) {
+                    at[j] = at[j] + PROBE_WIDTH >= s.cap ? 0 : at[j] + PROBE_WIDTH;  // on to the next group
+                } else if (free_slot) {
+                    claim |= 1u << j;
+                } else {
+                    rows[j] = (uint32_t)(at[j] + where[j]);
+                    live &= ~(1u << j);
+                }
+            }
+            uint64_t old[SMALL_ITEMS];
+#pragma unroll
+            for (int j = 0; j < SMALL_ITEMS; j++)
+                if (claim & (1u << j)) old[j] = atomicCAS(ull(&s.keys[at[j] + where[j]]), EMPTY_KEY, sg[j]);
+#pragma unroll
+            for (int j = 0; j < SMALL_ITEMS; j++) {
+                if (!(claim & (1u << j))) continue;
+                if (old[j] == EMPTY_KEY || old[j] == sg[j]) {
+                    rows[j] = (uint32_t)(at[j] + where[j]);
+                    if (old[j] == EMPTY_KEY) fresh |= 1u << j;
+                    live &= ~(1u << j);
+                }  // else another sign took the slot: the group is read again
             }
         }
         uint32_t r = rank0;
 #pragma unroll
         for (int j = 0; j < SMALL_ITEMS; j++) {
             if (!(firsts & (1u << j))) continue;
-            bool is_new = false;
-            const uint32_t row = sg[j] == EMPTY_KEY
-                                     ? probe_slot<true>(s, sg[j], is_new)
-                                     : probe_from<true>(s, sg[j], at[j], q[j][0], q[j][1], q[j][2], q[j][3], is_new);
-            if (row == NO_ROW) {
+            if (!(mine & (1u << j))) {
+                r++;
+                continue;
+            }
+            if (rows[j] == NO_ROW) {
                 err |= DEV_ERR_TABLE_FULL;
-            } else if (is_new) {
+            } else if (fresh & (1u << j)) {
                 const uint32_t k = atomicAdd(&sh_new, 1u);
                 new_sign[k] = sg[j];
-                new_row[k] = row;
+                new_row[k] = rows[j];
             }
-            rows[j] = row;
-            prow[d.lbase + r] = row;
-            bucket[j] = group_bucket(sg[j], nb2);
-            place[j] = atomicAdd(&hist2[bucket[j]], 1u);
+            prow[d.lbase + r] = rows[j];
+            place[j] = atomicAdd(&hist2[group_bucket(sg[j], nb2)], 1u);
             r++;
         }
     }
@@ -225,14 +273,19 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
 #pragma unroll
         for (int j = 0; j < SMALL_ITEMS; j++) {
             if (!(firsts & (1u << j))) continue;
-            const uint32_t at = hist2[bucket[j]] + place[j];
+            if (!(mine & (1u << j))) {
+                r++;
+                continue;
+            }
+            const uint32_t b = group_bucket(sg[j], nb2);
+            const uint32_t at = hist2[b] + place[j];
             if (at < (uint32_t)GRP_CAP) {
                 GroupRec rec;
                 rec.sign = sg[j];
                 rec.gi = r;  // the record's rank in its slot (k_group_emit<true> adds the slot's base)
-                rec.cnt = shows[j] | ((uint32_t)sl << 24);
-                recs[(size_t)bucket[j] * GRP_CAP + at] = rec;
-                rrow[(size_t)bucket[j] * GRP_CAP + at] = rows[j];
+                rec.cnt = cnts[h[j]] | ((uint32_t)sl << 24);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
+                recs[(size_t)b * GRP_CAP + at] = rec;
+                rrow[(size_t)b * GRP_CAP + at] = rows[j];
             } else {
                 err |= DEV_ERR_REMAP_OVERFLOW;  // the host repeats the call with more buckets
             }
@@ -241,13 +294,22 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     }
     if (err) atomicOr(&sh_err, err);
     __syncthreads();
+    // the lookups' outputs last: nothing in this kernel waits for these stores
+#pragma unroll
+    for (int j = 0; j < SMALL_ITEMS; j++) {
+        if (p0 + j >= n || (tid >> 6) % parts != part) continue;
+        const uint32_t r = minpos[h[j]];
+        d.mapped[p0 + j] = (int64_t)r;
+        vals_copy[d.lbase + p0 + j] = sg[j];
+        u_of_gi[d.lbase + p0 + j] = r | ((firsts & (1u << j)) ? FIRST_BIT : 0u);  // relative to the slot until the next launch
+    }
     if (tid == 0) {  // for the next launch, which adds up the slots' counts and publishes the call's status
         SlotOut out;
         out.n_unique = total;
         out.n_new = sh_new;
         out.err = sh_err;
         out.pad = 0;
-        state->slot_out[sl] = out;
+        state->slot_out[blockIdx.x] = out;
     }
 }
 
@@ -263,8 +325,8 @@ __global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
     uint32_t nb2, const uint32_t* __restrict__ cursor2, const GroupRec* __restrict__ recs, uint32_t big_k,
     uint2* __restrict__ aux, uint4* __restrict__ bcounts, Store s, const SlotDesc* __restrict__ descs,
     const uint32_t* __restrict__ lbase, uint32_t* ubase, int N, uint32_t L, const uint32_t* __restrict__ prow,
-    uint32_t* __restrict__ u_of_gi, const SmallState* __restrict__ state, DevStatus* status, uint32_t* host_dst,
-    uint32_t* host_seq, uint32_t seq) {
+    uint32_t* __restrict__ u_of_gi, const SmallState* __restrict__ state, uint32_t parts, DevStatus* status,
+    uint32_t* host_dst, uint32_t* host_seq, uint32_t seq) {
     __shared__ GroupCountLds lds;
     if (blockIdx.x < nb2) {
         group_count_bucket(blockIdx.x, lds, cursor2, recs, big_k, aux, bcounts);
@@ -277,13 +339,14 @@ __global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
     uint32_t* misc = reinterpret_cast<uint32_t*>(lds.rech);  // [0] new rows, [1] error flags, [2] distinct signs
     const uint32_t tid = threadIdx.x;
     const bool publisher = blockIdx.x == nb2;
+    static_assert(SMALL_SLOTS * SMALL_PARTS_MAX <= GRP_THREADS, "a thread per workgroup of k_small_slots");
     uint32_t mine = 0, nn = 0, ee = 0;
-    if (tid < (uint32_t)N) {
+    if (tid < (uint32_t)N * parts) {  // (every workgroup of a slot leaves the slot's count, and its own share of the rest)
         const SlotOut so = state->slot_out[tid];
-        mine = so.n_unique;
         nn = so.n_new;
         ee = so.err;
     }
+    if (tid < (uint32_t)N) mine = state->slot_out[tid * parts].n_unique;
     for (uint32_t i = tid; i <= (uint32_t)N; i += GRP_THREADS) lb[i] = lbase[i];
     if (tid < 2) misc[tid] = 0;
     const uint32_t base = block_excl_scan<uint32_t, GRP_THREADS / 64>(mine, wsum, &misc[2]);  // (barriers inside)

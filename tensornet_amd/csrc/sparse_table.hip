@@ -1595,10 +1595,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             const Store& s = t->store;
             DevStatus* ds = t->dplan;
             uint32_t* prow = w.first_of;  // row of the slot's distinct sign of rank r at [first lookup of the slot + r]
-            TN_LAUNCH_LDS(k_small_slots, dim3(N), dim3(SMALL_THREADS), small_slots_lds(entries, w.nb2), st,
+            // workgroups per slot: about a thousand lookups' worth of table probes each, within the device's CUs
+            uint32_t parts = (uint32_t)std::min<size_t>(SMALL_PARTS_MAX, (max_len + 1023) / 1024);
+            while (parts > 1 && (size_t)N * parts > 256) parts--;
+            if (parts < 1) parts = 1;
+            TN_LAUNCH_LDS(k_small_slots, dim3(N * parts), dim3(SMALL_THREADS), small_slots_lds(entries, w.nb2), st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.descs, p.lbase, N, (uint32_t)L, entries, s,
                           make_optdev(t), t->seed, p.vals_copy, p.u_of_gi, prow, w.nb2, cur, next, w.recs, w.rrow,
-                          t->small_state);
+                          t->small_state, parts);
             const uint32_t big_k = N <= SMALL_NO_BIG_SLOTS || big_threshold(s) == 0xFFFFFFFFu ? 0xFFFFFFFFu : SMALL_BIG_GROUP;
             t->plan_big_k = big_k;
             // the grouping's first pass (one workgroup per second-level bucket) and, beside it, a thread per
@@ -1607,11 +1611,11 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             if (vec)
                 TN_LAUNCH((k_small_group_finish<4>), dim3(w.nb2 + finish_blocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs,
                           big_k, w.aux, w.bcounts, s, p.descs, p.lbase, p.ubase, N, (uint32_t)L, prow, p.u_of_gi,
-                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
+                          t->small_state, parts, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
             else
                 TN_LAUNCH((k_small_group_finish<1>), dim3(w.nb2 + finish_blocks), dim3(GRP_THREADS), st, w.nb2, cur, w.recs,
                           big_k, w.aux, w.bcounts, s, p.descs, p.lbase, p.ubase, N, (uint32_t)L, prow, p.u_of_gi,
-                          t->small_state, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
+                          t->small_state, parts, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
             TN_LAUNCH((k_group_emit<true>), dim3(w.nb2), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
                       (const uint4*)nullptr, w.bcounts, (const uint8_t*)nullptr, (const uint32_t*)nullptr, (uint32_t)L,
                       big_k, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
