@@ -29,7 +29,8 @@ constexpr int SMALL_ITEMS = 4;                               // lookups per thre
 constexpr int SMALL_SLOT_MAX = SMALL_THREADS * SMALL_ITEMS;  // lookups of a slot at most
 constexpr int SMALL_SLOTS = GRP_SLOTS;                       // slots at most (the grouping's slot masks)
 constexpr int SMALL_NB2_MAX = 512;                           // second-level buckets at most
-constexpr int SMALL_PARTS_MAX = 4;                           // workgroups of k_small_slots per slot at most
+constexpr int SMALL_PARTS_MAX = 8;                           // workgroups of k_small_slots per slot at most
+constexpr int SMALL_SLOT_WORKGROUPS = 256;                   // ... and for all slots together
 constexpr int SMALL_TILE = 1024;                             // lookups per workgroup of k_small_verify
 
 // What a slot's workgroup leaves for the one that finishes last.
@@ -41,7 +42,7 @@ struct SlotOut {
 // bucket cursors and clears the other for the call after it.
 struct SmallState {
     uint32_t cursor2[2][SMALL_NB2_MAX];
-    SlotOut slot_out[SMALL_SLOTS * SMALL_PARTS_MAX];  // one per workgroup of k_small_slots
+    SlotOut slot_out[SMALL_SLOT_WORKGROUPS];  // one per workgroup of k_small_slots
 };
 
 // Bytes of dynamic LDS of k_small_slots for a table of `entries` entries and nb2 second-level buckets.
@@ -69,7 +70,8 @@ __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     // `parts` workgroups per slot: each of them works out the whole remap of the slot (in LDS, the same in all),
     // then takes every parts-th distinct sign through the table and every parts-th wavefront's lookups to the
     // outputs.  A CU sustains about 0.2 random 64-byte reads per nanosecond: the 2600 probes of a slot of 4096
-    // lookups keep one CU busy for 13 us, while most of the device has nothing to do.
+    // lookups keep one CU busy for 13 us (measured with the device's clock around the kernel's phases), while
+    // most of the device has nothing to do.
     const int sl = blockIdx.x / parts;
     const uint32_t part = blockIdx.x % parts;
     const uint32_t tid = threadIdx.x;
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
     uint32_t* misc = reinterpret_cast<uint32_t*>(lds.rech);  // [0] new rows, [1] error flags, [2] distinct signs
     const uint32_t tid = threadIdx.x;
     const bool publisher = blockIdx.x == nb2;
-    static_assert(SMALL_SLOTS * SMALL_PARTS_MAX <= GRP_THREADS, "a thread per workgroup of k_small_slots");
+    static_assert(SMALL_SLOT_WORKGROUPS <= GRP_THREADS && SMALL_SLOTS <= SMALL_SLOT_WORKGROUPS, "a thread per workgroup of k_small_slots");
     uint32_t mine = 0, nn = 0, ee = 0;
     if (tid < (uint32_t)N * parts) {  // (every workgroup of a slot leaves the slot's count, and its own share of the rest)
         const SlotOut so = state->slot_out[tid];

@@ -1595,10 +1595,9 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             const Store& s = t->store;
             DevStatus* ds = t->dplan;
             uint32_t* prow = w.first_of;  // row of the slot's distinct sign of rank r at [first lookup of the slot + r]
-            // workgroups per slot: about a thousand lookups' worth of table probes each, within the device's CUs
-            uint32_t parts = (uint32_t)std::min<size_t>(SMALL_PARTS_MAX, (max_len + 1023) / 1024);
-            while (parts > 1 && (size_t)N * parts > 256) parts--;
-            if (parts < 1) parts = 1;
+            // workgroups per slot: about five hundred lookups' worth of table probes each, within the device's CUs
+            uint32_t parts = (uint32_t)std::max<size_t>(1, std::min<size_t>(SMALL_PARTS_MAX, (max_len + 511) / 512));
+            while (parts > 1 && (size_t)N * parts > (size_t)SMALL_SLOT_WORKGROUPS) parts--;
             TN_LAUNCH_LDS(k_small_slots, dim3(N * parts), dim3(SMALL_THREADS), small_slots_lds(entries, w.nb2), st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.descs, p.lbase, N, (uint32_t)L, entries, s,
                           make_optdev(t), t->seed, p.vals_copy, p.u_of_gi, prow, w.nb2, cur, next, w.recs, w.rrow,
