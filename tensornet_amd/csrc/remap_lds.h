@@ -832,7 +832,7 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                                                     uint2* __restrict__ where_u,
                                                     const uint32_t* __restrict__ rrow,
                                                     uint32_t* __restrict__ grp_row, DevStatus* status,
-                                                    const uint32_t* __restrict__ ubase) {
+                                                    const uint32_t* __restrict__ ubase, uint32_t n_slots) {
     // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
     // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
     __shared__ Member s_list[GRP_CAP];
@@ -840,6 +840,9 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
     __shared__ uint32_t s_off[GRP_CAP], s_row[GRP_CAP];
     __shared__ uint16_t s_cnt[GRP_CAP];  // at most GRP_SLOTS records per group
     __shared__ uint4 s_part[EMIT_THREADS / 64];
+    __shared__ uint32_t s_ub[SLOT_RANKS ? GRP_SLOTS + 1 : 1];  // the slots' bases (a small batch: one round trip less per record)
+    if (SLOT_RANKS)
+        for (uint32_t i = threadIdx.x; i <= n_slots && i <= (uint32_t)GRP_SLOTS; i += EMIT_THREADS) s_ub[i] = ubase[i];
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
@@ -850,7 +853,8 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
             const uint32_t i = j * EMIT_THREADS + threadIdx.x;
-            if (i < n) {
+            // (a small batch reads the bucket's whole room, wanted or not: the loads do not wait for its count then)
+            if (SLOT_RANKS || i < n) {
                 rs[j] = recs[first + i];
                 as[j] = aux[first + i];
                 rows[j] = rrow[first + i];
@@ -894,7 +898,7 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++)
             if (j * EMIT_THREADS + threadIdx.x < n)
-                us[j] = SLOT_RANKS ? ubase[rs[j].cnt >> 24] + rs[j].gi : rank_of(flag8, wordpre, rs[j].gi);
+                us[j] = SLOT_RANKS ? s_ub[(rs[j].cnt >> 24) & (GRP_SLOTS - 1)] + rs[j].gi : rank_of(flag8, wordpre, rs[j].gi);
 #pragma unroll
         for (int j = 0; j < EMIT_RECS; j++) {
             if (j * EMIT_THREADS + threadIdx.x >= n) continue;

@@ -339,9 +339,20 @@ __global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
     uint32_t* ub = reinterpret_cast<uint32_t*>(lds.mhi);  // ub[N + 1]
     uint32_t* wsum = reinterpret_cast<uint32_t*>(lds.sh);
     uint32_t* misc = reinterpret_cast<uint32_t*>(lds.rech);  // [0] new rows, [1] error flags, [2] distinct signs
+    SlotDesc* sd = reinterpret_cast<SlotDesc*>(lds.keys);  // the slots' descriptors (N <= SMALL_SLOTS: 8 KB of the 16)
     const uint32_t tid = threadIdx.x;
     const bool publisher = blockIdx.x == nb2;
     static_assert(SMALL_SLOT_WORKGROUPS <= GRP_THREADS && SMALL_SLOTS <= SMALL_SLOT_WORKGROUPS, "a thread per workgroup of k_small_slots");
+    // what this thread moves: one 16-byte (or 4-byte) part of the row of one lookup position.  Its row number and
+    // the descriptors are read at once, beside the slots' counts: one round trip instead of three in a row.
+    const uint32_t chunks = (uint32_t)(s.wdim / VEC);
+    const uint64_t t = (uint64_t)(blockIdx.x - nb2) * GRP_THREADS + tid;
+    const bool in_range = t < (uint64_t)L * chunks;
+    const uint32_t gi = in_range ? (uint32_t)(t / chunks) : 0u;
+    const uint32_t c = (uint32_t)(t - (uint64_t)gi * chunks);
+    const uint32_t row = in_range ? prow[gi] : NO_ROW;
+    for (uint32_t i = tid; i < (uint32_t)N * (uint32_t)(sizeof(SlotDesc) / 4); i += GRP_THREADS)
+        reinterpret_cast<uint32_t*>(sd)[i] = reinterpret_cast<const uint32_t*>(descs)[i];
     uint32_t mine = 0, nn = 0, ee = 0;
     if (tid < (uint32_t)N * parts) {  // (every workgroup of a slot leaves the slot's count, and its own share of the rest)
         const SlotOut so = state->slot_out[tid];
@@ -382,19 +393,14 @@ __global__ __launch_bounds__(GRP_THREADS) void k_small_group_finish(
         if (tid == 0) host_store(host_seq, seq);
     }
     __syncthreads();
-    // one thread per (position, part of the row): few rows per thread would leave the rows' round trips in a queue
-    const uint32_t chunks = (uint32_t)(s.wdim / VEC);
-    const uint64_t t = (uint64_t)(blockIdx.x - nb2) * GRP_THREADS + tid;
-    if (t >= (uint64_t)L * chunks) return;
-    const uint32_t gi = (uint32_t)(t / chunks);
-    const uint32_t c = (uint32_t)(t - (uint64_t)gi * chunks);
+    // (one thread per position and part of the row: few rows per thread would leave the rows' round trips in a queue)
+    if (!in_range) return;
     const int sl = find_slot(lb, N, gi);
     if (c == 0) u_of_gi[gi] += ub[sl];
     const uint32_t r = gi - lb[sl];
     if (r >= ub[sl + 1] - ub[sl]) return;  // beyond the slot's distinct signs
-    const SlotDesc& d = descs[sl];
+    const SlotDesc& d = sd[sl];
     if ((int64_t)r >= d.rows) return;      // the host reports the variable as too small
-    const uint32_t row = prow[gi];
     if (row > s.cap) return;  // NO_ROW (table full): never address the table with it
     if (VEC == 4) {
         const float4 v = *reinterpret_cast<const float4*>(s.w + (uint64_t)row * s.wstride + c * 4);

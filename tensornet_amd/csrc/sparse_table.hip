@@ -824,7 +824,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         TN_LAUNCH((k_group_emit<false>), dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
                   own_offsets ? nullptr : w.bbase, w.bcounts, w.flag8, w.wordpre, L, big_threshold(s),
                   p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds,
-                  (const uint32_t*)nullptr);
+                  (const uint32_t*)nullptr, 0u);
         return TN_OK;  // the rows were found beside the grouping
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
@@ -1618,7 +1618,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             TN_LAUNCH((k_group_emit<true>), dim3(w.nb2), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
                       (const uint4*)nullptr, w.bcounts, (const uint8_t*)nullptr, (const uint32_t*)nullptr, (uint32_t)L,
                       big_k, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
-                      p.grp_row, ds, p.ubase);
+                      p.grp_row, ds, p.ubase, (uint32_t)N);
             TN_HIP(hipGetLastError());
             // the call returns when the second launch has reported: what follows is complete in stream order
             TN_HIP(hipEventRecord(t->tail_ev, st));
