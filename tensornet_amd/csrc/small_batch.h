@@ -12,8 +12,8 @@
 //                                distinct indices made global
 //         k_group_emit<true>     the groups of equal signs over all slots, as ever
 //   push  k_small_verify         slot descriptors in, comparison with the plan's signs, click sums
-//         k_small_apply          every group by one launch (tells the host that the comparison is complete)
-//         k_apply_big            with more than 12 slots: the signs with 5 records or more
+//         k_small_apply          every group by one launch (tells the host that the comparison is complete); with
+//                                more than 12 slots the signs with 5 records or more by wavefronts of their own in it
 //
 // Workgroups of one launch never wait for each other, and none needs another's results: what needs them runs
 // in the next launch.
@@ -479,18 +479,29 @@ __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs
     }
 }
 
-// Every group of the plan that k_apply_big does not take, one record or several, by one launch (the
-// lane groups of k_apply_vec, the records of a sign four at a time).  Nothing is reported to the host: on
-// the plan of the last pull every sign has its row, and the host has compared the slots' distinct counts with
-// the rows of the gradient matrices itself.
+// Bytes of dynamic LDS of k_small_apply when its launch includes the workgroups for the signs with many records:
+// per wavefront the staging and the row of apply_big_groups, then its pointer, count, flag and divisor arrays.
+inline size_t small_apply_wave_lds(int D) { return align_up(big_lds_bytes(D), 8) + BIG_CHUNK * (8 + 4 + 4 + 4); }
+inline size_t small_apply_big_lds(int D) { return 4 * small_apply_wave_lds(D); }
+
+// The updates of a small push by one launch.  The first big_blocks workgroups (if the plan lists signs with many
+// records; they start first, their chains are the longest): each of their wavefronts takes such signs the way
+// k_apply_big does -- as a launch of its own that kernel costs a small batch as much again as this one.  The
+// workgroups after those: every group with fewer than big_k records, one record or several, by the lane groups
+// of k_apply_vec, the records of a sign four at a time.
+// Nothing is reported to the host but that this kernel runs, which tells it that the comparison of the signs,
+// launched before, is complete: on the plan of the last pull every sign has its row, and the host has compared
+// the slots' distinct counts with the rows of the gradient matrices itself.
 template <int KIND, int LPG>
 __global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc src, int N, DevStatus* status,
                                                      const uint32_t* __restrict__ grp_row,
                                                      const uint32_t* __restrict__ grp_off,
                                                      const uint32_t* __restrict__ grp_cnt,
                                                      const Member* __restrict__ list, uint32_t big_k,
-                                                     uint32_t ids_cap, uint32_t* host_seq, uint32_t seq) {
-    // this kernel runs: the comparison of the signs, launched before it, is complete
+                                                     uint32_t ids_cap, uint32_t* host_seq, uint32_t seq,
+                                                     uint32_t big_blocks, const uint32_t* __restrict__ big_list,
+                                                     int gbuf_floats, uint32_t wave_lds, uint32_t wave_arrays) {
+    extern __shared__ unsigned long long big_lds[];  // (only the first big_blocks workgroups use it)
     if (blockIdx.x == 0 && threadIdx.x == 0) host_store(host_seq, seq);
     // the slots' gradient matrices and bases from LDS: one round trip less in every record's chain of loads
     __shared__ SlotDesc sd[SMALL_SLOTS];
@@ -506,11 +517,24 @@ __global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc 
     if (stop) return;
     src.descs = sd;
     src.ubase = ub;
+    if (blockIdx.x < big_blocks) {
+        const int wave = (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63);
+        char* base = reinterpret_cast<char*>(big_lds) + (size_t)wave * wave_lds;  // (wave_arrays: where the arrays start in it)
+        float* gbuf = reinterpret_cast<float*>(base);
+        const float** gptr = reinterpret_cast<const float**>(base + wave_arrays);
+        int* gshow = reinterpret_cast<int*>(gptr + BIG_CHUNK);
+        int* gok = gshow + BIG_CHUNK;
+        float* den = reinterpret_cast<float*>(gok + BIG_CHUNK);
+        apply_big_groups<KIND>(s, o, src, status, big_list, grp_row, grp_off, grp_cnt, list, gbuf_floats, nullptr, gbuf,
+                               gptr, gshow, gok, den, lane, blockIdx.x * 4 + (uint32_t)wave, big_blocks * 4,
+                               [] { wave_sync(); });
+        return;
+    }
     const int sub = threadIdx.x % LPG;
     const int lane0 = (int)__lane_id() - sub;
-    const uint32_t gstride = gridDim.x * (blockDim.x / LPG);
+    const uint32_t gstride = (gridDim.x - big_blocks) * (blockDim.x / LPG);
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
-    for (uint32_t t = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
+    for (uint32_t t = (blockIdx.x - big_blocks) * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
         const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;

@@ -1676,24 +1676,25 @@ inline size_t big_lds_bytes(int D) { return (size_t)(big_gbuf_floats(D) + 3 * D)
 // then the records are applied strictly in order -- for AdaGrad the g2sum
 // chain by one lane, the square roots by one lane per record, the element
 // updates by one lane per element.
-template <int KIND>
-__global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src, DevStatus* status,
-                                                  const uint32_t* __restrict__ big_list,
-                                                  const uint32_t* __restrict__ grp_row,
-                                                  const uint32_t* __restrict__ grp_off,
-                                                  const uint32_t* __restrict__ grp_cnt,
-                                                  const Member* __restrict__ list, int gbuf_floats,
-                                                  const float* const* __restrict__ gaddr) {
-    extern __shared__ float gbuf[];  // gbuf_floats floats of staging, then the row: rw[D], ra[D], rb[D]
-    __shared__ const float* gptr[BIG_CHUNK];
-    __shared__ int gshow[BIG_CHUNK], gok[BIG_CHUNK];
-    __shared__ float den[BIG_CHUNK];
+// The groups big_list[first], big_list[first + stride], ... by the wavefront that calls it (lane = the thread's
+// lane).  gbuf: gbuf_floats floats of staging followed by the row (rw[D], ra[D], rb[D]); gptr, gshow, gok,
+// den: BIG_CHUNK entries each, all in LDS and the wavefront's own.  sync(): makes what the lanes wrote to that
+// LDS visible to each other (a workgroup of one wavefront: __syncthreads; a wavefront among others: wave_sync).
+template <int KIND, typename Sync>
+__device__ __forceinline__ void apply_big_groups(const Store& s, const OptDev& o, const PushSrc& src, DevStatus* status,
+                                                 const uint32_t* __restrict__ big_list,
+                                                 const uint32_t* __restrict__ grp_row,
+                                                 const uint32_t* __restrict__ grp_off,
+                                                 const uint32_t* __restrict__ grp_cnt,
+                                                 const Member* __restrict__ list, int gbuf_floats,
+                                                 const float* const* __restrict__ gaddr, float* gbuf, const float** gptr,
+                                                 int* gshow, int* gok, float* den, int lane, uint32_t first,
+                                                 uint32_t stride, Sync sync) {
     const int D = s.D;
     float* rw = gbuf + gbuf_floats;
     float* ra = rw + D;
     float* rb = ra + D;
     const int Dp = D + 1;  // padded staging row: lanes walking down a column hit different banks
-    const int lane = threadIdx.x;
     // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
     if (status->mismatch | status->abort) return;
     const uint32_t n_big = status->n_big;
@@ -1704,7 +1705,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
     // D divides 64: the lanes tile (records, elements) as lane = record * D + element
     const bool tiled = D <= 64 && 64 % D == 0;
     const int li = tiled ? lane % D : 0, lm = tiled ? lane / D : 0, mstep = tiled ? 64 / D : 1;
-    for (uint32_t bi = blockIdx.x; bi < n_big; bi += gridDim.x) {
+    for (uint32_t bi = first; bi < n_big; bi += stride) {
         const uint32_t g = big_list[bi];
         const uint32_t row = grp_row[g];
         if (row == NO_ROW) continue;
@@ -1730,7 +1731,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             delta_show = __float_as_int(sp[2 * D + 1]);
         }
         bool any = false;
-        __syncthreads();
+        sync();
         for (uint32_t c0 = 0; c0 < k; c0 += per_chunk) {
             const int cn = (int)((k - c0) < (uint32_t)per_chunk ? (k - c0) : (uint32_t)per_chunk);
             // lane m resolves record m of the chunk and keeps its counts
@@ -1744,7 +1745,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                 gok[lane] = ok ? 1 : 0;
             }
             const unsigned long long okmask = __ballot(ok);  // the usable records, known to every lane
-            __syncthreads();
+            sync();
             // gradients into the staging, BIG_LOADS loads of a lane in flight at a time
             if (tiled) {  // lane = (record within a round, element): no division per element
                 for (int m0 = lm; m0 < cn; m0 += mstep * BIG_LOADS) {
@@ -1782,7 +1783,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                     }
                 }
             }
-            __syncthreads();
+            sync();
             if (KIND == OPT_ADAGRAD) {
                 // add_g2sum / dim of record `lane`: double sum of float products in element order
                 double mq = 0.0;
@@ -1805,7 +1806,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                     if (lane == m) myg2 = g2sum;
                 }
                 if (lane < cn) den[lane] = o.eps + sqrtf(myg2);
-                __syncthreads();
+                sync();
                 // the steps lr * g / den of all records and elements by all lanes (independent divisions),
                 // then per element the subtractions in record order
                 if (tiled) {
@@ -1816,7 +1817,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                         gbuf[m * Dp + i] = o.lr * gbuf[m * Dp + i] / den[m];
                     }
                 }
-                __syncthreads();
+                sync();
                 for (int i = lane; i < D; i += 64) {
                     float w = rw[i];
                     for (int m = 0; m < cn; m++)
@@ -1844,7 +1845,7 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
             const unsigned long long chunk_mask = cn == 64 ? ~0ull : (1ull << cn) - 1ull;
             if (okmask) any = true;
             if (lane == 0 && okmask != chunk_mask) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
-            __syncthreads();
+            sync();
         }
         if (any) {
             for (int i = lane; i < D; i += 64) {
@@ -1869,8 +1870,31 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                 }
             }
         }
-        __syncthreads();
+        sync();
     }
+}
+
+// Fences a wavefront's LDS traffic: what its lanes wrote before is what they read after (the LDS unit takes a
+// wavefront's instructions in order; the fence keeps the compiler from moving them across).
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int KIND>
+__global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src, DevStatus* status,
+                                                  const uint32_t* __restrict__ big_list,
+                                                  const uint32_t* __restrict__ grp_row,
+                                                  const uint32_t* __restrict__ grp_off,
+                                                  const uint32_t* __restrict__ grp_cnt,
+                                                  const Member* __restrict__ list, int gbuf_floats,
+                                                  const float* const* __restrict__ gaddr) {
+    extern __shared__ float gbuf[];  // gbuf_floats floats of staging, then the row: rw[D], ra[D], rb[D]
+    __shared__ const float* gptr[BIG_CHUNK];
+    __shared__ int gshow[BIG_CHUNK], gok[BIG_CHUNK];
+    __shared__ float den[BIG_CHUNK];
+    apply_big_groups<KIND>(s, o, src, status, big_list, grp_row, grp_off, grp_cnt, list, gbuf_floats, gaddr, gbuf, gptr,
+                           gshow, gok, den, (int)threadIdx.x, blockIdx.x, gridDim.x, [] { __syncthreads(); });
 }
 
 // Any dim / alignment: one thread per distinct sign, scalar loops.

@@ -41,12 +41,12 @@ constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS 
 // takes the path of few launches (small_batch.h).
 constexpr size_t SMALL_MAX_LOOKUPS = 1u << 18;
 
-// A small batch of at most this many slots leaves every sign to the lane groups of k_small_apply: no launch of
-// k_apply_big.  With more slots a sign with SMALL_BIG_GROUP records or more goes to k_apply_big: a small batch's
-// kernels are as long as their longest chain, and the records of a sign applied one after the other by a lane
-// group (four elements per lane) take four times as long as by a wavefront (measured, 4096 x 26 slots, Adam:
-// the updates take 0.040 ms with every sign left to the lane groups, 0.017 + 0.015 ms with the threshold at 5,
-// 0.017 + 0.026 ms at 16; 1024 x 8 slots: 0.012 ms without k_apply_big, 0.009 + 0.009 ms with it).
+// A small batch of at most this many slots leaves every sign to the lane groups of k_small_apply.  With more slots a
+// sign with SMALL_BIG_GROUP records or more is taken by a wavefront of its own (the first workgroups of the same
+// launch): a small batch's kernels are as long as their longest chain, and the records of a sign applied one after
+// the other by a lane group (four elements per lane) take four times as long as by a wavefront with a lane per
+// element (measured, 4096 x 26 slots, Adam: the updates take 0.040 ms with every sign left to the lane groups,
+// 0.020 ms with the threshold at 5; 1024 x 8 slots: no difference between 4 and 12 slots here).
 constexpr int SMALL_NO_BIG_SLOTS = 12;
 constexpr uint32_t SMALL_BIG_GROUP = 5;
 constexpr uint32_t BIG_GROUP_DEFAULT = 16;
@@ -914,17 +914,27 @@ int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* d
     }
 }
 
-// The updates of a small push: every group by one launch of k_small_apply (which also tells the host that the
-// comparison launched before it is complete), but the signs with many records, if the plan lists any, by
-// k_apply_big after it.
+// The updates of a small push, one launch: the lane groups' workgroups for every group below the plan's threshold
+// and, if the plan lists signs with many records, workgroups whose wavefronts take those (as a kernel of its own
+// after this one, k_apply_big made 4096 x 26 slots, Adam, 0.080 ms per pull + push; beside it on the table's side
+// stream 0.113 ms: the events that fork and join the streams cost more than the overlap wins).
 template <int KIND>
 int launch_small_apply_kind(SparseTable* t, int lpg, int N, const OptDev& o, const PushSrc& src, DevStatus* ds,
                             const Plan& p, int64_t n_upper, hipStream_t st, uint32_t* host_seq, uint32_t seq) {
     const Store& s = t->store;
     const uint32_t big_k = t->plan_big_k;
+    const bool with_big = big_k != 0xFFFFFFFFu && (uint32_t)N >= big_k;
+    // (a wavefront per sign with big_k records or more, four to a workgroup, 512 workgroups at most)
+    const int big_blocks = with_big ? launch_grid((n_upper / big_k + 1 + 3) / 4, 1, 512) : 0;
+    const size_t lds = with_big ? small_apply_big_lds(s.D) : 0;
 #define TN_LAUNCH_SMALL(LPG)                                                                                          \
-    TN_LAUNCH((k_small_apply<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, o, src, \
-              N, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, (uint32_t)n_upper, host_seq, seq)
+    do {                                                                                                              \
+        const int group_blocks = launch_grid(n_upper * LPG, 256, GRID_CAP * 4);                                       \
+        TN_LAUNCH_LDS((k_small_apply<KIND, LPG>), dim3(group_blocks + big_blocks), dim3(256), lds, st, s, o, src, N, ds, \
+                      p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, (uint32_t)n_upper, host_seq, seq,              \
+                      (uint32_t)big_blocks, p.big_list, big_gbuf_floats(s.D), (uint32_t)small_apply_wave_lds(s.D),    \
+                      (uint32_t)align_up(big_lds_bytes(s.D), 8));                                                    \
+    } while (0)
     switch (lpg) {
         case 1: TN_LAUNCH_SMALL(1); break;
         case 2: TN_LAUNCH_SMALL(2); break;
@@ -934,10 +944,6 @@ int launch_small_apply_kind(SparseTable* t, int lpg, int N, const OptDev& o, con
         default: TN_LAUNCH_SMALL(32); break;
     }
 #undef TN_LAUNCH_SMALL
-    if (big_k != 0xFFFFFFFFu && (uint32_t)N >= big_k)
-        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / big_k + 1, 1, 16384)), dim3(64),
-                      big_lds_bytes(s.D), st, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list,
-                      big_gbuf_floats(s.D), (const float* const*)nullptr);
     return TN_OK;
 }
 

@@ -13,6 +13,13 @@ The runs (MI355X box, from the repository root, after `cd /tmp && export TMPDIR=
     python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_trace --fetch gpurun_out/prof_fetch \\
         --write gpurun_out/prof_write --bench gpurun_out/bench_full.json --commit <commit of the profiled tree>
 
+With --trace and --title only (no counter runs) it writes a table of kernel durations, e.g. for the small
+configurations, whose steps are a handful of short kernels (one run per configuration):
+
+    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_cfg1 -o t -- python3 bench.py --config cfg1 --steps 50 --warmup 5 \
+        --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-traffic
+    python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_cfg1 --title "cfg1 ..." --out profiles/<name>.md [--append]
+
 FETCH_SIZE / WRITE_SIZE count in KiB per dispatch in units that are not bytes on every ASIC: both are
 scaled by the factor that makes the same counter reproduce the known traffic of the dense Adam stream of
 the same run (k_dense_adam_v4 on 2e8 parameters reads 16 B and writes 16 B per parameter).
@@ -57,13 +64,28 @@ def read_counter(directory):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--trace", required=True)
-    ap.add_argument("--fetch", required=True)
-    ap.add_argument("--write", required=True)
-    ap.add_argument("--bench", required=True, help="file holding the JSON line of a full bench.py run")
+    ap.add_argument("--fetch")
+    ap.add_argument("--write")
+    ap.add_argument("--bench", help="file holding the JSON line of a full bench.py run")
+    ap.add_argument("--title", help="durations only: heading of the table")
+    ap.add_argument("--note", default="", help="durations only: a line under the heading (the command, the step time)")
+    ap.add_argument("--append", action="store_true", help="durations only: add to --out instead of replacing it")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles", "cfg3_adagrad_dim16_pull_push.md"))
     ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "cfg3_traffic.json"))
     ap.add_argument("--commit", default=None, help="commit of the profiled tree (default: git rev-parse HEAD here)")
     args = ap.parse_args()
+    if not (args.fetch and args.write and args.bench):
+        if not args.title:
+            raise SystemExit("either --fetch, --write and --bench (the cfg3 profile) or --title (durations only)")
+        trace = read_trace(args.trace)
+        out = ["## %s\n" % args.title, args.note, "",
+               "| kernel | launches | avg us | min us | max us |", "|---|---|---|---|---|"]
+        out += ["| %s | %d | %.1f | %.1f | %.1f |" % (r["name"], r["calls"], r["avg_ns"] / 1e3, r["min_ns"] / 1e3, r["max_ns"] / 1e3)
+                for r in trace]
+        with open(args.out, "a" if args.append else "w") as f:
+            f.write("\n".join(out) + "\n\n")
+        print("wrote %s (%d kernels)" % (args.out, len(trace)))
+        return
     sys.path.insert(0, ROOT)
     import bench
 
