@@ -369,6 +369,30 @@ def main():
     }
 
     # ---- side measurement: a batch that overflows the buckets sized from the recent pulls ----------
+    # A batch small enough for the path of few launches: the same steps once more on the path every other batch
+    # takes (the library has a switch for that), to be quoted beside it.
+    if any(k.startswith("k_small") for k in per_step):
+        tn.core.set_sparse_table_small_batch_path(h, False)
+        reps = [i for i in timed]
+        for i in reps[:max(1, args.warmup)]:
+            step(i)
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in reps:
+            step(i)
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        other = (time.perf_counter() - t0) * 1e3 / len(reps)
+        tn.core.set_sparse_table_small_batch_path(h, True)
+        out["small_batch_path"] = {
+            "what": "the timed steps ran on the path of few launches that small batches take; the same batches again "
+                    "on the path every other batch takes",
+            "ms_per_step": ms_per_step,
+            "other_path_ms_per_step": other,
+        }
+        log("small-batch path %.4f ms/step, the other path %.4f ms/step" % (ms_per_step, other))
+
     # The second-level buckets follow the share of distinct records of the recent pulls.  A dozen pulls of a
     # batch that repeats a thousand signs shrink them; the next ordinary batch then overflows, and its pull is
     # repeated with buckets sized for a batch of distinct signs only.

@@ -349,6 +349,11 @@ int tn_sparse_table_last_unique_counts(uint32_t handle, int N, int64_t* counts);
  * stream themselves); its errors are then latched like push_op's. */
 int tn_sparse_table_set_async(uint32_t handle, int async_pull);
 
+/* Whether small batches (every slot at most 4096 lookups, at most 128 slots and 262144 lookups) take the path
+ * of few launches (the default) or the one every other batch takes.  Same results either way; a switch for
+ * measurements and tests, without a counterpart in the reference. */
+int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable);
+
 /* ------------------------------------------------------------- dense table */
 /* CreateDenseTable (core/ps/table/dense_table.cc:180-186); Adam or AdaGrad.  With shard_num > 1
  * the table is worker self_shard_id's share: after Init it owns the contiguous range

@@ -159,6 +159,12 @@ def set_sparse_table_async(table_handle, async_pull):
     _lib.check(_lib.load().tn_sparse_table_set_async(table_handle, 1 if async_pull else 0))
 
 
+def set_sparse_table_small_batch_path(table_handle, enable):
+    """Whether small batches take the path of few launches (the default) or the one every other batch takes:
+    same results, a switch for measurements and tests."""
+    _lib.check(_lib.load().tn_sparse_table_set_small_batch_path(table_handle, 1 if enable else 0))
+
+
 def sparse_table_key_count(table_handle):
     n = C.c_uint64()
     _lib.check(_lib.load().tn_sparse_table_key_count(table_handle, C.byref(n)))

@@ -135,6 +135,7 @@ struct SparseTable {
     int pull_slots = 0, push_slots = 0;  // N of the pending calls
     std::vector<int64_t> pending_rows;  // var rows of a pending async pull
     int async_pull = 0;
+    bool small_path = true;         // small batches take the path of few launches (tn_sparse_table_set_small_batch_path)
     int latched = TN_OK;
     std::string latched_msg;
     std::vector<int64_t> last_counts;
@@ -984,7 +985,7 @@ uint32_t small_entries(size_t max_len) {
 
 // Does the batch qualify for the path of few launches?  (nb2: its second-level buckets.)
 bool small_batch_fits(SparseTable* t, int N, const int64_t* lens, size_t L, uint32_t nb2) {
-    if (t->async_pull || N > SMALL_SLOTS || L == 0 || L > SMALL_MAX_LOOKUPS || nb2 > (uint32_t)SMALL_NB2_MAX) return false;
+    if (!t->small_path || t->async_pull || N > SMALL_SLOTS || L == 0 || L > SMALL_MAX_LOOKUPS || nb2 > (uint32_t)SMALL_NB2_MAX) return false;
     size_t max_len = 0;
     for (int s = 0; s < N; s++) max_len = std::max<size_t>(max_len, (size_t)lens[s]);
     if (max_len > (size_t)SMALL_SLOT_MAX) return false;
@@ -1146,6 +1147,14 @@ int tn_sparse_table_set_async(uint32_t handle, int async_pull) {
     if (!t) return fail(TN_ERR_BAD_HANDLE, "tn_sparse_table_set_async: bad table handle");
     std::lock_guard<std::mutex> lk(t->mu);
     t->async_pull = async_pull ? 1 : 0;
+    return TN_OK;
+}
+
+int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad sparse table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->small_path = enable != 0;
     return TN_OK;
 }
 
@@ -1879,7 +1888,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         return TN_OK;
     };
     const int small_lpg = lanes_per_group(t->store, vec && t->store.wstride % 4 == 0);
-    if (reuse && t->plan_small && !pooled && small_lpg != 0 && N <= SMALL_SLOTS) {
+    if (reuse && t->plan_small && t->small_path && !pooled && small_lpg != 0 && N <= SMALL_SLOTS) {
         // A small batch on the plan of its small pull: slot descriptors, comparison of the signs and click sums by
         // one launch, the updates by one or two more (small_batch.h).  The call's status block is the plan's:
         // nothing of the next call runs beside this one.  The device has nothing to report: every sign of the plan

@@ -151,3 +151,50 @@ def test_small_and_large_batches_alternate_on_one_table(tn, oracle):
     grads = synth.make_grads(small_counts, D, 0.01, seed=9)
     pair.push_op(small, grads, [np.zeros(len(v), np.int64) for v in small])
     pair.assert_rows_match(np.unique(np.concatenate(seen)))
+
+
+@pytest.mark.parametrize("opt,hyper,dim,slots,per", [("AdaGrad", ADAGRAD_HP, 8, 8, 1024), ("Adam", ADAM_HP, 16, 26, 2000),
+                                                     ("Ftrl", FTRL_HP, 4, 40, 500)])
+def test_both_paths_leave_the_same_table(tn, oracle, opt, hyper, dim, slots, per):
+    """Two tables, the same seed and the same batches, one on the path of few launches and one with it switched off:
+    mapped ids, pulled rows (new rows included: same seed, same signs) and the rows after every push are the same
+    bit for bit -- both paths apply a sign's records in slot order with the same arithmetic."""
+    rng = np.random.default_rng(99)
+    pool = synth.splitmix64(np.arange(1, 40001, dtype=np.uint64)).view(np.int64)
+    tables = []
+    for small in (True, False):
+        gopt = getattr(tn.core, opt)(**hyper)
+        h = tn.core.create_sparse_table(gopt, "", dim, False, "")
+        tn.core.reserve_sparse_table(h, 300000)
+        tn.core.set_sparse_table_seed(h, 1234)
+        tn.core.set_sparse_table_small_batch_path(h, small)
+        tables.append(h)
+    wf, sf = tn.core.sparse_table_row_layout(tables[0])
+    seen = []
+    for step in range(3):
+        values = batch(rng, slots, per, pool, hot=3, fresh=0.1)
+        gvalues = [dev(v) for v in values]
+        labels = [dev((rng.random(len(v)) < 0.3).astype(np.int64)) for v in values]
+        outs = []
+        for h in tables:
+            gvars = [torch.full((per + 1, wf), -7.0, device="cuda") for _ in values]
+            launched = kernels_of(tn, lambda: outs.append((tn.ops.sparse_table_pull(gvars, gvalues, h), gvars)))
+            assert any(k.startswith("k_small") for k in launched) == (h == tables[0])
+        counts = tn.ops.sparse_table_last_unique_counts(tables[0], slots)
+        assert counts == tn.ops.sparse_table_last_unique_counts(tables[1], slots)
+        for a, b in zip(outs[0][0], outs[1][0]):
+            assert torch.equal(a, b)
+        for a, b in zip(outs[0][1], outs[1][1]):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+        grads = [dev(g) for g in synth.make_grads(counts, wf, 0.01, seed=step)]
+        for h in tables:
+            tn.ops.sparse_table_push(gvalues, grads, labels, h)
+            tn.ops.sparse_table_sync(h)
+        seen.append(all_signs(values))
+        signs = dev(np.unique(np.concatenate(seen)).view(np.int64))
+        w0, s0, f0 = tn.ops.table_export_rows(tables[0], signs)
+        w1, s1, f1 = tn.ops.table_export_rows(tables[1], signs)
+        assert bool(f0.all()) and bool(f1.all())
+        assert torch.equal(w0.view(torch.int32), w1.view(torch.int32))
+        assert torch.equal(s0.view(torch.int32), s1.view(torch.int32))
+    assert tn.core.sparse_table_key_count(tables[0]) == tn.core.sparse_table_key_count(tables[1])
