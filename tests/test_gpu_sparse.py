@@ -870,9 +870,11 @@ def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
     pair.populate(pool.view(np.uint64))
     s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
     torch.cuda.synchronize()
-    for step in range(2):
-        # step 0: a batch large enough for the side streams (more than 3 M lookups), step 1: a small one
-        per_slot = (200000, 230000) if step == 0 else (3000, 6000)
+    for step in range(3):
+        # step 0: a batch large enough for the side streams (more than 3 M lookups), step 1: a small one, step 2:
+        # one for the path of few launches (every slot within 4096 lookups), whose pull also returns before its
+        # last kernels have run
+        per_slot = ((200000, 230000), (3000, 6000), (500, 3000))[step]
         values = [pool[rng.integers(0, 600000, int(rng.integers(*per_slot)))] for _ in range(16)]
         assert (sum(len(v) for v in values) > 3 << 20) == (step == 0)
         rows = [len(v) + 1 for v in values]
