@@ -171,15 +171,23 @@ __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ h
 }
 
 // host_dst: a DevStatus followed by n_ubase words.  With count != nullptr the rows the call
-// inserted are added to the table's number of resident keys.
+// inserted are added to the table's number of resident keys.  With host_seq != nullptr the word seq is written
+// there once everything else is on the host: a host that polls that word has the status a few microseconds
+// after this kernel, well before a wait on the stream would return.
 __global__ __launch_bounds__(256) void k_publish(const DevStatus* __restrict__ status,
                                                  const uint32_t* __restrict__ ubase, uint32_t n_ubase,
-                                                 uint32_t* __restrict__ host_dst, unsigned long long* count) {
+                                                 uint32_t* __restrict__ host_dst, unsigned long long* count,
+                                                 uint32_t* host_seq, uint32_t seq) {
     if (count && threadIdx.x == 0) *count += status->n_new;
     const uint32_t sw = sizeof(DevStatus) / 4;
     const uint32_t* sp = reinterpret_cast<const uint32_t*>(status);
     for (uint32_t i = threadIdx.x; i < sw + n_ubase; i += blockDim.x)
         host_dst[i] = i < sw ? sp[i] : ubase[i - sw];
+    if (host_seq) {
+        __threadfence_system();
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_store(host_seq, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 __global__ void k_finish_insert(Store s, const DevStatus* status) {

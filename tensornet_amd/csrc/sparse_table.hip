@@ -1684,9 +1684,17 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         // call's status (counts, new rows, errors) is final before the gather starts: it is published
         // on the side stream beside the gather, and the call returns when the host has it.  The
         // variables are complete in stream order, as the outputs of any call that takes a stream.
-        const bool early = use_lds && N <= GRP_SLOTS && !t->async_pull && !t->one_stream;
+        const bool final_early = use_lds && N <= GRP_SLOTS && !t->async_pull;
+        const bool early = final_early && !t->one_stream;
+        // A call that keeps to the caller's stream publishes there, ahead of the gather, and tells the host through
+        // a word in pinned memory: the host prepares the push while the gather runs.
+        const bool early_inline = final_early && t->one_stream;
+        const uint32_t seq = early_inline ? ++t->seq_pull : 0;
         const uint32_t* rows_of_groups = (use_lds && N <= GRP_SLOTS) ? nullptr : p.grp_row;
         if (early) TN_HIP(hipEventRecord(t->ready_ev, st));
+        if (early_inline)
+            TN_LAUNCH(k_publish, dim3(1), dim3(256), st, ds, p.ubase, (uint32_t)(N + 1),
+                      reinterpret_cast<uint32_t*>(t->hpull), s.count, t->hseq + 0, seq);
         if (vec)
             TN_LAUNCH((k_gather_vars<4>), dim3(launch_grid((int64_t)L * (wdim / 4), 256, GRID_CAP * 4)), dim3(256), st, s,
                       ds, rows_of_groups, p.where_u, p.ubase, N, p.descs);
@@ -1694,13 +1702,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             TN_LAUNCH((k_gather_vars<1>), dim3(launch_grid((int64_t)L * wdim, 256, GRID_CAP * 4)), dim3(256), st, s, ds,
                       rows_of_groups, p.where_u, p.ubase, N, p.descs);
         TN_HIP(hipGetLastError());
-        if (early) {
+        if (early || early_inline) {
             TN_HIP(hipEventRecord(t->tail_ev, st));
             t->tail_recorded = true;
-            TN_HIP(hipStreamWaitEvent(t->side, t->ready_ev, 0));
         }
-        TN_LAUNCH(k_publish, dim3(1), dim3(256), early ? t->side : st, ds, p.ubase, (uint32_t)(N + 1),
-                  reinterpret_cast<uint32_t*>(t->hpull), s.count);
+        if (early) TN_HIP(hipStreamWaitEvent(t->side, t->ready_ev, 0));
+        if (!early_inline)
+            TN_LAUNCH(k_publish, dim3(1), dim3(256), early ? t->side : st, ds, p.ubase, (uint32_t)(N + 1),
+                      reinterpret_cast<uint32_t*>(t->hpull), s.count, (uint32_t*)nullptr, 0u);
         if (early) TN_HIP(hipEventRecord(t->pub_ev, t->side));
         t->pull_pending = true;
         t->pull_slots = N;
@@ -1716,6 +1725,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         if (t->async_pull) return TN_OK;
         if (early)
             TN_HIP(hipEventSynchronize(t->pub_ev));
+        else if (early_inline)
+            TN_TRY(wait_reported(t->hseq + 0, seq, st, "SparseTablePull"));
         else
             TN_HIP(hipStreamSynchronize(st));
         if (use_lds && (t->hpull->st.err & DEV_ERR_REMAP_OVERFLOW)) {
@@ -1738,6 +1749,10 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             harvest(t);
             t->flow = FLOW_PULL;
             t->flow_stream = st;
+            return take_latched(t);
+        }
+        if (early_inline) {
+            harvest(t);
             return take_latched(t);
         }
         return sync_table(t, st);
@@ -2003,7 +2018,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         TN_HIP(hipStreamWaitEvent(t->side, t->apply_ev, 0));
     }
     TN_LAUNCH(k_publish, dim3(1), dim3(256), pub_on_side ? t->side : st, ds, pub_ubase ? pub_ubase : p.ubase,
-              (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr);
+              (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr, (uint32_t*)nullptr, 0u);
     t->push_pending = true;
     t->push_pub_on_side = pub_on_side;
     t->push_slots = N;
