@@ -33,7 +33,8 @@ constexpr int SMALL_PARTS_MAX = 8;                           // workgroups of k_
 constexpr int SMALL_SLOT_WORKGROUPS = 256;                   // ... and for all slots together
 constexpr int SMALL_TILE = 1024;                             // lookups per workgroup of k_small_verify
 
-// What a slot's workgroup leaves for the one that finishes last.
+// What a workgroup of k_small_slots leaves for the launch after it: the slot's distinct signs (the same in
+// every workgroup of the slot), the rows it inserted and the error flags it raised.
 struct SlotOut {
     uint32_t n_unique, n_new, err, pad;
 };
@@ -54,6 +55,11 @@ __device__ __forceinline__ void host_store(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// First launch of a small pull (see the head of the file).  host_descs: the slot descriptors in the host's pinned
+// staging buffer; descs, lbase: where they go in device memory, for the launches after this one.  entries: the
+// size of the workgroup's LDS table, a power of two and at least twice the longest slot.  prow[first lookup of
+// the slot + r]: table row of the slot's distinct sign of rank r.  cursor2 / recs / rrow: the second-level
+// buckets, as k_lds_dedup<true> and k_probe_recs fill them, but a record carries its rank in its slot (gi).
 __global__ __launch_bounds__(SMALL_THREADS) void k_small_slots(
     const SlotDesc* host_descs, SlotDesc* descs, uint32_t* lbase, int N, uint32_t L, uint32_t entries,
     Store s, OptDev o, uint64_t seed, uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ u_of_gi,
