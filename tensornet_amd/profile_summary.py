@@ -20,6 +20,16 @@ configurations, whose steps are a handful of short kernels (one run per configur
         --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-traffic
     python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_cfg1 --title "cfg1 ..." --out profiles/<name>.md [--append]
 
+With --counters (one or more directories of `rocprofv3 --pmc <SQ counters>` runs of the same command, at most 8 SQ
+counters a run) and --title it writes the per-dispatch averages of those counters for the step's kernels and a few
+ratios of them (what share of its wavefronts' time a kernel waits, and on what):
+
+    rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_WAIT_ANY SQ_WAIT_INST_ANY SQ_WAIT_INST_LDS SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT \
+        -d gpurun_out/pmc_a -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback
+    rocprofv3 --pmc SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_LDS SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_ACTIVE_INST_VMEM SQ_ACTIVE_INST_VALU SQ_INST_LEVEL_VMEM \
+        -d gpurun_out/pmc_b -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback
+    python3 -m tensornet_amd.profile_summary --counters gpurun_out/pmc_a gpurun_out/pmc_b --title "..." --out profiles/<name>.md
+
 FETCH_SIZE / WRITE_SIZE count in KiB per dispatch in units that are not bytes on every ASIC: both are
 scaled by the factor that makes the same counter reproduce the known traffic of the dense Adam stream of
 the same run (k_dense_adam_v4 on 2e8 parameters reads 16 B and writes 16 B per parameter).
@@ -63,7 +73,8 @@ def read_counter(directory):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--trace", required=True)
+    ap.add_argument("--trace")
+    ap.add_argument("--counters", nargs="+", help="directories of --pmc runs: a table of their counters per kernel")
     ap.add_argument("--fetch")
     ap.add_argument("--write")
     ap.add_argument("--bench", help="file holding the JSON line of a full bench.py run")
@@ -74,6 +85,46 @@ def main():
     ap.add_argument("--traffic", default=os.path.join(ROOT, "profiles", "cfg3_traffic.json"))
     ap.add_argument("--commit", default=None, help="commit of the profiled tree (default: git rev-parse HEAD here)")
     args = ap.parse_args()
+    if args.counters:
+        if not args.title:
+            raise SystemExit("--counters needs --title")
+        table, names = {}, []
+        for d in args.counters:
+            cur = _db(d)
+            for k, c, n, v in cur.execute("select kernel_name, counter_name, count(*), avg(value) from counters_collection "
+                                          "where kernel_name like '%tn::%' group by kernel_name, counter_name"):
+                table.setdefault(short(k), {})[c] = v
+                table[short(k)]["_n"] = n
+                if c not in names:
+                    names.append(c)
+        skip = ("k_load_rows", "k_probe<true>", "k_finish_insert", "k_reset_status")
+        rows = sorted(((k, v) for k, v in table.items() if not k.startswith(skip)),
+                      key=lambda kv: -kv[1].get("SQ_BUSY_CYCLES", 0))
+        out = ["# %s\n" % args.title, args.note, "",
+               "Per-dispatch averages (summed over the device's shader engines / XCDs as rocprofv3 reports them).\n",
+               "| kernel | " + " | ".join(n.replace("SQ_", "") for n in names) + " |", "|---|" + "---|" * len(names)]
+        for k, v in rows:
+            out.append("| %s | " % k + " | ".join("%.3g" % v.get(n, 0) for n in names) + " |")
+
+        def ratio(v, a, b):
+            return "%.2f" % (v[a] / v[b]) if v.get(a) is not None and v.get(b) else "-"
+
+        out += ["", "Ratios: share of its wavefronts' cycles a kernel waits for anything / for an instruction to come back / "
+                    "for LDS; LDS bank-conflict cycles per cycle the LDS is busy with the kernel's instructions; vector "
+                    "memory instructions in flight per wavefront cycle (of 1).\n",
+                "| kernel | WAIT_ANY / WAVE_CYCLES | WAIT_INST_ANY / WAVE_CYCLES | WAIT_INST_LDS / WAVE_CYCLES | "
+                "LDS_BANK_CONFLICT / ACTIVE_INST_LDS | INST_LEVEL_VMEM / WAVE_CYCLES |", "|---|---|---|---|---|---|"]
+        for k, v in rows:
+            out.append("| %s | %s | %s | %s | %s | %s |" % (
+                k, ratio(v, "SQ_WAIT_ANY", "SQ_WAVE_CYCLES"), ratio(v, "SQ_WAIT_INST_ANY", "SQ_WAVE_CYCLES"),
+                ratio(v, "SQ_WAIT_INST_LDS", "SQ_WAVE_CYCLES"), ratio(v, "SQ_LDS_BANK_CONFLICT", "SQ_ACTIVE_INST_LDS"),
+                ratio(v, "SQ_INST_LEVEL_VMEM", "SQ_WAVE_CYCLES")))
+        with open(args.out, "w") as f:
+            f.write("\n".join(out) + "\n")
+        print("wrote %s (%d kernels, %d counters)" % (args.out, len(rows), len(names)))
+        return
+    if not args.trace:
+        raise SystemExit("--trace is needed (or --counters)")
     if not (args.fetch and args.write and args.bench):
         if not args.title:
             raise SystemExit("either --fetch, --write and --bench (the cfg3 profile) or --title (durations only)")
