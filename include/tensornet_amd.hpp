@@ -169,6 +169,8 @@ public:
     // HBM sizing (no counterpart in the reference, whose host maps grow by themselves).
     int Reserve(uint64_t max_keys) { return tn_sparse_table_reserve(handle_, max_keys); }
     int Clear() { return tn_sparse_table_clear(handle_); }
+    // small batches on the path of few launches (the default) or on the one every other batch takes: same results
+    int SetSmallBatchPath(bool enable) { return tn_sparse_table_set_small_batch_path(handle_, enable ? 1 : 0); }
     int Sync() { return tn_sparse_table_sync(handle_); }
 
 private:
