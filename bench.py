@@ -84,7 +84,7 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
 
     table = {
         # remap through LDS
-        "k_lds_hist": 16 * L,                  # reads every sign, keeps a copy for the push
+        "k_lds_hist": 8 * L + L // 32,         # reads every sign, leaves 16 bytes of fingerprint per 64 of them
         "k_lds_scatter": 20 * L,               # reads every sign, writes {sign, position} by bucket
         "k_lds_dedup": 16 * L + 16 * U,        # reads {sign, position}, writes first positions and the distinct records
         "k_lds_flags": 4 * L,
@@ -102,7 +102,8 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
         "k_probe_recs": 8 * U + 8 * U + 4 * U, # the record's sign in, one stored-key compare, row number out
         "k_gather_vars": U * (2 * row + 4),    # row read + variable row write
         # push
-        "k_verify_values": 24 * L,             # the op's signs against the pull's copy, labels
+        # the op's signs and labels, against the pull's copy of the signs (COPY) or its fingerprints of them
+        "k_verify_values": (24 * L if name.endswith(", true>") else 16 * L + L // 32),
         "k_reset_counts": 8 * U,
         "k_apply_single": apply_bytes(shape["G1"], shape["G1"]),
         "k_apply_vec": apply_bytes(shape["Rm"], shape["Gm"]),

@@ -135,10 +135,13 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
 
 // Also presets first_of to "every lookup is its own first occurrence", which is
 // what a lookup keeps if an overflow leaves it unprocessed (its count is then
-// meaningless, but every index stays in bounds until the host repeats the call).
+// meaningless, but every index stays in bounds until the host repeats the call),
+// and leaves the fingerprints of the batch's signs, which a push compares its own with
+// (k_verify_values): one per wavefront of a tile, the same tiles in both kernels.
+static_assert(LDS_TILE == VERIFY_TILE, "k_lds_hist and k_verify_values fingerprint the same runs of lookups");
 __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
                                                   int N, uint32_t L, uint32_t* bcount,
-                                                  uint64_t* __restrict__ vals_copy, uint32_t* __restrict__ first_of,
+                                                  ulonglong2* __restrict__ prints, uint32_t* __restrict__ first_of,
                                                   DevStatus* status, uint32_t span_cap) {
     extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]
     uint32_t* lb = smem;
@@ -150,8 +153,9 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
         const uint32_t span = tile_span(tile, descs, lb, N, L, span_cap, b0);
         for (uint32_t i = threadIdx.x; i < span; i += 256) hist[i] = 0;
         __syncthreads();
+        Fingerprint print;
         for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
-            vals_copy[gi] = sign;
+            print.add(gi, sign);
             first_of[gi] = gi;
             const uint32_t local = bucket_of(d, sign) - b0;
             if (local < span)
@@ -159,6 +163,8 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
             else
                 flag_overflow(status);
         });
+        print.wave_sum();
+        if ((threadIdx.x & 63) == 0) prints[tile * (256 / 64) + (threadIdx.x >> 6)] = make_ulonglong2(print.a, print.b);
         __syncthreads();
         for (uint32_t i = threadIdx.x; i < span; i += 256)
             if (hist[i]) atomicAdd(&bcount[b0 + i], hist[i]);
@@ -242,7 +248,10 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
     __shared__ uint32_t cnts[LDS_TABLE + 1];
     __shared__ uint32_t hist2[EMIT ? LDS_SPAN2 : 1];
     __shared__ uint32_t c_lo_sh, slot_sh;
-    for (uint32_t b = blockIdx.x; b < nbuckets; b += gridDim.x) {
+    // The buckets of a slot scatter four-byte words over the same stretch of first_of and cnt_at (the slot's
+    // positions): on one die they meet in one L2 and leave it as whole lines.
+    const DieShare share(nbuckets);
+    for (uint32_t b = share.first; b < share.end; b += share.step) {
         const uint32_t lo = bstart[b], hi = bstart[b + 1];
         if (lo == hi) continue;
         // The bucket's lookups are taken DEDUP_ITEMS per thread at a time, all loads of a round

@@ -1271,13 +1271,38 @@ __global__ __launch_bounds__(256) void k_member_grads(PushSrc src, const DevStat
 // sign that takes a few percent of a slot's lookups receives thousands of adds): a workgroup
 // first sums the labels of its tile per distinct record in an LDS table and then adds every
 // entry to memory once.  A label that finds the table crowded goes to memory directly.
+//
+// What the signs are compared with: COPY, the plan's copy of them (the pulls that leave one: the small
+// batches' and the one through the global table); else the fingerprints that k_lds_hist left, one per 64 strided
+// lookups of a tile (the lookups of one wavefront, here as there): 16 bytes to read instead of 512.  A
+// fingerprint is two 64-bit sums over the run, of mix64(sign) and of its halves exchanged, each term times an
+// odd weight drawn from the position.  One changed sign always alters the sums (the hash is a bijection, the
+// weight odd); signs that changed places, or several changed signs, escape only if both sums come out equal by
+// chance, which for hashes that behave as random numbers has odds below 2^-66.  (The reference has no such
+// check: every push analyses its batch from scratch, sparse_table_ops.cc:274-297.)
+struct Fingerprint {
+    uint64_t a = 0, b = 0;
+    __device__ __forceinline__ void add(uint32_t gi, uint64_t sign) {
+        const uint64_t m = mix64(sign);
+        const uint32_t w = (gi * 0x9E3779B1u) | 1u;
+        a += m * w;
+        b += ((m << 32) | (m >> 32)) * w;
+    }
+    __device__ __forceinline__ void wave_sum() {
+#pragma unroll
+        for (int o = 32; o; o >>= 1) {
+            a += __shfl_xor((unsigned long long)a, o);
+            b += __shfl_xor((unsigned long long)b, o);
+        }
+    }
+};
 constexpr int VERIFY_ITEMS = 8;
 constexpr int VERIFY_TILE = 256 * VERIFY_ITEMS;  // lookups per tile
 constexpr int CLICK_BITS = 11;
 constexpr int CLICK_TABLE = 1 << CLICK_BITS;     // entries of the tile's click table
 constexpr int CLICK_TRIES = 16;
 
-template <bool CLICKS>
+template <bool CLICKS, bool COPY>
 __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ lbase, int N, uint32_t L,
                                                        const uint64_t* __restrict__ vals_copy, DevStatus* status,
@@ -1317,7 +1342,7 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                 const int sl = one_slot ? s0 : find_slot(lb, N, gi);
                 const SlotDesc& d = descs[sl];
                 now[j] = (uint64_t)d.values[gi - lb[sl]];
-                then[j] = vals_copy[gi];
+                if (COPY) then[j] = vals_copy[gi];
                 if (CLICKS) {
                     label[j] = (int)d.labels[gi - lb[sl]];
                     u[j] = u_of_gi[gi] & ~FIRST_BIT;
@@ -1330,9 +1355,20 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                 }
             }
         }
+        if (!COPY) {
+            Fingerprint print;
+#pragma unroll
+            for (int j = 0; j < VERIFY_ITEMS; j++) {
+                const uint32_t gi = g0 + j * 256 + threadIdx.x;
+                if (gi <= g1) print.add(gi, now[j]);
+            }
+            print.wave_sum();
+            const ulonglong2 left = reinterpret_cast<const ulonglong2*>(vals_copy)[tile * (256 / 64) + (threadIdx.x >> 6)];
+            bad |= print.a != left.x || print.b != left.y;
+        }
 #pragma unroll
         for (int j = 0; j < VERIFY_ITEMS; j++) {
-            bad |= now[j] != then[j];
+            if (COPY) bad |= now[j] != then[j];
             if (CLICKS && label[j] != 0) {
                 uint32_t h = (u[j] * 2654435761u) >> (32 - CLICK_BITS);
                 bool placed = false;

@@ -102,6 +102,7 @@ struct SparseTable {
     uint32_t small_calls = 0;  // (its parity: which set of bucket cursors the next small pull uses)
     size_t small_lds = 0;
     bool plan_small = false;   // the plan was left by a small pull: a push may take the small path, too
+    bool plan_prints = false;  // the plan holds fingerprints of the batch's signs, not a copy of them
     uint32_t plan_big_k = BIG_GROUP_DEFAULT;  // records from which the plan lists a sign as one for k_apply_big
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
@@ -464,7 +465,7 @@ struct Plan {
     uint32_t* push_ubase;  // ... and its copy of ubase, which its status is published from (the next pull rewrites ubase)
     uint32_t* lbase;
     uint32_t* ubase;
-    uint64_t* vals_copy;   // signs of every lookup, concatenated
+    uint64_t* vals_copy;   // signs of every lookup, concatenated; after a pull through LDS their fingerprints instead
     uint32_t* u_of_gi;     // lookup -> index of its distinct sign
     uint64_t* uniq_sign;   // per-slot distinct signs, slot-major, first-occurrence order
     uint32_t* uniq_slot;
@@ -546,7 +547,7 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     p.lbase = c.take<uint32_t>(N + 1);
     p.ubase = c.take<uint32_t>(N + 1);
     p.push_ubase = c.take<uint32_t>(N + 1);
-    p.vals_copy = c.take<uint64_t>(L);
+    p.vals_copy = c.take<uint64_t>(std::max<size_t>(L, 16));  // (the fingerprints of a short batch: 64 bytes a tile)
     p.u_of_gi = c.take<uint32_t>(L);
     p.uniq_sign = c.take<uint64_t>(L);
     p.uniq_slot = c.take<uint32_t>(L);
@@ -753,8 +754,8 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     if (use_lds) {
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
         const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
-        TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount, p.vals_copy,
-                      w.first_of, ds, w.span_cap);
+        TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount,
+                      reinterpret_cast<ulonglong2*>(p.vals_copy), w.first_of, ds, w.span_cap);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
         TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.prec,
                       w.span_cap);
@@ -1646,6 +1647,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             t->plan_small = true;
             t->plan_clicks_dirty = false;
             t->plan_has_show = true;
+            t->plan_prints = false;
             t->plan_N = N;
             t->plan_lens.assign(value_lens, value_lens + N);
             t->plan_epoch = t->epoch;
@@ -1719,6 +1721,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         t->plan_valid = true;
         t->plan_clicks_dirty = false;  // a new plan's click sums start at zero
         t->plan_has_show = use_lds;
+        t->plan_prints = use_lds;
         t->plan_N = N;
         t->plan_lens.assign(value_lens, value_lens + N);
         t->plan_epoch = t->epoch;
@@ -1972,16 +1975,25 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         const PushSrc vsrc = op_source(p, grad_dim, pd);
         const bool addr_in_verify = !pooled && t->plan_big_k != 0xFFFFFFFFu;
         const float** vgaddr = addr_in_verify ? p.gaddr : nullptr;
+        // (a macro: the profiler names a kernel by the text of its launch)
+#define TN_VERIFY(CLICKS, COPY)                                                                                      \
+    TN_LAUNCH_LDS((k_verify_values<CLICKS, COPY>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L, \
+                  p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr)
+        const bool copy = !t->plan_prints;
         if (clicks) {
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);
             t->plan_clicks_dirty = true;
-            TN_LAUNCH_LDS((k_verify_values<true>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L,
-                          p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
+            if (copy)
+                TN_VERIFY(true, true);
+            else
+                TN_VERIFY(true, false);
+        } else if (copy) {
+            TN_VERIFY(false, true);
         } else {
-            TN_LAUNCH_LDS((k_verify_values<false>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L,
-                          p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr);
+            TN_VERIFY(false, false);
         }
+#undef TN_VERIFY
         TN_HIP(hipEventRecord(t->verify_ev, st));
         // Counts and apply kernels are queued before the host knows the outcome: the counts only
         // touch the plan's member lists, which a mismatch discards anyway, and the apply kernels

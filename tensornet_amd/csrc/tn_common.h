@@ -92,6 +92,22 @@ struct DevStatus {
     uint32_t pad[2];
 };
 
+// The chip is eight dies, each with an L2 of its own, and the workgroups of a launch go to the dies in turn
+// (workgroup i to die i % 8).  A kernel whose neighbouring work items touch the same memory gives every die a
+// contiguous share of the items, taken up by the die's workgroups in launch order: neighbours then meet in one L2
+// instead of eight.  `for (i = share.first; i < share.end; i += share.step)` in place of a grid-stride loop over
+// n items; any grid covers every item once.
+constexpr uint32_t XCDS = 8;
+struct DieShare {
+    uint32_t first, end, step;
+    __device__ __forceinline__ explicit DieShare(uint32_t n) {
+        const uint32_t dies = min(XCDS, (uint32_t)gridDim.x), die = blockIdx.x % dies, per_die = (n + dies - 1) / dies;
+        first = min(n, die * per_die) + blockIdx.x / dies;
+        end = min(n, (die + 1) * per_die);
+        step = (gridDim.x - die + dies - 1) / dies;  // workgroups of the launch on this die
+    }
+};
+
 __device__ __forceinline__ uint64_t mix64(uint64_t x) {
     x ^= x >> 33;
     x *= 0xff51afd7ed558ccdull;

@@ -521,6 +521,77 @@ def test_bound_ops_over_several_steps_without_waiting(tn, oracle):
     pair.assert_rows_match(base)
 
 
+@pytest.mark.parametrize("change", ["one sign", "neighbours change places", "change places across tiles",
+                                    "last lookup", "two signs to one"])
+def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, change):
+    """After a pull through LDS the plan keeps fingerprints of the batch's signs, 16 bytes per 64 lookups, not the
+    signs: a push whose value tensors were edited in place since the pull, in one place or with two signs
+    changing places, must analyse its batch itself (the oracle is given the edited batch); the unedited batch is
+    pushed on the pull's plan."""
+    from tensornet_amd import _lib
+
+    D = 8
+    rng = np.random.default_rng(55)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=200000)
+    vocab = 20000
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    values = random_batch(rng, 3, 9000, vocab, ragged=False)  # 4.4 tiles of 2048 lookups a slot
+    gvalues = [dev(v) for v in values]
+    gvars = [torch.zeros((len(v) + 1, D), device="cuda") for v in values]
+    labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+    glabels = [dev(l) for l in labels]
+
+    def launched(fn):
+        lib = _lib.load()
+        lib.tn_profile_reset()
+        lib.tn_profile_enable(1)
+        try:
+            fn()
+            torch.cuda.synchronize()
+        finally:
+            lib.tn_profile_enable(0)
+        names = set(_lib.profile_summary())
+        lib.tn_profile_reset()
+        return names
+
+    def step(edited, seed):
+        tn.ops.sparse_table_pull(gvars, gvalues, pair.h)
+        pair.o.pull_op(values, [np.zeros((len(v) + 1, D), np.float32) for v in values])
+        for s, v in enumerate(edited):
+            gvalues[s].copy_(dev(v))
+        counts = [len(np.unique(v)) for v in edited]
+        grads = synth.make_grads(counts, D, 0.01, seed=seed)
+        assert pair.o.push_op(edited, grads, labels)[0] == 0
+        names = launched(lambda: tn.ops.sparse_table_push(gvalues, [dev(g) for g in grads], glabels, pair.h))
+        tn.ops.sparse_table_sync(pair.h)
+        pair.assert_rows_match(base)
+        for s, v in enumerate(values):
+            gvalues[s].copy_(dev(v))
+        return names
+
+    names = step(values, 0)
+    assert "k_verify_values<true, false>" in names and "k_remap_insert" not in names  # fingerprints, plan reused
+    edited = [v.copy() for v in values]
+    v = edited[1]
+    if change == "one sign":
+        v[4321] = next(int(x) for x in base.view(np.int64)[:2] if x != v[4321])  # another resident sign
+    elif change == "neighbours change places":
+        i = int(np.flatnonzero(v[:-1] != v[1:])[0])
+        v[i], v[i + 1] = v[i + 1], v[i]
+    elif change == "change places across tiles":
+        j = int(np.flatnonzero(v[5000:] != v[10])[0]) + 5000
+        v[10], v[j] = v[j], v[10]
+    elif change == "last lookup":
+        edited[2][-1] = edited[2][0] if edited[2][-1] != edited[2][0] else edited[2][1]
+    else:
+        a, b = int(v[100]), int(v[np.flatnonzero(v != v[100])[0]])
+        v[v == b] = a
+    assert any((e != o).any() for e, o in zip(edited, values))
+    names = step(edited, 1)
+    assert "k_remap_insert" in names  # the push worked the batch out itself
+    assert "k_verify_values<true, false>" in step(values, 2)
+
+
 @pytest.mark.parametrize("D", [8, 12, 64, 128])
 @pytest.mark.parametrize("opt,hyper", [("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP)])
 def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper, D):
