@@ -12,7 +12,7 @@
 // belongs to one slot, and the positions it writes to lie inside that slot's
 // window of the concatenated lookup order, so the scatter back stays local.
 //
-//   k_lds_hist     bucket sizes (+ copy of the signs for the plan)
+//   k_lds_hist     bucket sizes (+ fingerprints of the signs for the plan)
 //   k_lds_offsets  exclusive scan of the bucket sizes (one workgroup)
 //   k_lds_scatter  {sign, position, slot} records grouped by bucket
 //   k_lds_dedup    per bucket: LDS hash table -> first_of[position], occurrence counts
