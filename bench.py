@@ -193,6 +193,9 @@ def main():
                     help="leave roofline.traffic out (development runs on kernels newer than the committed profile)")
     ap.add_argument("--no-fallback", action="store_true", help="skip the side measurement of a pull whose buckets overflow")
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
+    ap.add_argument("--detached-updates", action="store_true",
+                    help="the timed steps with the push's update kernels detached (tn_sparse_table_set_detached_updates)")
+    ap.add_argument("--no-detached", action="store_true", help="skip the side measurement of detached updates")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -219,6 +222,8 @@ def main():
     opt = getattr(tn.core, opt_name)(**cfg["hyper"])
     h = tn.core.create_sparse_table(opt, "bench", dim, False, "")
     tn.core.reserve_sparse_table(h, int(resident * 1.02) + 16 * 1024 * 1024)
+    if args.detached_updates:
+        tn.core.set_sparse_table_detached_updates(h, True)
     populate(tn, h, resident, dim)
 
     # ---- inputs, resident in HBM -------------------------------------------------
@@ -345,6 +350,7 @@ def main():
             "globally_distinct_keys_of_a_batch": G0,
             "distinct_batches": nb,
             "new_keys_per_step": new_keys / args.steps,
+            "push_updates": "detached" if args.detached_updates else "in the order of the caller's stream",
         },
         "rows_per_s": total_U / wall,
         "step_algorithmic_GBps": alg / wall / 1e9,
@@ -393,6 +399,46 @@ def main():
             "other_path_ms_per_step": other,
         }
         log("small-batch path %.4f ms/step, the other path %.4f ms/step" % (ms_per_step, other))
+
+    # ---- side measurement: the same step with the push's update kernels detached from the caller's stream ------
+    # (tn_sparse_table_set_detached_updates: they then run beside the analysis of the next pull's batch; the
+    # gradient tensors must outlive the call, which is why the timed steps above do not use it.)  Batches of
+    # their own again, so that the steps insert their share of new signs.
+    if mean_L >= (3 << 20) and not args.no_detached and not args.detached_updates:
+        dsteps, dwarm = 10, 2
+        more = []
+        for b in range(nb + 2, nb + 2 + dwarm + dsteps):
+            hb = synth.make_batch(cfg, b)
+            values = [torch.from_numpy(v).cuda() for v in hb]
+            labels = [torch.from_numpy(l).cuda() for l in synth.make_labels(hb, b)]
+            grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
+            vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
+            more.append((tn.ops.BoundSparseTablePull(vars_, values, h),
+                         tn.ops.BoundSparseTablePush(values, grads, labels, h), sum(v.numel() for v in values)))
+        tn.core.set_sparse_table_detached_updates(h, True)
+        for pull, push, _ in more[:dwarm]:
+            pull()
+            push()
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for pull, push, _ in more[dwarm:]:
+            pull()
+            push()
+        tn.ops.sparse_table_sync(h)
+        torch.cuda.synchronize()
+        dwall = time.perf_counter() - t0
+        tn.core.set_sparse_table_detached_updates(h, False)
+        out["detached_updates"] = {
+            "what": "the same step with tn_sparse_table_set_detached_updates: the push's update kernels run on the "
+                    "table's own streams beside the analysis of the next pull's batch (the gradients must then stay "
+                    "untouched until the table's next waiting call returns)",
+            "steps": dsteps,
+            "ms_per_step": dwall * 1e3 / dsteps,
+            "keys_per_s": sum(n for _, _, n in more[dwarm:]) / dwall,
+        }
+        log("detached updates: %.4f ms/step" % (dwall * 1e3 / dsteps))
+        del more
 
     # The second-level buckets follow the share of distinct records of the recent pulls.  A dozen pulls of a
     # batch that repeats a thousand signs shrink them; the next ordinary batch then overflows, and its pull is

@@ -354,6 +354,17 @@ int tn_sparse_table_set_async(uint32_t handle, int async_pull);
  * measurements and tests, without a counterpart in the reference. */
 int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable);
 
+/* The reference's push op hands its gradients to the servers and returns; the rows are updated while the
+ * worker goes on (SparseTablePushKernel::ComputeAsync, sparse_table_ops.cc:346-365: requests started, done()
+ * called).  With detached updates a large push_op (3 M lookups or more, on the plan of the pull before it) does
+ * the same on the device: its update kernels run on the table's own streams and `stream` does not wait for
+ * them, so that what the caller queues next runs beside them -- above all the analysis of the next pull's
+ * batch, which orders itself behind the updates only where it first touches what they read or write (the
+ * next pull's variables hold the updated rows, as ever).  The price is the one an asynchronous op pays: the
+ * gradient matrices of the push must stay as they are until the table's next pull_op, sync or other waiting
+ * call has returned.  Off by default (then everything a push reads is read in the order of `stream`). */
+int tn_sparse_table_set_detached_updates(uint32_t handle, int enable);
+
 /* ------------------------------------------------------------- dense table */
 /* CreateDenseTable (core/ps/table/dense_table.cc:180-186); Adam or AdaGrad.  With shard_num > 1
  * the table is worker self_shard_id's share: after Init it owns the contiguous range

@@ -171,6 +171,9 @@ public:
     int Clear() { return tn_sparse_table_clear(handle_); }
     // small batches on the path of few launches (the default) or on the one every other batch takes: same results
     int SetSmallBatchPath(bool enable) { return tn_sparse_table_set_small_batch_path(handle_, enable ? 1 : 0); }
+    // the updates of a large push beside what the caller queues next; its gradients then stay untouched until the
+    // table's next waiting call has returned (the reference's push is asynchronous in the same way)
+    int SetDetachedUpdates(bool enable) { return tn_sparse_table_set_detached_updates(handle_, enable ? 1 : 0); }
     int Sync() { return tn_sparse_table_sync(handle_); }
 
 private:

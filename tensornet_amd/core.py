@@ -165,6 +165,13 @@ def set_sparse_table_small_batch_path(table_handle, enable):
     _lib.check(_lib.load().tn_sparse_table_set_small_batch_path(table_handle, 1 if enable else 0))
 
 
+def set_sparse_table_detached_updates(table_handle, enable):
+    """With detached updates the update kernels of a large push run on the table's own streams, beside whatever
+    the caller queues next (the analysis of the next pull's batch); the gradient tensors of the push must then
+    stay untouched until the table's next pull, sync or other waiting call has returned.  Off by default."""
+    _lib.check(_lib.load().tn_sparse_table_set_detached_updates(table_handle, 1 if enable else 0))
+
+
 def sparse_table_key_count(table_handle):
     n = C.c_uint64()
     _lib.check(_lib.load().tn_sparse_table_key_count(table_handle, C.byref(n)))

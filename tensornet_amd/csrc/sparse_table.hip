@@ -112,6 +112,15 @@ struct SparseTable {
     hipStream_t aux = nullptr;
     hipEvent_t fork_ev = nullptr, join_ev = nullptr, join2_ev = nullptr;
     hipEvent_t apply_ev = nullptr;  // a push's updates are done (its status is published beside what follows)
+    // Detached updates (tn_sparse_table_set_detached_updates): the update kernels of a large push run on the
+    // table's own streams and the caller's stream does not wait for them, so that whatever the caller queues next
+    // -- above all the analysis of the next pull's batch, which touches no table row -- runs beside them.
+    // upd_ev marks their end (and that of the push's status); every call on the table orders its stream behind
+    // it before it touches a row, the plan's groups or the table's memory (order_after_updates).
+    bool detach_updates = false;
+    bool detached_now = false;      // the push being queued has its updates detached
+    bool upd_pending = false;       // upd_ev has been recorded and no host-side wait has covered it since
+    hipEvent_t upd_ev = nullptr;
     // The call before this one on the table, if it left work behind on `flow_stream` that the next call of the
     // training loop may overlap with: FLOW_PULL = a pull that returned before its gather, FLOW_PUSH = a push
     // on that pull's plan.  Every entry point clears it (ensure_allocated); pull and push set it again.
@@ -278,6 +287,7 @@ int ensure_side_buffers(SparseTable* t) {
     TN_HIP(hipEventCreateWithFlags(&t->pub_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->tail_ev, hipEventDisableTiming));
     TN_HIP(hipEventCreateWithFlags(&t->apply_ev, hipEventDisableTiming));
+    TN_HIP(hipEventCreateWithFlags(&t->upd_ev, hipEventDisableTiming));
     TN_HIP(hipStreamCreateWithFlags(&t->side, hipStreamNonBlocking));  // default priority
     TN_HIP(hipStreamCreateWithFlags(&t->side2, hipStreamNonBlocking));
     TN_HIP(hipStreamCreateWithFlags(&t->aux, hipStreamNonBlocking));
@@ -299,8 +309,17 @@ uint64_t reserved_slots(const SparseTable* t, uint64_t keys) {
     return (roomy + 1) * (pitch + sizeof(uint64_t)) <= total_b / 2 ? roomy : tight;
 }
 
-int ensure_allocated(SparseTable* t, hipStream_t st) {
+// Orders `st` behind the detached updates of the last push, if any (a wait for an event that has completed
+// costs nothing on the device).
+int order_after_updates(SparseTable* t, hipStream_t st) {
+    if (t->upd_pending) TN_HIP(hipStreamWaitEvent(st, t->upd_ev, 0));
+    return TN_OK;
+}
+
+// beside_updates: the caller (the pull op) orders its stream behind detached updates itself, as late as it can.
+int ensure_allocated(SparseTable* t, hipStream_t st, bool beside_updates = false) {
     TN_TRY(ensure_side_buffers(t));
+    if (!beside_updates) TN_TRY(order_after_updates(t, st));
     // work of the last pull that its caller did not wait for was queued on that call's stream
     if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
     t->flow = FLOW_NONE;  // pull and push read it before they get here and set it again
@@ -345,6 +364,7 @@ void harvest(SparseTable* t) {
             t->push_pub_on_side = false;
             const hipError_t e = hipStreamSynchronize(t->side);
             if (e != hipSuccess) latch(t, TN_ERR_HIP, std::string("sparse push: ") + hipGetErrorString(e));
+            t->upd_pending = false;  // (detached updates end on that stream, ahead of the status)
         }
         const HostStatus& h = *t->hpush;
         int N = t->push_slots;
@@ -387,6 +407,10 @@ int take_latched(SparseTable* t) {
 }
 
 int sync_table(SparseTable* t, hipStream_t st) {
+    if (t->upd_pending) {
+        TN_HIP(hipEventSynchronize(t->upd_ev));
+        t->upd_pending = false;
+    }
     TN_HIP(hipStreamSynchronize(st));
     if (t->last_stream && t->last_stream != st) TN_HIP(hipStreamSynchronize(t->last_stream));
     harvest(t);
@@ -430,6 +454,7 @@ int read_count(SparseTable* t, hipStream_t st, uint64_t* out) {
 int ensure_room(SparseTable* t, uint64_t incoming, hipStream_t st) {
     Store& s = t->store;
     if ((double)(t->count_upper + incoming) > MAX_LOAD * (double)s.cap) {
+        TN_TRY(order_after_updates(t, st));  // growing moves the rows
         uint64_t cnt = 0;  // the bound may be loose: read the true count
         TN_TRY(read_count(t, st, &cnt));
         if ((double)(cnt + incoming) > MAX_LOAD * (double)s.cap) {
@@ -817,6 +842,8 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
                   p.u_of_gi, for_pull ? 1 : 0);
     }
     const uint32_t* ushow = use_lds ? p.ushow : nullptr;
+    // from here on the groups and member lists are written, which detached updates of the push before still read
+    TN_TRY(order_after_updates(t, st));
     if (lds_groups) {
         const int bblocks = launch_grid(w.nb2, 1, GRID_CAP * 4);
         if (!t->one_stream) {
@@ -845,22 +872,29 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
 // at the device's rate for random row updates); k_apply_big and k_apply_vec are bound by
 // dependent chains and instruction issue, so they run one after the other on the table's side
 // stream beside it, forked from and joined back into the caller's stream by events.
+//
+// detach: none of them on the caller's stream, which does not wait for them either -- k_apply_single on the
+// auxiliary stream; the caller of this function records their end (see SparseTable::upd_ev).
 template <int KIND>
 int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
-                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready, uint32_t big_k) {
+                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready, uint32_t big_k, bool detach) {
     const uint32_t ids_cap = (uint32_t)n_upper;
     const bool with_big = big_k != 0xFFFFFFFFu;
     const float* const* gaddr = (with_big && !src.infos && !src.flat) ? p.gaddr : nullptr;
+    detach = detach && !t->one_stream && lpg != 0;
+    t->detached_now = detach;
+    const bool forked = (with_big || detach) && !t->one_stream;
+    // op-level gradients: their addresses for the records of the groups with several records, once, in a
+    // coalesced pass ahead of everything (beside k_apply_single it would take several times as long)
+    if (with_big && gaddr && !addr_ready)
+        TN_LAUNCH(k_member_grads, dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, src, ds, p.list,
+                  p.gaddr, ids_cap);
+    if (forked) {
+        TN_HIP(hipEventRecord(t->fork_ev, st));
+        TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+        if (detach) TN_HIP(hipStreamWaitEvent(t->aux, t->fork_ev, 0));
+    }
     if (with_big) {
-        // op-level gradients: their addresses for the records of the groups with several records, once, in a
-        // coalesced pass ahead of everything (beside k_apply_single it would take several times as long)
-        if (gaddr && !addr_ready)
-            TN_LAUNCH(k_member_grads, dim3(launch_grid(n_upper, 256, GRID_CAP * 2)), dim3(256), st, src, ds, p.list,
-                      p.gaddr, ids_cap);
-        if (!t->one_stream) {
-            TN_HIP(hipEventRecord(t->fork_ev, st));
-            TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
-        }
         const int gfloats = big_gbuf_floats(s.D);
         TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
                       big_lds_bytes(s.D), t->one_stream ? st : t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
@@ -868,10 +902,10 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
-        TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256), st, s, \
-                  o, src, ds, p.grp_row, p.list);                                                                 \
+        TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256),    \
+                  detach ? t->aux : st, s, o, src, ds, p.grp_row, p.list);                                        \
         TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256),    \
-                  with_big && !t->one_stream ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,    \
+                  forked ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,  \
                   gaddr);                                                                                         \
     } while (0)
     switch (lpg) {
@@ -886,7 +920,7 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
                       p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap);
     }
 #undef TN_LAUNCH_VEC
-    if (with_big && !t->one_stream) {
+    if (forked && !detach) {
         TN_HIP(hipEventRecord(t->join_ev, t->side));
         TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
     }
@@ -904,15 +938,15 @@ int lanes_per_group(const Store& s, bool vec_ok) {
 // addr_ready: p.gaddr already holds the gradient addresses of the multi-record groups' records.
 // big_k: the number of records from which the plan's grouping listed a sign for k_apply_big (0: the table's default).
 int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
-                 hipStream_t st, bool addr_ready = false, uint32_t big_k = 0) {
+                 hipStream_t st, bool addr_ready = false, uint32_t big_k = 0, bool detach = false) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     const int lpg = lanes_per_group(s, vec_ok);
     if (big_k == 0) big_k = big_threshold(s);
     switch (o.kind) {
-        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
-        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
-        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k);
+        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
+        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
+        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
     }
 }
 
@@ -1156,6 +1190,14 @@ int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable) {
     if (!t) return fail(TN_ERR_BAD_HANDLE, "bad sparse table handle");
     std::lock_guard<std::mutex> lk(t->mu);
     t->small_path = enable != 0;
+    return TN_OK;
+}
+
+int tn_sparse_table_set_detached_updates(uint32_t handle, int enable) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad sparse table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->detach_updates = enable != 0;
     return TN_OK;
 }
 
@@ -1541,7 +1583,9 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     hipStream_t st = (hipStream_t)stream;
     // the call before was a push on the last pull's plan, on this stream: its updates may still be running
     bool behind_push = t->flow == FLOW_PUSH && t->flow_stream == st;
-    TN_TRY(ensure_allocated(t, st));
+    // (detached updates of the push before: the analysis of this call's batch runs beside them; the stream is
+    // ordered behind them where the call first touches what they read or write)
+    TN_TRY(ensure_allocated(t, st, true));
     const int wdim = t->dim + (t->use_cvm ? 2 : 0);
     if (var_dim != wdim)
         return fail(TN_ERR_DIM_MISMATCH, "SparseTablePull: variable dim " + std::to_string(var_dim) +
@@ -1549,6 +1593,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     // An earlier push on the same stream need not be waited for: this call runs behind it and
     // collects its status when it waits for its own work.
     const bool same_stream = !t->last_stream || t->last_stream == st;
+    if (!same_stream || t->async_pull) TN_TRY(order_after_updates(t, st));
     if (t->pull_pending || (t->push_pending && (t->async_pull || !same_stream))) {
         if (!same_stream) TN_HIP(hipStreamSynchronize(t->last_stream));
         TN_HIP(hipStreamSynchronize(st));
@@ -1596,6 +1641,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         w.span_cap = span_cap;
         t->plan_valid = false;
         if (small) {
+            TN_TRY(order_after_updates(t, st));
             if (t->stage_pending) {
                 TN_HIP(hipEventSynchronize(t->stage_ev));
                 t->stage_pending = false;
@@ -1672,7 +1718,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         // Behind a push of the training loop the descriptors go in on the auxiliary stream, beside that push's
         // updates: those read the push's own descriptors and status block, and nothing of the scratch buffer.
         // (Same slot count: the arrays at the head of the plan buffer keep their places.)
-        const bool hoist = behind_push && attempt == 0 && !t->one_stream && N == t->plan_N;
+        const bool hoist = behind_push && attempt == 0 && !t->one_stream && N == t->plan_N && !t->upd_pending;
         behind_push = false;
         if (hoist && t->tail_recorded) TN_HIP(hipStreamWaitEvent(t->aux, t->tail_ev, 0));  // the gather that read p.descs
         TN_TRY(upload_slots(t, p.descs, p.lbase, t->dplan, descs, lbase, hoist ? t->aux : st, STATUS_NEW_PLAN,
@@ -2000,9 +2046,22 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         // return at once when the mismatch flag is set.  The device never waits for the host.
         if (!t->plan_has_show) TN_TRY(launch_counts());
         TN_TRY(prepare_src());
-        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify, t->plan_big_k));
+        TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify, t->plan_big_k,
+                            t->detach_updates && !pooled));
+        if (t->detached_now) {
+            // their end, for whoever touches the table next; the status goes out behind them (below)
+            TN_HIP(hipEventRecord(t->apply_ev, t->aux));
+            TN_HIP(hipStreamWaitEvent(t->side, t->apply_ev, 0));
+        }
         TN_HIP(hipEventSynchronize(t->verify_ev));
         reuse = t->hpush->st.mismatch == 0;
+        if (t->detached_now && !reuse) {
+            // (the update kernels return at once on a mismatch; what follows works on the caller's stream)
+            TN_HIP(hipEventRecord(t->upd_ev, t->side));
+            t->upd_pending = true;
+            t->detached_now = false;
+            TN_TRY(order_after_updates(t, st));
+        }
     }
     if (!reuse) {
         // another batch than the last pull's: analyse it here, on the global-table path
@@ -2025,12 +2084,18 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     // The status of a large push goes out on the side stream, behind the updates and beside whatever the caller's
     // stream runs next (a pull's status follows it on that stream, so whoever has that one has this one too).
     const bool pub_on_side = reuse && !t->one_stream;
-    if (pub_on_side) {
+    const bool detached = reuse && t->detached_now;  // (the side stream is behind all update kernels already)
+    t->detached_now = false;
+    if (pub_on_side && !detached) {
         TN_HIP(hipEventRecord(t->apply_ev, st));
         TN_HIP(hipStreamWaitEvent(t->side, t->apply_ev, 0));
     }
     TN_LAUNCH(k_publish, dim3(1), dim3(256), pub_on_side ? t->side : st, ds, pub_ubase ? pub_ubase : p.ubase,
               (uint32_t)(N + 1), reinterpret_cast<uint32_t*>(t->hpush), (unsigned long long*)nullptr, (uint32_t*)nullptr, 0u);
+    if (detached) {
+        TN_HIP(hipEventRecord(t->upd_ev, t->side));
+        t->upd_pending = true;
+    }
     t->push_pending = true;
     t->push_pub_on_side = pub_on_side;
     t->push_slots = N;

@@ -592,6 +592,74 @@ def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, chang
     assert "k_verify_values<true, false>" in step(values, 2)
 
 
+def test_detached_updates_are_seen_by_whatever_touches_the_table_next(tn, oracle):
+    """tn_sparse_table_set_detached_updates: the update kernels of a large push (3 M lookups or more) run beside
+    what the caller queues next.  Steps queued back to back without the host waiting in between -- the next pull's
+    batch shares most signs with the push before it, so its variables must hold the updated rows; a small batch
+    and a table-level call in between, a push of another batch than the pull's, and the final table -- against
+    the oracle, which runs the same sequence one call after the other."""
+    D = 16
+    rng = np.random.default_rng(2024)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=10 ** 6)
+    tn.core.set_sparse_table_detached_updates(pair.h, True)
+    vocab = 300000
+    base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
+    pool = base.view(np.int64)
+    hot = pool[:40]
+
+    def batch(slots, per):
+        out = []
+        for _ in range(slots):
+            v = pool[(rng.random(per) ** 3 * vocab).astype(np.int64)]
+            v[: len(hot)] = hot  # signs with a record in every slot: updated record after record, in slot order
+            out.append(v)
+        return out
+
+    big = [batch(64, 50000) for _ in range(2)]  # 3.2 M lookups each: updates on the table's own streams
+    assert all(sum(len(v) for v in b) >= 3 << 20 for b in big)
+    small = batch(8, 1000)
+    sequence = [big[0], big[1], small, big[0], big[1]]
+    steps = []
+    for k, values in enumerate(sequence):
+        counts = [len(np.unique(v)) for v in values]
+        steps.append(dict(values=values, gvalues=[dev(v) for v in values],
+                          gvars=[torch.zeros((len(v) + 1, D), device="cuda") for v in values],
+                          grads=synth.make_grads(counts, D, 0.01, seed=k),
+                          labels=[(rng.random(len(v)) < 0.2).astype(np.int64) for v in values]))
+    for st in steps:  # (the gradient tensors stay alive and untouched until the end: what the mode asks for)
+        st["ggrads"] = [dev(g) for g in st["grads"]]
+        st["glabels"] = [dev(l) for l in st["labels"]]
+    # the device side, nothing waited for but what the pulls wait for themselves
+    for k, st in enumerate(steps):
+        st["gmapped"] = tn.ops.sparse_table_pull(st["gvars"], st["gvalues"], pair.h)
+        tn.ops.sparse_table_push(st["gvalues"], st["ggrads"], st["glabels"], pair.h)
+        if k == 1:  # a table-level call right behind a detached push: the rows it reads are the updated ones
+            st["table_pull"] = tn.ops.table_pull(pair.h, dev(hot), D)
+    # a push of another batch than the last pull's, behind a detached push
+    other = batch(64, 50000)
+    other_counts = [len(np.unique(v)) for v in other]
+    other_grads = synth.make_grads(other_counts, D, 0.01, seed=99)
+    other_labels = [np.zeros(len(v), np.int64) for v in other]
+    gother = ([dev(v) for v in other], [dev(g) for g in other_grads], [dev(l) for l in other_labels])
+    tn.ops.sparse_table_push(gother[0], gother[1], gother[2], pair.h)
+    tn.ops.sparse_table_sync(pair.h)
+    # the oracle, call by call
+    for k, st in enumerate(steps):
+        cvars = [np.zeros((len(v) + 1, D), np.float32) for v in st["values"]]
+        rc, cmapped, counts = pair.o.pull_op(st["values"], cvars)
+        assert rc == 0
+        for s in range(len(cvars)):
+            assert (st["gmapped"][s].cpu().numpy() == cmapped[s]).all()
+            np.testing.assert_allclose(st["gvars"][s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
+        assert pair.o.push_op(st["values"], st["grads"], st["labels"])[0] == 0
+        if k == 1:
+            cw, _, cf = pair.o.get_rows(hot.view(np.uint64))
+            assert cf.all()
+            np.testing.assert_allclose(st["table_pull"].cpu().numpy(), cw[:, :D], rtol=RTOL, atol=ATOL)
+    assert pair.o.push_op(other, other_grads, other_labels)[0] == 0
+    assert pair.assert_rows_match(base) > 0.99
+
+
 @pytest.mark.parametrize("D", [8, 12, 64, 128])
 @pytest.mark.parametrize("opt,hyper", [("AdaGrad", ADAGRAD_HP), ("Adam", ADAM_HP)])
 def test_table_push_one_sign_with_very_many_records(tn, oracle, opt, hyper, D):
