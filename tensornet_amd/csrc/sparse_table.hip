@@ -121,6 +121,10 @@ struct SparseTable {
     bool detached_now = false;      // the push being queued has its updates detached
     bool upd_pending = false;       // upd_ev has been recorded and no host-side wait has covered it since
     hipEvent_t upd_ev = nullptr;
+    // what the detached kernels read of the plan buffer: the slot arrays at its head (laid out by the slot count)
+    // and the groups from upd_groups_off on, less the first upd_slack bytes (the groups' signs, which they leave alone)
+    int upd_N = 0;
+    size_t upd_groups_off = 0, upd_slack = 0;
     // The call before this one on the table, if it left work behind on `flow_stream` that the next call of the
     // training loop may overlap with: FLOW_PULL = a pull that returned before its gather, FLOW_PUSH = a push
     // on that pull's plan.  Every entry point clears it (ensure_allocated); pull and push set it again.
@@ -1640,6 +1644,12 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         carve_scratch((char*)t->ws.p, w, L, dt_entries, lds_scratch, t->distinct_est);
         w.span_cap = span_cap;
         t->plan_valid = false;
+        // Detached updates of the push before read its plan in this same buffer.  A batch of the same slot count
+        // and about the same size lays its plan out over it array by array, and what this call writes before it
+        // orders itself behind them (the per-lookup arrays) stays clear of what they read; any other batch waits.
+        if (t->upd_pending && (N != t->upd_N || (size_t)((const char*)p.grp_sign - (const char*)t->plan_buf.p) >
+                                                    t->upd_groups_off + t->upd_slack))
+            TN_TRY(order_after_updates(t, st));
         if (small) {
             TN_TRY(order_after_updates(t, st));
             if (t->stage_pending) {
@@ -2095,6 +2105,9 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     if (detached) {
         TN_HIP(hipEventRecord(t->upd_ev, t->side));
         t->upd_pending = true;
+        t->upd_N = N;
+        t->upd_groups_off = (size_t)((const char*)p.grp_sign - (const char*)t->plan_buf.p);
+        t->upd_slack = (size_t)((const char*)p.grp_row - (const char*)p.grp_sign);
     }
     t->push_pending = true;
     t->push_pub_on_side = pub_on_side;

@@ -607,7 +607,7 @@ def test_detached_updates_are_seen_by_whatever_touches_the_table_next(tn, oracle
     pool = base.view(np.int64)
     hot = pool[:40]
 
-    def batch(slots, per):
+    def batch(slots, per):  # (every batch used below has 3 M lookups or more, but `small`)
         out = []
         for _ in range(slots):
             v = pool[(rng.random(per) ** 3 * vocab).astype(np.int64)]
@@ -618,7 +618,9 @@ def test_detached_updates_are_seen_by_whatever_touches_the_table_next(tn, oracle
     big = [batch(64, 50000) for _ in range(2)]  # 3.2 M lookups each: updates on the table's own streams
     assert all(sum(len(v) for v in b) >= 3 << 20 for b in big)
     small = batch(8, 1000)
-    sequence = [big[0], big[1], small, big[0], big[1]]
+    # (a batch with more slots and one with many more lookups than the push before it: their plans do not lie over
+    # the plan the update kernels still read, so those pulls wait for the updates first)
+    sequence = [big[0], big[1], small, big[0], batch(80, 42000), big[1], batch(64, 72000), big[0]]
     steps = []
     for k, values in enumerate(sequence):
         counts = [len(np.unique(v)) for v in values]
