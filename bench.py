@@ -195,7 +195,7 @@ def main():
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
     ap.add_argument("--detached-updates", action="store_true",
                     help="the timed steps with the push's update kernels detached (tn_sparse_table_set_detached_updates)")
-    ap.add_argument("--no-detached", action="store_true", help="skip the side measurement of detached updates")
+    ap.add_argument("--detached", action="store_true", help="add the side measurement of detached updates")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -404,7 +404,7 @@ def main():
     # (tn_sparse_table_set_detached_updates: they then run beside the analysis of the next pull's batch; the
     # gradient tensors must outlive the call, which is why the timed steps above do not use it.)  Batches of
     # their own again, so that the steps insert their share of new signs.
-    if mean_L >= (3 << 20) and not args.no_detached and not args.detached_updates:
+    if mean_L >= (3 << 20) and args.detached and not args.detached_updates:
         dsteps, dwarm = 10, 2
         more = []
         for b in range(nb + 2, nb + 2 + dwarm + dsteps):
