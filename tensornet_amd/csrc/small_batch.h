@@ -543,7 +543,7 @@ __global__ __launch_bounds__(256) void k_small_apply(Store s, OptDev o, PushSrc 
     for (uint32_t t = (blockIdx.x - big_blocks) * (blockDim.x / LPG) + threadIdx.x / LPG; t < n_single + n_multi; t += gstride) {
         const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
         const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;
+        if (row > s.cap) continue;  // NO_ROW, or no row number at all: never address the table with it
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
         apply_group_vec<KIND, LPG, 4>(s, o, src, status, row, k, list + grp_off[g], nullptr, sub, lane0, c1, c2);

@@ -1448,7 +1448,7 @@ __global__ __launch_bounds__(256) void k_apply_single(Store s, OptDev o, PushSrc
     const float c1 = 1 - o.beta1, c2 = 1 - o.beta2;
     for (uint32_t g = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; g < n_single; g += gstride) {
         const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
+        if (row > s.cap) continue;  // NO_ROW (unknown sign: flagged by the probe), or no row number at all
         const float* gp;
         int bshow, bclick;
         if (!src_record(src, list[g], gp, bshow, bclick)) {
@@ -1682,7 +1682,7 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
     for (uint32_t gi = blockIdx.x * (blockDim.x / LPG) + threadIdx.x / LPG; gi < n_multi; gi += gstride) {
         const uint32_t g = ids_cap - n_multi + gi;  // groups with several records sit at the top of the id space
         const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;  // unknown sign: already flagged by the probe
+        if (row > s.cap) continue;  // NO_ROW (unknown sign: flagged by the probe), or no row number at all
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
         apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g], gaddr ? gaddr + grp_off[g] : nullptr, sub,
@@ -1752,7 +1752,7 @@ __device__ __forceinline__ void apply_big_groups(const Store& s, const OptDev& o
     for (uint32_t bi = first; bi < n_big; bi += stride) {
         const uint32_t g = big_list[bi];
         const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;
+        if (row > s.cap) continue;  // NO_ROW, or no row number at all: never address the table with it
         const uint32_t k = grp_cnt[g];
         const uint32_t off = grp_off[g];
         float* wp = s.w + (uint64_t)row * s.wstride;
@@ -1957,7 +1957,7 @@ __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc
     for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < n_single + n_multi; t += stride) {
         const uint32_t g = group_id(t, n_single, n_multi, ids_cap);
         const uint32_t row = grp_row[g];
-        if (row == NO_ROW) continue;
+        if (row > s.cap) continue;  // NO_ROW, or no row number at all: never address the table with it
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
         const Member* mem = list + grp_off[g];
