@@ -740,16 +740,16 @@ __global__ __launch_bounds__(1024) void k_group_offsets(const uint4* __restrict_
 // and streaming work).  A sign present in several slots is probed once per slot; whichever
 // thread claims a free slot first owns the insertion, the others find the key there.
 // A new row is not filled here: one or two lanes of a wavefront drawing sixteen normal deviates would hold up
-// the other sixty (with 1 % of the lookups new, most wavefronts have such a lane); the record is listed in
-// newlist and k_init_new_recs fills the rows with every lane busy.
+// the other sixty (with 1 % of the lookups new, most wavefronts have such a lane); the record is listed and
+// k_init_new_recs fills the rows with every lane busy.  The list is the bucket's own -- newrec[c * GRP_CAP ...],
+// newcnt[c] entries -- not one list of the call: places in one list are handed out by atomics on one counter,
+// which take about 11 ns each one after the other (one per wavefront, tens of thousands, took longer than all the
+// probes together; one per bucket still kept every workgroup waiting for its turn among a thousand).
 __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, uint32_t* __restrict__ rrow,
-                                                    uint32_t* __restrict__ newlist, Store s, DevStatus* status) {
-    // The new rows of a bucket are collected in LDS and get their places in newlist with ONE atomic on the
-    // call's counter: an atomic per wavefront (tens of thousands on one address, about 11 ns each one after
-    // the other) took longer than all the probes together.
-    __shared__ uint32_t s_new[GRP_CAP];
-    __shared__ uint32_t s_count, s_base;
+                                                    uint32_t* __restrict__ newrec, uint32_t* __restrict__ newcnt,
+                                                    Store s, DevStatus* status) {
+    __shared__ uint32_t s_count;
     for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
         const uint32_t n = min(cursor2[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
@@ -764,15 +764,10 @@ __global__ __launch_bounds__(256) void k_probe_recs(uint32_t nb2, const uint32_t
                 rrow[first + i] = row;
                 if (row == NO_ROW) atomicOr(&status->err, DEV_ERR_TABLE_FULL);
             }
-            if (is_new) s_new[atomicAdd(&s_count, 1u)] = i;  // rare: about one record in forty
+            if (is_new) newrec[first + atomicAdd(&s_count, 1u)] = i;  // rare: about one record in forty (at most n)
         }
         __syncthreads();
-        const uint32_t cnt = s_count;
-        if (cnt) {
-            if (threadIdx.x == 0) s_base = atomicAdd(&status->n_new, cnt);
-            __syncthreads();
-            for (uint32_t j = threadIdx.x; j < cnt; j += 256) newlist[s_base + j] = (uint32_t)(first + s_new[j]);
-        }
+        if (threadIdx.x == 0) newcnt[c] = s_count;
         __syncthreads();
     }
 }
@@ -797,20 +792,31 @@ __device__ __forceinline__ void init_row_pair(const Store& s, const OptDev& o, u
     }
 }
 
-// Fills the rows k_probe_recs inserted: one lane per pair of elements.
+// Fills the rows k_probe_recs inserted, a workgroup per bucket's list and one lane per pair of elements; the first
+// workgroup also adds up the lists' lengths: the call's number of new rows.
 __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64_t seed,
                                                        const GroupRec* __restrict__ recs,
-                                                       const uint32_t* __restrict__ rrow,
-                                                       const uint32_t* __restrict__ newlist, const DevStatus* status) {
-    const uint32_t n_new = status->n_new;
+                                                       const uint32_t* __restrict__ rrow, uint32_t nb2,
+                                                       const uint32_t* __restrict__ newrec,
+                                                       const uint32_t* __restrict__ newcnt, DevStatus* status) {
+    __shared__ uint32_t red[4];
+    if (blockIdx.x == 0) {
+        uint32_t mine = 0;
+        for (uint32_t c = threadIdx.x; c < nb2; c += 256) mine += min(newcnt[c], (uint32_t)GRP_CAP);
+        uint32_t total;
+        block_excl_scan_256<uint32_t>(mine, red, &total);
+        if (threadIdx.x == 0) status->n_new = total;
+    }
     const uint32_t pairs = (uint32_t)(s.D + 1) / 2;
-    const uint64_t total = (uint64_t)n_new * pairs;
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     const float stddev = (float)(1.0 / sqrt((double)s.D));
-    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += stride) {
-        const uint32_t j = (uint32_t)(t / pairs), q = (uint32_t)(t - (uint64_t)j * pairs);
-        const uint32_t i = newlist[j];
-        init_row_pair(s, o, seed, recs[i].sign, rrow[i], q, stddev);
+    for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
+        const uint32_t cnt = min(newcnt[c], (uint32_t)GRP_CAP);
+        const size_t first = (size_t)c * GRP_CAP;
+        for (uint32_t t = threadIdx.x; t < cnt * pairs; t += 256) {
+            const uint32_t j = t / pairs, q = t - j * pairs;
+            const size_t i = first + min(newrec[first + j], (uint32_t)GRP_CAP - 1);
+            init_row_pair(s, o, seed, recs[i].sign, rrow[i], q, stddev);
+        }
     }
 }
 

@@ -26,7 +26,6 @@ constexpr double MAX_LOAD = 0.75;                       // optimizer_kernel.h:26
 constexpr double RESERVE_LOAD = 0.5;                    // what a reservation is sized for where memory allows
 constexpr uint64_t DEFAULT_SLOTS = 8ull * 15485863ull;  // optimizer_kernel.h:43,263
 constexpr uint64_t MAX_SLOTS_PER_TABLE = 0xFFFFFFF0ull; // rows are addressed with 32 bits
-constexpr int INIT_NEW_GRID = 512;    // workgroups of k_init_new_recs (the number of new rows is known on the device only)
 constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 512-1024 are best)
 // Below this many lookups a call keeps all its kernels on the caller's stream.  The kernels of a smaller
 // batch are too short for the overlap on the side streams to win back what the events that fork and
@@ -506,7 +505,6 @@ struct Plan {
     Member* list;          // members of every group, ascending (with their show / click counts)
     uint2* where_u;        // record -> {its place in `list`, its group}
     uint32_t* big_list;    // groups with BIG_GROUP records or more
-    uint32_t* newlist;     // groups whose row was inserted by the pull
     const float** gaddr;   // gradient row of every record of the groups with several records (a push fills it)
 };
 
@@ -535,6 +533,8 @@ struct Scratch {
     GroupRec* recs;
     uint2* aux;
     uint32_t* rrow;      // per distinct record: table row of its sign
+    uint32_t* newrec;    // per second-level bucket: its records whose rows the pull inserted ...
+    uint32_t* newcnt;    // ... and how many
     uint4* bcounts;
     uint4* bbase;
     void* gt;  // GroupEntry[] or MaskEntry[]
@@ -558,7 +558,6 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.list = c.take<Member>(n);
     p.where_u = c.take<uint2>(n);
     p.big_list = c.take<uint32_t>(n / std::min<uint32_t>(BIG_GROUP, SMALL_BIG_GROUP) + 64);  // (the lowest threshold a plan may use)
-    p.newlist = c.take<uint32_t>(n);
     p.gaddr = c.take<const float*>(n);
 }
 
@@ -607,6 +606,8 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.recs = c.take<GroupRec>(nb2_room * GRP_CAP);
         w.aux = c.take<uint2>(nb2_room * GRP_CAP);
         w.rrow = c.take<uint32_t>(nb2_room * GRP_CAP);
+        w.newrec = c.take<uint32_t>(nb2_room * GRP_CAP);
+        w.newcnt = c.take<uint32_t>(nb2_room);
         w.bcounts = c.take<uint4>(nb2_room);
         w.bbase = c.take<uint4>(nb2_room);
         w.bstart = c.take<uint32_t>(nb1_room + 1);
@@ -814,9 +815,9 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             }
             // few workgroups: enough probes in flight for the memory system, most of every CU left to the grouping
             TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), sd2, w.nb2, w.cursor2, w.recs, w.rrow,
-                      p.newlist, s, ds);
-            TN_LAUNCH(k_init_new_recs, dim3(INIT_NEW_GRID), dim3(256), sd2, s, make_optdev(t), t->seed, w.recs, w.rrow,
-                      p.newlist, ds);
+                      w.newrec, w.newcnt, s, ds);
+            TN_LAUNCH(k_init_new_recs, dim3(std::min(bblocks, GRID_CAP)), dim3(256), sd2, s, make_optdev(t), t->seed,
+                      w.recs, w.rrow, w.nb2, w.newrec, w.newcnt, ds);
             if (!t->one_stream) TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
