@@ -792,13 +792,15 @@ __device__ __forceinline__ void init_row_pair(const Store& s, const OptDev& o, u
     }
 }
 
-// Fills the rows k_probe_recs inserted, a workgroup per bucket's list and one lane per pair of elements; the first
-// workgroup also adds up the lists' lengths: the call's number of new rows.
+// Fills the rows k_probe_recs inserted, `parts` workgroups per bucket's list (a batch of few buckets and many new
+// signs still fills the device) and one lane per pair of elements; the first workgroup also adds up the lists'
+// lengths: the call's number of new rows.
 __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64_t seed,
                                                        const GroupRec* __restrict__ recs,
                                                        const uint32_t* __restrict__ rrow, uint32_t nb2,
                                                        const uint32_t* __restrict__ newrec,
-                                                       const uint32_t* __restrict__ newcnt, DevStatus* status) {
+                                                       const uint32_t* __restrict__ newcnt, DevStatus* status,
+                                                       uint32_t parts) {
     __shared__ uint32_t red[4];
     if (blockIdx.x == 0) {
         uint32_t mine = 0;
@@ -809,10 +811,11 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
     }
     const uint32_t pairs = (uint32_t)(s.D + 1) / 2;
     const float stddev = (float)(1.0 / sqrt((double)s.D));
-    for (uint32_t c = blockIdx.x; c < nb2; c += gridDim.x) {
+    for (uint32_t w = blockIdx.x; w < nb2 * parts; w += gridDim.x) {
+        const uint32_t c = w / parts, part = w - c * parts;
         const uint32_t cnt = min(newcnt[c], (uint32_t)GRP_CAP);
         const size_t first = (size_t)c * GRP_CAP;
-        for (uint32_t t = threadIdx.x; t < cnt * pairs; t += 256) {
+        for (uint32_t t = part * 256 + threadIdx.x; t < cnt * pairs; t += parts * 256) {
             const uint32_t j = t / pairs, q = t - j * pairs;
             const size_t i = first + min(newrec[first + j], (uint32_t)GRP_CAP - 1);
             init_row_pair(s, o, seed, recs[i].sign, rrow[i], q, stddev);

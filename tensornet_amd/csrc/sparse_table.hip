@@ -816,8 +816,9 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
             // few workgroups: enough probes in flight for the memory system, most of every CU left to the grouping
             TN_LAUNCH(k_probe_recs, dim3(std::min(bblocks, PROBE_RECS_GRID)), dim3(256), sd2, w.nb2, w.cursor2, w.recs, w.rrow,
                       w.newrec, w.newcnt, s, ds);
-            TN_LAUNCH(k_init_new_recs, dim3(std::min(bblocks, GRID_CAP)), dim3(256), sd2, s, make_optdev(t), t->seed,
-                      w.recs, w.rrow, w.nb2, w.newrec, w.newcnt, ds);
+            const uint32_t init_parts = std::max<uint32_t>(1, (uint32_t)GRID_CAP / w.nb2);
+            TN_LAUNCH(k_init_new_recs, dim3(launch_grid((int64_t)w.nb2 * init_parts, 1, GRID_CAP)), dim3(256), sd2, s,
+                      make_optdev(t), t->seed, w.recs, w.rrow, w.nb2, w.newrec, w.newcnt, ds, init_parts);
             if (!t->one_stream) TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
         TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
