@@ -782,7 +782,9 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     // second-level buckets up to which k_group_emit adds up the bucket counts itself (one bucket per workgroup)
     const bool own_offsets = w.nb2 <= (uint32_t)GRID_CAP * 4;
     if (use_lds) {
-        const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP);
+        // (a workgroup per tile up to twice what the chip holds at once: the workgroups queued behind the resident ones
+        // start as those end, which evens the tail out better than a second tile for some of them)
+        const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP * 2);
         const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
         TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount,
                       reinterpret_cast<ulonglong2*>(p.vals_copy), w.first_of, ds, w.span_cap);
