@@ -151,7 +151,8 @@ class Table(object):
         self.sf = load().orc_table_state_floats(self._h)
 
     def __del__(self):
-        if getattr(self, "_h", None):
+        # (at interpreter exit the module's globals may be gone before the last table is)
+        if getattr(self, "_h", None) and load is not None:
             load().orc_table_destroy(self._h)
             self._h = None
 
