@@ -179,8 +179,10 @@ int tn_sparse_table_row_layout(uint32_t handle, int* weight_floats, int* state_f
 int tn_sparse_table_pull(uint32_t handle, const uint64_t* signs, int64_t n, int dim, float* out, void* stream);
 
 /*
- * The same pull for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no hipMalloc / hipFree:
+ * The same pull for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, code that runs between the captures of HIP graphs -- the call itself waits for its stream and
+ * copies its status to the host, so it cannot be recorded into a graph).  No counterpart in the reference.
+ * It calls no hipMalloc / hipFree:
  * the row numbers and the new-row list of the call live in a static device array of the library (8 MiB + 256 B,
  * held by every GPU the library runs on until the process ends), so
  *   - n is at most 1048576 signs per call (TN_ERR_UNSUPPORTED beyond that);
@@ -247,9 +249,14 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
  * sign batch_show = occurrences and batch_click = sum of labels
  * (sparse_table_ops.cc:283-296); records are applied slot-major, so a sign
  * present in k slots receives k sequential Applies, slot 0 first.
- * Enqueues the update and returns without waiting, like the reference op
- * (sparse_table_ops.cc:363-367); errors of the enqueued work are reported by
- * the next synchronising call on the table or by tn_sparse_table_sync().
+ * Enqueues the updates and returns without waiting for them, like the
+ * reference op (sparse_table_ops.cc:363-367); errors of the enqueued work are
+ * reported by the next synchronising call on the table or by
+ * tn_sparse_table_sync().  One wait remains: a push that follows the pull op
+ * of the same batch reuses what that pull worked out about the batch once the
+ * device has confirmed that the signs are the same, and the call returns when
+ * that comparison (one pass over the signs, queued ahead of the updates) has
+ * reported to the host.
  */
 int tn_sparse_table_push_op(uint32_t table_handle, int N, const int64_t* const* values, const int64_t* value_lens,
                             const float* const* grads, const int64_t* grad_rows, int grad_dim,
@@ -353,6 +360,14 @@ int tn_sparse_table_set_async(uint32_t handle, int async_pull);
  * of few launches (the default) or the one every other batch takes.  Same results either way; a switch for
  * measurements and tests, without a counterpart in the reference. */
 int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable);
+
+/* How a push_op recognises the batch of the pull_op before it on large batches (the reference has no such
+ * step: every push analyses its batch itself, sparse_table_ops.cc:274-297).  By default the device compares
+ * fingerprints of the signs, 16 bytes per 64 lookups (one changed sign always shows; several changed signs
+ * escape only if two 64-bit hash sums agree by chance).  With exact verify the pull keeps a copy of its
+ * signs (8 bytes per lookup more in the table's plan buffer) and the push compares the signs themselves,
+ * as the pushes of small batches always do.  Off by default; takes effect from the next pull_op. */
+int tn_sparse_table_set_exact_verify(uint32_t handle, int enable);
 
 /* The reference's push op hands its gradients to the servers and returns; the rows are updated while the
  * worker goes on (SparseTablePushKernel::ComputeAsync, sparse_table_ops.cc:346-365: requests started, done()

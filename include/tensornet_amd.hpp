@@ -174,6 +174,8 @@ public:
     // the updates of a large push beside what the caller queues next; its gradients then stay untouched until the
     // table's next waiting call has returned (the reference's push is asynchronous in the same way)
     int SetDetachedUpdates(bool enable) { return tn_sparse_table_set_detached_updates(handle_, enable ? 1 : 0); }
+    // a large push compares the signs of its batch with a copy the pull kept, instead of with their fingerprints
+    int SetExactVerify(bool enable) { return tn_sparse_table_set_exact_verify(handle_, enable ? 1 : 0); }
     int Sync() { return tn_sparse_table_sync(handle_); }
 
 private:

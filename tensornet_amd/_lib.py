@@ -128,6 +128,7 @@ SIGNATURES = {
     "tn_sparse_table_set_async": (C.c_int, [C.c_uint32, C.c_int]),
     "tn_sparse_table_set_small_batch_path": (C.c_int, [C.c_uint32, C.c_int]),
     "tn_sparse_table_set_detached_updates": (C.c_int, [C.c_uint32, C.c_int]),
+    "tn_sparse_table_set_exact_verify": (C.c_int, [C.c_uint32, C.c_int]),
     "tn_dense_table_create": (C.c_int, [C.c_int32, C.c_int, C.c_int, C.POINTER(C.c_uint32)]),
     "tn_dense_table_init": (C.c_int, [C.c_uint32, C.c_int, _PP, _I64P, _P]),
     "tn_dense_table_push_pull": (C.c_int, [C.c_uint32, C.c_int, _PP, _PP, _I64P, C.c_float, _P]),

@@ -16,7 +16,6 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtensornet_amd.so")
 SOURCES = ["core.hip", "dense_table.hip", "sparse_table.hip", "checkpoint.hip"]
-HEADERS = ["tn_common.h", "sparse_kernels.h"]
 
 FLAGS = [
     "--offload-arch=gfx950",

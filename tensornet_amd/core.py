@@ -172,6 +172,12 @@ def set_sparse_table_detached_updates(table_handle, enable):
     _lib.check(_lib.load().tn_sparse_table_set_detached_updates(table_handle, 1 if enable else 0))
 
 
+def set_sparse_table_exact_verify(table_handle, enable):
+    """With exact verify a large pull keeps a copy of its signs and the push that follows compares the signs
+    themselves instead of their fingerprints (16 bytes per 64 lookups).  Off by default."""
+    _lib.check(_lib.load().tn_sparse_table_set_exact_verify(table_handle, 1 if enable else 0))
+
+
 def sparse_table_key_count(table_handle):
     n = C.c_uint64()
     _lib.check(_lib.load().tn_sparse_table_key_count(table_handle, C.byref(n)))

@@ -141,8 +141,9 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
 static_assert(LDS_TILE == VERIFY_TILE, "k_lds_hist and k_verify_values fingerprint the same runs of lookups");
 __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
                                                   int N, uint32_t L, uint32_t* bcount,
-                                                  ulonglong2* __restrict__ prints, uint32_t* __restrict__ first_of,
-                                                  DevStatus* status, uint32_t span_cap) {
+                                                  ulonglong2* __restrict__ prints, uint64_t* __restrict__ exact,
+                                                  uint32_t* __restrict__ first_of, DevStatus* status,
+                                                  uint32_t span_cap) {
     extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]
     uint32_t* lb = smem;
     uint32_t* hist = smem + N + 1;
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ d
         Fingerprint print;
         for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
             print.add(gi, sign);
+            if (exact) exact[gi] = sign;  // a push is to compare the signs themselves
             first_of[gi] = gi;
             const uint32_t local = bucket_of(d, sign) - b0;
             if (local < span)

@@ -6,6 +6,7 @@
 #include "small_batch.h"
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstring>
 
@@ -102,6 +103,8 @@ struct SparseTable {
     size_t small_lds = 0;
     bool plan_small = false;   // the plan was left by a small pull: a push may take the small path, too
     bool plan_prints = false;  // the plan holds fingerprints of the batch's signs, not a copy of them
+    bool exact_verify = false; // pulls that leave fingerprints keep a copy of the signs as well, pushes compare that
+    bool plan_exact = false;   // the plan holds such a copy
     uint32_t plan_big_k = BIG_GROUP_DEFAULT;  // records from which the plan lists a sign as one for k_apply_big
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
@@ -319,12 +322,20 @@ int order_after_updates(SparseTable* t, hipStream_t st) {
     return TN_OK;
 }
 
+// A call on another stream than the table's last one: what that call left running there (a pull's gather, a small
+// push's updates: tail_ev) is waited for on the device, and a call whose status is still pending on the host.
+int order_after_other_stream(SparseTable* t, hipStream_t st) {
+    if (!t->last_stream || t->last_stream == st) return TN_OK;
+    if (t->tail_recorded) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
+    if (t->push_pending || t->pull_pending) TN_HIP(hipStreamSynchronize(t->last_stream));
+    return TN_OK;
+}
+
 // beside_updates: the caller (the pull op) orders its stream behind detached updates itself, as late as it can.
 int ensure_allocated(SparseTable* t, hipStream_t st, bool beside_updates = false) {
     TN_TRY(ensure_side_buffers(t));
     if (!beside_updates) TN_TRY(order_after_updates(t, st));
-    // work of the last pull that its caller did not wait for was queued on that call's stream
-    if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
+    TN_TRY(order_after_other_stream(t, st));
     t->flow = FLOW_NONE;  // pull and push read it before they get here and set it again
     if (t->allocated) return TN_OK;
     uint64_t cap = DEFAULT_SLOTS;
@@ -506,6 +517,7 @@ struct Plan {
     uint2* where_u;        // record -> {its place in `list`, its group}
     uint32_t* big_list;    // groups with BIG_GROUP records or more
     const float** gaddr;   // gradient row of every record of the groups with several records (a push fills it)
+    uint64_t* vals_exact;  // copy of the signs beside their fingerprints (tn_sparse_table_set_exact_verify), else nullptr
 };
 
 // Per-call scratch of the analysis.
@@ -568,7 +580,7 @@ void carve_group_scratch(Carver& c, Scratch& w, size_t n) {
     w.arrival = c.take<uint32_t>(n);
 }
 
-size_t carve_plan(char* base, Plan& p, int N, size_t L) {
+size_t carve_plan(char* base, Plan& p, int N, size_t L, bool exact = false) {
     Carver c{base};
     p.descs = c.take<SlotDesc>(N);
     p.push_descs = c.take<SlotDesc>(N);
@@ -581,6 +593,7 @@ size_t carve_plan(char* base, Plan& p, int N, size_t L) {
     p.uniq_slot = c.take<uint32_t>(L);
     p.ushow = c.take<uint32_t>(L);
     carve_groups(c, p, L);
+    p.vals_exact = exact ? c.take<uint64_t>(L) : nullptr;  // last: the other arrays keep their places either way
     return align_up(c.off, 256);
 }
 
@@ -723,12 +736,15 @@ int upload_slots(SparseTable* t, SlotDesc* dst_descs, uint32_t* dst_lbase, DevSt
     return TN_OK;
 }
 
-PushSrc op_source(const Plan& p, int dim, const SlotDesc* descs = nullptr) {
+// own_copies: the source of a push on the last pull's plan, whose kernels may still run (detached updates) or
+// be staged (the next pull's descriptors go in beside them) while the next pull rewrites p.descs and p.ubase:
+// it reads the push's own descriptors and its own copy of the slots' distinct bases.
+PushSrc op_source(const Plan& p, int dim, bool own_copies = false) {
     PushSrc src{};
     src.uniq_sign = p.uniq_sign;
     src.uniq_slot = p.uniq_slot;
-    src.ubase = p.ubase;
-    src.descs = descs ? descs : p.descs;
+    src.ubase = own_copies ? p.push_ubase : p.ubase;
+    src.descs = own_copies ? p.push_descs : p.descs;
     src.dim = dim;
     return src;
 }
@@ -787,7 +803,7 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP * 2);
         const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
         TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount,
-                      reinterpret_cast<ulonglong2*>(p.vals_copy), w.first_of, ds, w.span_cap);
+                      reinterpret_cast<ulonglong2*>(p.vals_copy), p.vals_exact, w.first_of, ds, w.span_cap);
         TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
         TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.prec,
                       w.span_cap);
@@ -1046,13 +1062,18 @@ int wait_reported(const uint32_t* flag, uint32_t want, hipStream_t st, const cha
     const auto t0 = std::chrono::steady_clock::now();
     for (;;) {
         for (int i = 0; i < 256; i++) {
-            if (*f == want) return TN_OK;
+            if (*f == want) {
+                // what the device wrote before the word (the status block) is read after it
+                std::atomic_thread_fence(std::memory_order_acquire);
+                return TN_OK;
+            }
             __builtin_ia32_pause();
         }
         if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) break;
     }
     TN_HIP(hipStreamSynchronize(st));
     if (*f != want) return fail(TN_ERR_HIP, std::string(what) + ": the device did not report");
+    std::atomic_thread_fence(std::memory_order_acquire);
     return TN_OK;
 }
 
@@ -1201,6 +1222,14 @@ int tn_sparse_table_set_small_batch_path(uint32_t handle, int enable) {
     return TN_OK;
 }
 
+int tn_sparse_table_set_exact_verify(uint32_t handle, int enable) {
+    SparseTable* t = get_table(handle);
+    if (!t) return fail(TN_ERR_BAD_HANDLE, "bad sparse table handle");
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->exact_verify = enable != 0;
+    return TN_OK;
+}
+
 int tn_sparse_table_set_detached_updates(uint32_t handle, int enable) {
     SparseTable* t = get_table(handle);
     if (!t) return fail(TN_ERR_BAD_HANDLE, "bad sparse table handle");
@@ -1319,8 +1348,10 @@ int tn_sparse_table_pull_static(uint32_t handle, const uint64_t* signs, int64_t 
     if (dev != t->device)
         return fail(TN_ERR_INVALID_ARGUMENT, "tn_sparse_table_pull_static: the table lives on device " +
                                                  std::to_string(t->device) + ", the current device is " + std::to_string(dev));
-    // work of the last pull that its caller did not wait for was queued on that call's stream
-    if (t->tail_recorded && t->last_stream != st) TN_HIP(hipStreamWaitEvent(st, t->tail_ev, 0));
+    // the prologue every entry point shares (ensure_allocated), less the allocation
+    TN_TRY(order_after_updates(t, st));
+    TN_TRY(order_after_other_stream(t, st));
+    t->flow = FLOW_NONE;
     const int wdim = t->dim + (t->use_cvm ? 2 : 0);
     if (dim != wdim)
         return fail(TN_ERR_DIM_MISMATCH, "tn_sparse_table_pull_static: dim " + std::to_string(dim) +
@@ -1642,8 +1673,9 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         if (small) dt_entries = 1;  // no first-level buckets
         Plan p{};
         Scratch w{};
-        TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L)));
-        carve_plan((char*)t->plan_buf.p, p, N, L);
+        const bool exact = t->exact_verify && use_lds && !small;
+        TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L, exact)));
+        carve_plan((char*)t->plan_buf.p, p, N, L, exact);
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, lds_scratch, t->distinct_est)));
         carve_scratch((char*)t->ws.p, w, L, dt_entries, lds_scratch, t->distinct_est);
         w.span_cap = span_cap;
@@ -1708,6 +1740,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             t->plan_clicks_dirty = false;
             t->plan_has_show = true;
             t->plan_prints = false;
+            t->plan_exact = false;
             t->plan_N = N;
             t->plan_lens.assign(value_lens, value_lens + N);
             t->plan_epoch = t->epoch;
@@ -1782,6 +1815,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         t->plan_clicks_dirty = false;  // a new plan's click sums start at zero
         t->plan_has_show = use_lds;
         t->plan_prints = use_lds;
+        t->plan_exact = exact;
         t->plan_N = N;
         t->plan_lens.assign(value_lens, value_lens + N);
         t->plan_epoch = t->epoch;
@@ -1901,7 +1935,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
     PushSrc src{};
     const uint32_t* pub_ubase = nullptr;  // a push on the pull's plan publishes its own copy of the distinct counts
     auto prepare_src = [&]() -> int {
-        src = op_source(p, grad_dim, pd);
+        src = op_source(p, grad_dim, pd == p.push_descs);
         if (!pooled) return TN_OK;
         if (!t->place_lds) {
             t->place_lds = big_lds_bytes_for(reinterpret_cast<const void*>(k_place_lookups));
@@ -1997,7 +2031,14 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
             TN_LAUNCH_LDS((k_small_verify<false>), dim3(tiles), dim3(256), vlds, st,
                           reinterpret_cast<const SlotDesc*>(t->hstage), p.push_descs, p.lbase, N, (uint32_t)L, p.vals_copy,
                           ds, p.u_of_gi, p.where_u, p.list, &t->hpush->st.mismatch);
-        TN_TRY(launch_small_apply(t, small_lpg, N, op_source(p, grad_dim, pd), ds, p, (int64_t)L, st, t->hseq + 1, seq_v));
+        // (the small path stages no copy of the slots' bases: its kernels all run on the caller's stream, ahead of
+        // whatever rewrites the plan's)
+        PushSrc small_src = op_source(p, grad_dim, true);
+        small_src.ubase = p.ubase;
+        TN_TRY(launch_small_apply(t, small_lpg, N, small_src, ds, p, (int64_t)L, st, t->hseq + 1, seq_v));
+        // what a call on another stream has to wait for: the updates are still running when this call returns
+        TN_HIP(hipEventRecord(t->tail_ev, st));
+        t->tail_recorded = true;
         TN_HIP(hipGetLastError());
         // the outcome of the comparison: the updates are queued behind it and do nothing on a mismatch
         TN_TRY(wait_reported(t->hseq + 1, seq_v, st, "SparseTablePush"));
@@ -2012,7 +2053,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         }
         reuse = false;  // another batch than the last pull's: analysed below
     } else if (reuse) {
-        carve_plan((char*)t->plan_buf.p, p, N, L);
+        carve_plan((char*)t->plan_buf.p, p, N, L, t->plan_exact);
         pd = p.push_descs;
         // behind a pull that returned before its gather the descriptors go in on the auxiliary stream, beside
         // that gather (the plan's counts are final from ready_ev on)
@@ -2032,14 +2073,15 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         uint32_t* host_mismatch = &t->hpush->st.mismatch;
         // op-level gradients (not pooled): the verify pass also works out the gradient addresses of the records
         // of the groups with several records (see k_member_grads)
-        const PushSrc vsrc = op_source(p, grad_dim, pd);
+        const PushSrc vsrc = op_source(p, grad_dim, true);
         const bool addr_in_verify = !pooled && t->plan_big_k != 0xFFFFFFFFu;
         const float** vgaddr = addr_in_verify ? p.gaddr : nullptr;
         // (a macro: the profiler names a kernel by the text of its launch)
 #define TN_VERIFY(CLICKS, COPY)                                                                                      \
     TN_LAUNCH_LDS((k_verify_values<CLICKS, COPY>), dim3(vblocks), dim3(256), vlds, st, pd, p.lbase, N, (uint32_t)L, \
-                  p.vals_copy, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr)
-        const bool copy = !t->plan_prints;
+                  then_vals, ds, p.u_of_gi, p.where_u, p.list, host_mismatch, vsrc, vgaddr)
+        const bool copy = !t->plan_prints || t->plan_exact;
+        const uint64_t* then_vals = t->plan_exact ? p.vals_exact : p.vals_copy;
         if (clicks) {
             if (t->plan_clicks_dirty)
                 TN_LAUNCH(k_reset_counts, dim3(lblocks), dim3(256), st, p.list, ds, (uint32_t)L, 1);

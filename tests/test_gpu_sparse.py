@@ -521,18 +521,22 @@ def test_bound_ops_over_several_steps_without_waiting(tn, oracle):
     pair.assert_rows_match(base)
 
 
+@pytest.mark.parametrize("exact", [False, True])
 @pytest.mark.parametrize("change", ["one sign", "neighbours change places", "change places across tiles",
                                     "last lookup", "two signs to one"])
-def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, change):
+def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, change, exact):
     """After a pull through LDS the plan keeps fingerprints of the batch's signs, 16 bytes per 64 lookups, not the
     signs: a push whose value tensors were edited in place since the pull, in one place or with two signs
     changing places, must analyse its batch itself (the oracle is given the edited batch); the unedited batch is
-    pushed on the pull's plan."""
+    pushed on the pull's plan.  exact: with tn_sparse_table_set_exact_verify the pull keeps a copy of the signs
+    as well and the push compares those."""
     from tensornet_amd import _lib
 
     D = 8
     rng = np.random.default_rng(55)
     pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=200000)
+    tn.core.set_sparse_table_exact_verify(pair.h, exact)
+    verify = "k_verify_values<true, true>" if exact else "k_verify_values<true, false>"
     vocab = 20000
     base = pair.populate(synth.splitmix64(np.arange(1, vocab + 1, dtype=np.uint64)))
     values = random_batch(rng, 3, 9000, vocab, ragged=False)  # 4.4 tiles of 2048 lookups a slot
@@ -570,7 +574,7 @@ def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, chang
         return names
 
     names = step(values, 0)
-    assert "k_verify_values<true, false>" in names and "k_remap_insert" not in names  # fingerprints, plan reused
+    assert verify in names and "k_remap_insert" not in names  # fingerprints (or the copy), plan reused
     edited = [v.copy() for v in values]
     v = edited[1]
     if change == "one sign":
@@ -589,7 +593,7 @@ def test_a_push_notices_any_change_of_the_signs_since_the_pull(tn, oracle, chang
     assert any((e != o).any() for e, o in zip(edited, values))
     names = step(edited, 1)
     assert "k_remap_insert" in names  # the push worked the batch out itself
-    assert "k_verify_values<true, false>" in step(values, 2)
+    assert verify in step(values, 2)
 
 
 def test_detached_updates_are_seen_by_whatever_touches_the_table_next(tn, oracle):
@@ -1042,6 +1046,54 @@ def test_calls_on_another_stream_wait_for_the_last_pull(tn, oracle):
             assert np.array_equal(gmapped2[s].cpu().numpy(), cmapped[s])
             np.testing.assert_allclose(gvars[s].cpu().numpy(), cvars[s], rtol=RTOL, atol=ATOL)
             np.testing.assert_allclose(gvars2[s].cpu().numpy(), cvars2[s], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.gpu
+def test_pull_on_another_stream_waits_for_the_updates_of_a_small_push(tn, oracle):
+    """The push of a small batch returns when its signs are compared, with its update kernel still running on
+    its stream.  A pull issued at once on ANOTHER stream reads the rows that kernel writes: it has to order
+    itself behind it (table-level and op-level pulls alike)."""
+    D = 16
+    rng = np.random.default_rng(79)
+    pair = Pair(tn, oracle, "AdaGrad", D, ADAGRAD_HP, reserve=400000, zero_init=True)
+    pool = synth.splitmix64(np.arange(1, 100001, dtype=np.uint64)).view(np.int64)
+    pair.populate(pool.view(np.uint64))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for step in range(4):
+        values = [pool[rng.integers(0, 100000, int(rng.integers(2000, 4000)))] for _ in range(24)]
+        rows = [len(v) + 1 for v in values]
+        cvars = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
+        rc, cmapped, counts = pair.o.pull_op(values, cvars)
+        assert rc == 0
+        grads = synth.make_grads(counts, D, 0.05, seed=step)
+        labels = [rng.integers(0, 2, len(v)).astype(np.int64) for v in values]
+        assert pair.o.push_op(values, grads, labels)[0] == 0
+        cvars2 = [np.full((r, pair.wf), -7.0, np.float32) for r in rows]
+        assert pair.o.pull_op(values, cvars2)[0] == 0
+        gvalues, ggrads, glabels = [dev(v) for v in values], [dev(g) for g in grads], [dev(l) for l in labels]
+        gvars = [torch.full((r, pair.wf), -7.0, device="cuda") for r in rows]
+        gvars2 = [torch.full((r, pair.wf), -7.0, device="cuda") for r in rows]
+        some = np.unique(np.concatenate(values))[:5000]
+        gsome = dev(some)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s2):
+            tn.ops.sparse_table_pull(gvars, gvalues, pair.h)
+            tn.ops.sparse_table_push(gvalues, ggrads, glabels, pair.h)
+        with torch.cuda.stream(s1):  # no synchronisation in between
+            if step % 2 == 0:
+                gmapped2 = tn.ops.sparse_table_pull(gvars2, gvalues, pair.h)
+            else:
+                table_rows = tn.ops.table_pull(pair.h, gsome, D)
+        torch.cuda.synchronize()
+        if step % 2 == 0:
+            for s in range(len(values)):
+                assert np.array_equal(gmapped2[s].cpu().numpy(), cmapped[s])
+                np.testing.assert_allclose(gvars2[s].cpu().numpy(), cvars2[s], rtol=RTOL, atol=ATOL)
+        else:
+            cw, _, cf = pair.o.get_rows(some.view(np.uint64))
+            assert cf.all()
+            np.testing.assert_allclose(table_rows.cpu().numpy(), cw[:, :D], rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.gpu

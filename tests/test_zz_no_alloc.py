@@ -47,8 +47,13 @@ def test_static_pull_matches_the_allocating_pull(tn):
         out_a = torch.full((n, dim), -3.0, device="cuda")
         out_b = torch.full((n, dim), -5.0, device="cuda")
         _lib.check(lib.tn_sparse_table_pull(ha, _ptr(signs), n, dim, _ptr(out_a), _stream()))
+        # the call allocates nothing: the device's free memory is the same before and after (hipMemGetInfo;
+        # the tensors above are allocated already, and torch's caching allocator is not called in between)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         _lib.check(lib.tn_sparse_table_pull_static(hb, _ptr(signs), n, dim, _ptr(out_b), _stream()))
         torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
         assert torch.equal(out_a.view(torch.int32), out_b.view(torch.int32))
         assert tn.core.sparse_table_key_count(ha) == tn.core.sparse_table_key_count(hb)
         # resident rows are the snapshot's, bit for bit
