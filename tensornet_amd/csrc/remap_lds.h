@@ -2,20 +2,21 @@
 // (core/kernels/sparse_table_ops.cc:119-131) for large batches.
 //
 // A global hash table costs one or two random 64-byte granules and up to two
-// device atomics per lookup.  Here the lookups of every slot are first
-// partitioned by a hash of the sign into buckets of 768 to 1536 lookups (an LDS
-// histogram and an LDS cursor per 2048-lookup tile: the only global atomics
-// are one per tile and bucket); then one workgroup per bucket builds the
-// bucket's hash table in LDS -- sign, smallest position, number of
-// occurrences -- and writes for every lookup the position of its sign's first
-// occurrence.  All lookups of one (slot, sign) land in one bucket, a bucket
-// belongs to one slot, and the positions it writes to lie inside that slot's
-// window of the concatenated lookup order, so the scatter back stays local.
+// device atomics per lookup.  Here every tile of 2048 consecutive lookups first
+// combines its own repeats in an LDS hash table and hands one record per
+// distinct sign to a bucket chosen by the slot and a hash of the sign (fixed
+// room per bucket; the only global atomics are one per tile and run of
+// records for a bucket); then one workgroup per bucket builds the bucket's
+// hash table in LDS -- sign, smallest position, number of occurrences -- and
+// writes for the first occurrence of every tile the position of the sign's
+// first occurrence in the slot.  All records of one (slot, sign) land in one
+// bucket, a bucket belongs to one slot, and the positions it writes to lie
+// inside that slot's window of the concatenated lookup order, so the scatter
+// back stays local.
 //
-//   k_lds_hist     bucket sizes (+ fingerprints of the signs for the plan)
-//   k_lds_offsets  exclusive scan of the bucket sizes (one workgroup)
-//   k_lds_scatter  {sign, position, slot} records grouped by bucket
-//   k_lds_dedup    per bucket: LDS hash table -> first_of[position], occurrence counts
+//   k_tile_dedup   per tile of 2048 lookups: LDS hash table -> first position of every sign inside the tile,
+//                  one record per distinct sign of the tile handed to its bucket (+ fingerprints of the signs)
+//   k_lds_dedup    per bucket: LDS hash table -> first position in the slot, occurrence counts
 //   k_lds_flags    first-occurrence flags per tile (coalesced: first_of[gi] == gi)
 //   k_lds_assign   ranks, distinct lists, show counts; the tiles' offsets come from a sum over the
 //                  counts of the tiles before (k_scan_tiles, shared with the global-table path,
@@ -41,14 +42,21 @@
 
 namespace tn {
 
-constexpr int LDS_TILE = 2048;          // lookups per tile of the partition kernels
-constexpr int LDS_TILE_ITEMS = LDS_TILE / 256;
-constexpr int LDS_SPAN = 4096;          // buckets one tile may touch
-constexpr int LDS_BUCKET_TARGET = 768;  // average lookups per bucket
+#ifndef TN_CURSOR_STRIDE
+#define TN_CURSOR_STRIDE 1
+#endif
+constexpr int CURSOR_STRIDE = TN_CURSOR_STRIDE;  // words from one first-level bucket's cursor to the next
+constexpr int LDS_TILE = 2048;          // lookups per tile of the partition kernel
+constexpr int TILE_THREADS = 512;
+constexpr int TILE_ITEMS = LDS_TILE / TILE_THREADS;
+constexpr int TILE_TABLE = 2 * LDS_TILE;  // entries of a tile's LDS hash table: two per lookup
+static_assert(LDS_TILE % TILE_THREADS == 0, "whole rounds");
+constexpr int L1_ROOM = 1536;           // room of a first-level bucket
 constexpr int LDS_MAX_SUB = 4096;       // buckets per slot at most
-constexpr int LDS_TABLE = 2048;         // entries of a bucket's LDS hash table
+constexpr int LDS_TABLE = 2048;         // entries of a bucket's LDS hash table (> L1_ROOM: an insert always ends)
 constexpr int DEDUP_THREADS = 512;      // a bucket's phases are short and separated by barriers: many wavefronts hide them
-constexpr int DEDUP_ITEMS = 4;          // lookups a thread of k_lds_dedup holds in registers
+constexpr int DEDUP_ITEMS = L1_ROOM / DEDUP_THREADS;  // records a thread of k_lds_dedup holds in registers
+static_assert(L1_ROOM % DEDUP_THREADS == 0 && L1_ROOM < LDS_TABLE, "a bucket fits its table and the registers of one workgroup");
 constexpr int LDS_SPAN2 = 512;          // second-level buckets whose counts one first-level bucket gathers in LDS
 constexpr int GRP_TARGET = 1024;        // records per second-level bucket if every lookup were distinct
 constexpr int GRP_CAP = 1536;           // room of a second-level bucket
@@ -60,7 +68,7 @@ constexpr int EMIT_THREADS = 512;
 constexpr int EMIT_RECS = GRP_CAP / EMIT_THREADS;  // records per thread of k_group_emit
 constexpr int GRP_ITEMS = (GRP_TABLE + 1 + GRP_THREADS - 1) / GRP_THREADS;
 constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
-static_assert((uint64_t)LDS_MAX_SUB * LDS_BUCKET_TARGET <= 0xFFFFFFull && GRP_SLOTS <= 256,
+static_assert((uint64_t)LDS_MAX_SUB * L1_ROOM <= 0xFFFFFFull && GRP_SLOTS <= 256,
               "a record's word holds the occurrences of a sign in its slot and the slot");
 
 // Raises DEV_ERR_REMAP_OVERFLOW.  A batch that overflows does so in a million places at once: atomics on the one
@@ -77,55 +85,17 @@ struct GroupRec {
 };
 constexpr uint32_t REC_CNT_MASK = 0xFFFFFFu;
 
+
+// [0, n) from a 32-bit hash without a division; grows with the hash
+__device__ __forceinline__ uint32_t scale32(uint32_t h, uint32_t n) { return __umulhi(h, n); }
+
+// First-level bucket of a slot, place in a tile's LDS table, second-level bucket, home slot in the table: all
+// grow with the one hash of the sign (the first two with its upper half).  The signs of a first-level bucket
+// therefore go to a few neighbouring second-level buckets, whose cursors its workgroup gathers in LDS, and the
+// signs of a second-level bucket lie in one stretch of the table, which keeps the probes of a workgroup within
+// few pages.
 __device__ __forceinline__ uint32_t group_bucket(uint64_t sign, uint32_t nb2) {
     return (uint32_t)__umul64hi(mix64(sign), (uint64_t)nb2);
-}
-
-// In this mode SlotDesc::tbase is the slot's first bucket and SlotDesc::tcap its number of buckets.
-__device__ __forceinline__ uint32_t bucket_of(const SlotDesc& d, uint64_t sign) {
-    return d.tbase + (uint32_t)__umul64hi(mix64(sign), (uint64_t)d.tcap);
-}
-
-// One pass over a tile: calls f(gi, slot, descriptor, sign) for each of its
-// lookups.  A tile usually lies inside one slot: then the slot is looked up
-// once, its descriptor sits in registers and the loads of the signs do not
-// depend on anything.
-template <typename F>
-__device__ __forceinline__ void for_tile(uint32_t tile, const SlotDesc* descs, const uint32_t* lb, int N, uint32_t L,
-                                         F f) {
-    const uint32_t g0 = tile * LDS_TILE;
-    const uint32_t g1 = min(L, g0 + (uint32_t)LDS_TILE) - 1;
-    const int s0 = find_slot(lb, N, g0);
-    if (g1 < lb[s0 + 1]) {
-        const SlotDesc d = descs[s0];
-        const uint32_t base = lb[s0];
-#pragma unroll
-        for (int j = 0; j < LDS_TILE_ITEMS; j++) {
-            const uint32_t gi = g0 + j * 256 + threadIdx.x;
-            if (gi <= g1) f(gi, s0, d, (uint64_t)d.values[gi - base]);
-        }
-    } else {
-#pragma unroll 4
-        for (int j = 0; j < LDS_TILE_ITEMS; j++) {
-            const uint32_t gi = g0 + j * 256 + threadIdx.x;
-            if (gi > g1) break;
-            const int sl = find_slot(lb, N, gi);
-            f(gi, sl, descs[sl], (uint64_t)descs[sl].values[gi - lb[sl]]);
-        }
-    }
-}
-
-// Buckets a tile can touch: from the first bucket of its first slot (b0) up to the
-// last bucket of its last slot, span_cap at most (the host sizes the LDS histogram for the
-// widest tile of the call, LDS_SPAN at most).
-__device__ __forceinline__ uint32_t tile_span(uint32_t tile, const SlotDesc* descs, const uint32_t* lb, int N,
-                                              uint32_t L, uint32_t span_cap, uint32_t& b0) {
-    const uint32_t g0 = tile * LDS_TILE;
-    const uint32_t g1 = min(L, g0 + (uint32_t)LDS_TILE) - 1;
-    const SlotDesc& first = descs[find_slot(lb, N, g0)];
-    const SlotDesc& last = descs[find_slot(lb, N, g1)];
-    b0 = first.tbase;
-    return min(span_cap, last.tbase + last.tcap - b0);
 }
 
 __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
@@ -133,114 +103,220 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
 }
 
-// Also presets first_of to "every lookup is its own first occurrence", which is
-// what a lookup keeps if an overflow leaves it unprocessed (its count is then
-// meaningless, but every index stays in bounds until the host repeats the call),
-// and leaves the fingerprints of the batch's signs, which a push compares its own with
-// (k_verify_values): one per wavefront of a tile, the same tiles in both kernels.
-static_assert(LDS_TILE == VERIFY_TILE, "k_lds_hist and k_verify_values fingerprint the same runs of lookups");
-__global__ __launch_bounds__(256) void k_lds_hist(const SlotDesc* __restrict__ descs, const uint32_t* __restrict__ lbase,
-                                                  int N, uint32_t L, uint32_t* bcount,
-                                                  ulonglong2* __restrict__ prints, uint64_t* __restrict__ exact,
-                                                  uint32_t* __restrict__ first_of, DevStatus* status,
-                                                  uint32_t span_cap) {
-    extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]
-    uint32_t* lb = smem;
-    uint32_t* hist = smem + N + 1;
-    load_lbase(lb, lbase, N);
-    const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
-    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        uint32_t b0;  // lowest bucket the tile can touch
-        const uint32_t span = tile_span(tile, descs, lb, N, L, span_cap, b0);
-        for (uint32_t i = threadIdx.x; i < span; i += 256) hist[i] = 0;
-        __syncthreads();
-        Fingerprint print;
-        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int, const SlotDesc& d, uint64_t sign) {
-            print.add(gi, sign);
-            if (exact) exact[gi] = sign;  // a push is to compare the signs themselves
-            first_of[gi] = gi;
-            const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < span)
-                atomicAdd(&hist[local], 1u);
-            else
-                flag_overflow(status);
-        });
-        print.wave_sum();
-        if ((threadIdx.x & 63) == 0) prints[tile * (256 / 64) + (threadIdx.x >> 6)] = make_ulonglong2(print.a, print.b);
-        __syncthreads();
-        for (uint32_t i = threadIdx.x; i < span; i += 256)
-            if (hist[i]) atomicAdd(&bcount[b0 + i], hist[i]);
-        __syncthreads();
+// What a tile hands to a first-level bucket: one record per distinct sign of the tile (per slot, where a tile
+// spans several).  y: bits 0-31 the position of the sign's first occurrence in the tile, 32-43 its occurrences in
+// the tile (1 .. LDS_TILE), 44-55 the slot.
+__device__ __forceinline__ ulonglong2 tile_record(uint64_t sign, uint32_t gi, uint32_t cnt, uint32_t slot) {
+    return make_ulonglong2(sign, (uint64_t)gi | ((uint64_t)cnt << 32) | ((uint64_t)slot << 44));
+}
+static_assert(LDS_TILE < (1 << 12) && MAX_SLOTS < (1 << 12), "a tile record's fields");
+
+// The first pass over the lookups.  A tile of LDS_TILE consecutive lookups first combines its own repeats in an
+// LDS hash table -- every lookup learns the first position of its sign inside the tile (first_of, written in
+// order) -- and hands ONE record per distinct sign on to the sign's first-level bucket: sign, first position in
+// the tile, occurrences in the tile.  However often a sign occurs in a slot, it puts at most one record per tile
+// into its bucket, so buckets of fixed room do (bcursor[b] = records handed to bucket b, the records at
+// prec[b * L1_ROOM ...]); no histogram of the lookups and no scan of bucket sizes is needed, and the passes that
+// follow work on the tiles' distinct signs instead of on the lookups.
+//
+// The table has two entries per lookup of the tile.  The lookups of a slot own the entries [2 a, 2 b) if they sit
+// at the tile's positions [a, b): tiles that span slots (any number of them) keep the slots apart without a pass
+// per slot.  The last entry of a slot's range belongs to the sign that equals EMPTY_KEY; the others are filled by
+// linear probing.  The lookup that turns out to be its sign's first in the tile hands the record on: it holds the
+// sign and its hash in registers already, so the table is never walked (most of its entries are free, and a walk
+// pays for every one of them).  Places in the buckets: an LDS counter per bucket the tile can touch gives a
+// record its place among the tile's records for the bucket, one global atomic per touched bucket reserves the
+// tile's slice of it.
+//
+// It also leaves the fingerprints of the batch's signs, which a push compares its own with (k_verify_values: one
+// per 64 strided lookups of a tile of 256 x 8, which are the lookups of the wavefronts w and w + 4 here), and,
+// with exact != nullptr, a copy of the signs.
+static_assert(LDS_TILE == VERIFY_TILE && TILE_THREADS == 512, "k_tile_dedup and k_verify_values fingerprint the same runs of lookups");
+constexpr int TILE_LDS_SLOTS = 128;  // up to this many slots their value pointers and bucket ranges sit in LDS
+constexpr int LDS_SPAN = 4096;       // first-level buckets one tile may touch (its LDS counters)
+// dynamic LDS of k_tile_dedup: lb[N + 1], then (few slots) the slots' value pointers and bucket ranges, then a
+// counter per bucket the widest tile touches
+inline size_t tile_dedup_lds(int N, uint32_t span_cap) {
+    const size_t lb = align_up(((size_t)N + 1) * sizeof(uint32_t), 8);
+    return (N <= TILE_LDS_SLOTS ? lb + (size_t)N * (sizeof(uint64_t) + sizeof(uint2)) : lb) + (size_t)span_cap * sizeof(uint32_t);
+}
+__global__ __launch_bounds__(TILE_THREADS) __attribute__((amdgpu_waves_per_eu(6, 8))) void k_tile_dedup(const SlotDesc* __restrict__ descs,
+                                                             const uint32_t* __restrict__ lbase, int N, uint32_t L,
+                                                             uint32_t* bcursor, ulonglong2* __restrict__ prec,
+                                                             ulonglong2* __restrict__ prints,
+                                                             uint64_t* __restrict__ exact,
+                                                             uint32_t* __restrict__ first_of, DevStatus* status,
+                                                             uint32_t span_cap) {
+    extern __shared__ uint32_t lb[];  // lb[N + 1], sized by the launch; then vals[N], tb[N], hist[span_cap] (see tile_dedup_lds)
+    __shared__ unsigned long long keys[TILE_TABLE];
+    __shared__ uint32_t word[TILE_TABLE];  // bits 16-31 smallest position in the tile, 0-15 occurrences
+    __shared__ ulonglong2 fp[TILE_THREADS / 64];
+    // With few slots everything a tile needs of its slots' descriptors comes in with the slots' first lookups, in
+    // one round trip, instead of in a second one once the tile knows its slot.
+    const bool lds_descs = N <= TILE_LDS_SLOTS;
+    const int64_t** vals = reinterpret_cast<const int64_t**>(lb + ((N + 2) & ~1));
+    uint2* tb = reinterpret_cast<uint2*>(vals + N);
+    uint32_t* hist = lds_descs ? reinterpret_cast<uint32_t*>(tb + N) : lb + ((N + 2) & ~1);
+    for (int i = threadIdx.x; i <= N; i += TILE_THREADS) {
+        lb[i] = lbase[i];
+        if (lds_descs && i < N) {
+            vals[i] = descs[i].values;
+            tb[i] = make_uint2(descs[i].tbase, descs[i].tcap);
+        }
     }
-}
-
-// bstart[b] = number of lookups in buckets before b; bcursor starts as a copy.
-__global__ __launch_bounds__(1024) void k_lds_offsets(const uint32_t* __restrict__ bcount, uint32_t* __restrict__ bstart,
-                                                      uint32_t* __restrict__ bcursor, uint32_t nbuckets) {
-    __shared__ uint32_t wsum[16];
-    __shared__ uint32_t carry_sh;
-    const uint32_t total = scan_u32_1024(bcount, nbuckets, wsum, &carry_sh, [&](uint32_t i, uint32_t v) {
-        bstart[i] = v;
-        bcursor[i] = v;
-    });
-    if (threadIdx.x == 0) bstart[nbuckets] = total;
-}
-
-__global__ __launch_bounds__(256) void k_lds_scatter(const SlotDesc* __restrict__ descs,
-                                                     const uint32_t* __restrict__ lbase, int N, uint32_t L,
-                                                     uint32_t* bcursor, ulonglong2* __restrict__ prec,
-                                                     uint32_t span_cap) {
-    extern __shared__ uint32_t smem[];  // lb[N + 1], hist[span_cap]: first the tile's count per bucket, then its write cursor
-    uint32_t* lb = smem;
-    uint32_t* hist = smem + N + 1;
-    load_lbase(lb, lbase, N);
+    __syncthreads();
+    auto slot_values = [&](int sl) { return lds_descs ? vals[sl] : descs[sl].values; };
+    auto slot_buckets = [&](int sl) { return lds_descs ? tb[sl] : make_uint2(descs[sl].tbase, descs[sl].tcap); };
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t ntiles = (L + LDS_TILE - 1) / LDS_TILE;
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        uint32_t b0;
-        const uint32_t span = tile_span(tile, descs, lb, N, L, span_cap, b0);
-        for (uint32_t i = threadIdx.x; i < span; i += 256) hist[i] = 0;
+        const uint32_t g0 = tile * LDS_TILE;
+        const uint32_t g1 = min(L, g0 + (uint32_t)LDS_TILE) - 1;
+        const uint32_t n_tile = g1 - g0 + 1;
+        const int s0 = find_slot(lb, N, g0);
+        const bool one_slot = g1 < lb[s0 + 1];  // the usual case: the slot's values and buckets sit in registers
+        const int64_t* v0 = slot_values(s0) - lb[s0];
+        uint64_t sg[TILE_ITEMS];
+        int sl[TILE_ITEMS];
+#pragma unroll
+        for (int j = 0; j < TILE_ITEMS; j++) {
+            const uint32_t gi = g0 + j * TILE_THREADS + threadIdx.x;
+            sg[j] = 0;
+            sl[j] = s0;
+            if (gi <= g1) {
+                if (one_slot) {
+                    sg[j] = (uint64_t)v0[gi];
+                } else {
+                    sl[j] = find_slot(lb, N, gi);
+                    sg[j] = (uint64_t)slot_values(sl[j])[gi - lb[sl[j]]];
+                }
+            }
+        }
+        // buckets the tile can touch: from the first bucket of its first slot to the last bucket of its last slot
+        // (span_cap at most: the host sizes the counters for the widest tile of the call, LDS_SPAN at most)
+        const uint2 b0 = slot_buckets(s0);
+        uint32_t span = b0.y;
+        if (!one_slot) {
+            const uint2 bl = slot_buckets(find_slot(lb, N, g1));
+            span = bl.x + bl.y - b0.x;
+        }
+        span = min(span, span_cap);
+        for (int i = threadIdx.x; i < TILE_TABLE; i += TILE_THREADS) {
+            keys[i] = EMPTY_KEY;
+            word[i] = 0xFFFF0000u;
+        }
+        for (uint32_t i = threadIdx.x; i < span; i += TILE_THREADS) hist[i] = 0;
+        // the hash of every sign once: fingerprint, place in the table, bucket
+        uint32_t hs[TILE_ITEMS];
+        {
+            Fingerprint print;
+#pragma unroll
+            for (int j = 0; j < TILE_ITEMS; j++) {
+                const uint32_t gi = g0 + j * TILE_THREADS + threadIdx.x;
+                const uint64_t m = mix64(sg[j]);
+                hs[j] = (uint32_t)(m >> 32);
+                if (gi <= g1) {
+                    print.add_mixed(gi, m);
+                    if (exact) exact[gi] = sg[j];  // a push is to compare the signs themselves
+                }
+            }
+            print.wave_sum();
+            if (lane == 0) fp[wave] = make_ulonglong2(print.a, print.b);
+        }
         __syncthreads();
-        for_tile(tile, descs, lb, N, L, [&](uint32_t, int, const SlotDesc& d, uint64_t sign) {
-            const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < span) atomicAdd(&hist[local], 1u);
-        });
+        if (threadIdx.x < 4)
+            prints[tile * 4 + threadIdx.x] = make_ulonglong2(fp[threadIdx.x].x + fp[threadIdx.x + 4].x,
+                                                             fp[threadIdx.x].y + fp[threadIdx.x + 4].y);
+        // every lookup finds or claims the entry of its sign and lowers the entry's position to its own
+        uint32_t ent[TILE_ITEMS];
+#pragma unroll
+        for (int j = 0; j < TILE_ITEMS; j++) {
+            const uint32_t pos = j * TILE_THREADS + threadIdx.x;
+            ent[j] = 0;
+            if (pos >= n_tile) continue;
+            uint32_t a = 0, m = n_tile;  // the slot's lookups sit at the tile's positions [a, a + m)
+            if (!one_slot) {
+                a = max(lb[sl[j]], g0) - g0;
+                m = min(lb[sl[j] + 1], g1 + 1) - g0 - a;
+            }
+            const uint32_t lo = 2 * a, size = 2 * m - 1;
+            uint32_t e = lo + size;  // the entry of the sign EMPTY_KEY
+            if (sg[j] != EMPTY_KEY) {
+                e = lo + scale32(hs[j], size);
+                for (;;) {  // at most m distinct signs in 2 m - 1 entries: a free one exists
+                    const unsigned long long old = atomicCAS(&keys[e], (unsigned long long)EMPTY_KEY, sg[j]);
+                    if (old == EMPTY_KEY || old == sg[j]) break;
+                    e = (e + 1 == lo + size) ? lo : e + 1;
+                }
+            }
+            atomicMin(&word[e], pos << 16);
+            ent[j] = e;
+        }
+        __syncthreads();
+        // ... counts itself there and reads the sign's first position in the tile; the lookup at that position
+        // takes a place among the tile's records for its bucket
+        uint32_t place[TILE_ITEMS];  // 0xFFFFFFFF: not a first occurrence (or no lookup)
+        uint32_t bloc[TILE_ITEMS];   // the bucket, counted from the tile's first
+#pragma unroll
+        for (int j = 0; j < TILE_ITEMS; j++) {
+            const uint32_t pos = j * TILE_THREADS + threadIdx.x;
+            place[j] = 0xFFFFFFFFu;
+            bloc[j] = 0;
+            if (pos >= n_tile) continue;
+            const uint32_t old = atomicAdd(&word[ent[j]], 1u);
+            const uint32_t f = old >> 16;
+            first_of[g0 + pos] = g0 + f;
+            if (f == pos) {
+                const uint2 bb = one_slot ? b0 : slot_buckets(sl[j]);
+                bloc[j] = bb.x + scale32(hs[j], bb.y) - b0.x;
+                if (bloc[j] < span)
+                    place[j] = atomicAdd(&hist[bloc[j]], 1u);
+                else
+                    flag_overflow(status);  // (more buckets under one tile than it has counters for)
+            }
+        }
         __syncthreads();
         // the tile's slice of every bucket it touches; all atomics of a thread are in flight together
-        for (uint32_t i0 = 0; i0 < span; i0 += 256 * 4) {
+        for (uint32_t i0 = 0; i0 < span; i0 += TILE_THREADS * 4) {
             uint32_t got[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const uint32_t i = i0 + q * 256 + threadIdx.x;
+                const uint32_t i = i0 + q * TILE_THREADS + threadIdx.x;
                 const uint32_t cnt = i < span ? hist[i] : 0;
-                got[q] = cnt ? atomicAdd(&bcursor[b0 + i], cnt) : 0;
+                got[q] = cnt ? atomicAdd(&bcursor[(size_t)(b0.x + i) * CURSOR_STRIDE], cnt) : 0;
             }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const uint32_t i = i0 + q * 256 + threadIdx.x;
+                const uint32_t i = i0 + q * TILE_THREADS + threadIdx.x;
                 if (i < span) hist[i] = got[q];
             }
         }
         __syncthreads();
-        for_tile(tile, descs, lb, N, L, [&](uint32_t gi, int sl, const SlotDesc& d, uint64_t sign) {
-            const uint32_t local = bucket_of(d, sign) - b0;
-            if (local < span) {
-                const uint32_t at = atomicAdd(&hist[local], 1u);
-                // one 16-byte store per lookup (these stores are what the pass costs): sign, position, slot
-                prec[at] = make_ulonglong2(sign, (uint64_t)gi | ((uint64_t)(uint32_t)sl << 32));
-            }
-        });
+#pragma unroll
+        for (int j = 0; j < TILE_ITEMS; j++) {
+            if (place[j] == 0xFFFFFFFFu) continue;
+            const uint32_t pos = j * TILE_THREADS + threadIdx.x;
+            const uint32_t at = hist[bloc[j]] + place[j];
+            if (at < (uint32_t)L1_ROOM)
+                prec[(size_t)(b0.x + bloc[j]) * L1_ROOM + at] =
+                    tile_record(sg[j], g0 + pos, word[ent[j]] & 0xFFFFu, (uint32_t)sl[j]);
+            else
+                flag_overflow(status);
+        }
         __syncthreads();
     }
 }
 
 __device__ __forceinline__ uint32_t lds_slot(uint64_t sign) { return (uint32_t)(mix64(sign) >> 7) & (LDS_TABLE - 1); }
 
-// One workgroup per bucket.  first_of[gi] = position of the first occurrence
-// of gi's sign in its slot; cnt_at[first position] = occurrences of the sign.
-// With EMIT every distinct sign of the bucket is also appended to its
-// second-level bucket (recs[c * GRP_CAP ...], cursor2[c] = records handed in).
+// One workgroup per first-level bucket: the records its tiles handed in, one per distinct sign of a tile, are
+// combined in an LDS hash table -- sign, smallest position, occurrences.  first_of[position of a tile's first
+// occurrence] = position of the sign's first occurrence in its slot (k_tile_dedup left the tile's own there, and
+// left every other lookup pointing at its tile's: two hops from any lookup); cnt_at[first position] =
+// occurrences of the sign.  With EMIT every distinct sign of the bucket is also appended to its second-level
+// bucket (recs[c * GRP_CAP ...], cursor2[c] = records handed in).
 template <bool EMIT>
-__global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __restrict__ bstart, uint32_t nbuckets,
+__global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __restrict__ bcursor, uint32_t nbuckets,
                                                    const ulonglong2* __restrict__ prec,
                                                    uint32_t* __restrict__ first_of, uint32_t* __restrict__ cnt_at,
                                                    DevStatus* status, uint32_t nb2, uint32_t* cursor2,
@@ -254,26 +330,22 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
     // positions): on one die they meet in one L2 and leave it as whole lines.
     const DieShare share(nbuckets);
     for (uint32_t b = share.first; b < share.end; b += share.step) {
-        const uint32_t lo = bstart[b], hi = bstart[b + 1];
-        if (lo == hi) continue;
-        // The bucket's lookups are taken DEDUP_ITEMS per thread at a time, all loads of a round
-        // issued together; a bucket that fits one round (the usual case) is read once.  The first
-        // round's loads are in flight while the tables are cleared.
+        const uint32_t n = min(bcursor[(size_t)b * CURSOR_STRIDE], (uint32_t)L1_ROOM);
+        if (n == 0) continue;
+        const size_t first = (size_t)b * L1_ROOM;
+        // The bucket's records sit in registers, all loads issued together and in flight while the tables
+        // are cleared.
         uint64_t sg[DEDUP_ITEMS];
-        uint32_t gp[DEDUP_ITEMS];
-        const uint32_t round = DEDUP_THREADS * DEDUP_ITEMS;
-        const bool one_round = hi - lo <= round;
-        auto load_round = [&](uint32_t base) {
+        uint32_t gp[DEDUP_ITEMS], mu[DEDUP_ITEMS];
 #pragma unroll
-            for (int j = 0; j < DEDUP_ITEMS; j++) {
-                const uint32_t i = base + j * DEDUP_THREADS + threadIdx.x;
-                const ulonglong2 r = (i < hi) ? prec[i] : make_ulonglong2(0, 0xFFFFFFFFull);  // no position: nothing to do
-                sg[j] = r.x;
-                gp[j] = (uint32_t)r.y;
-                if (EMIT && j == 0 && i == lo) slot_sh = (uint32_t)(r.y >> 32);  // every lookup of a bucket is of one slot
-            }
-        };
-        load_round(lo);
+        for (int j = 0; j < DEDUP_ITEMS; j++) {
+            const uint32_t i = j * DEDUP_THREADS + threadIdx.x;
+            const ulonglong2 r = (i < n) ? prec[first + i] : make_ulonglong2(0, 0xFFFFFFFFull);  // no position: nothing to do
+            sg[j] = r.x;
+            gp[j] = (uint32_t)r.y;
+            mu[j] = (uint32_t)(r.y >> 32) & 0xFFFu;
+            if (EMIT && i == 0) slot_sh = (uint32_t)(r.y >> 44);  // every record of a bucket is of one slot
+        }
         for (int i = threadIdx.x; i <= LDS_TABLE; i += DEDUP_THREADS) {
             keys[i] = EMPTY_KEY;
             minpos[i] = 0xFFFFFFFFu;
@@ -285,54 +357,27 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
         }
         __syncthreads();
         uint32_t c_min = 0xFFFFFFFFu;
-        for (uint32_t base = lo; base < hi; base += round) {
-            if (base != lo) load_round(base);
+        uint32_t hs[DEDUP_ITEMS];
 #pragma unroll
-            for (int j = 0; j < DEDUP_ITEMS; j++) {
-                const uint64_t sign = sg[j];
-                uint32_t gi = gp[j];
-                uint32_t mult = 1;
-                bool valid = gi != 0xFFFFFFFFu;
-                // A frequent sign fills whole wavefronts: the lanes that hold the same sign as the
-                // first valid lane hand their smallest position and their number to that lane,
-                // instead of queueing up on one LDS address.
-                const unsigned long long vmask = __ballot(valid);
-                if (vmask == 0) continue;
-                const int leader = __ffsll((long long)vmask) - 1;
-                const uint64_t lead_sign = ((uint64_t)(uint32_t)__shfl((int)(sign >> 32), leader) << 32) |
-                                           (uint32_t)__shfl((int)(uint32_t)sign, leader);
-                const bool same = valid && sign == lead_sign;
-                const unsigned long long smask = __ballot(same);
-                if (__popcll(smask) >= 8) {
-                    uint32_t m = same ? gi : 0xFFFFFFFFu;
-                    for (int o = 32; o > 0; o >>= 1) m = min(m, (uint32_t)__shfl_xor((int)m, o));
-                    if ((int)(threadIdx.x & 63) == leader) {
-                        gi = m;
-                        mult = (uint32_t)__popcll(smask);
-                    } else if (same) {
-                        valid = false;
-                    }
+        for (int j = 0; j < DEDUP_ITEMS; j++) {
+            const uint64_t sign = sg[j];
+            const uint32_t gi = gp[j];
+            hs[j] = LDS_TABLE;
+            if (gi == 0xFFFFFFFFu) continue;
+            if (EMIT) c_min = min(c_min, group_bucket(sign, nb2));
+            uint32_t h = LDS_TABLE;
+            if (sign != EMPTY_KEY) {
+                h = lds_slot(sign);
+                for (;;) {  // at most L1_ROOM < LDS_TABLE distinct signs: a free entry exists
+                    unsigned long long old = keys[h];
+                    if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
+                    if (old == EMPTY_KEY || old == sign) break;
+                    h = (h + 1) & (LDS_TABLE - 1);
                 }
-                if (!valid) continue;
-                if (EMIT) c_min = min(c_min, group_bucket(sign, nb2));
-                uint32_t h = LDS_TABLE;
-                if (sign != EMPTY_KEY) {
-                    h = lds_slot(sign);
-                    int tries = 0;
-                    for (; tries < LDS_TABLE; tries++) {
-                        unsigned long long old = keys[h];
-                        if (old == EMPTY_KEY) old = atomicCAS(&keys[h], (unsigned long long)EMPTY_KEY, sign);
-                        if (old == EMPTY_KEY || old == sign) break;
-                        h = (h + 1) & (LDS_TABLE - 1);
-                    }
-                    if (tries == LDS_TABLE) {  // table full: keep indices in bounds, let the host fall back
-                        flag_overflow(status);
-                        continue;
-                    }
-                }
-                atomicMin(&minpos[h], gi);
-                atomicAdd(&cnts[h], mult);
             }
+            atomicMin(&minpos[h], gi);
+            atomicAdd(&cnts[h], mu[j]);
+            hs[j] = h;
         }
         if (EMIT) {
             for (int o = 32; o > 0; o >>= 1) c_min = min(c_min, (uint32_t)__shfl_xor((int)c_min, o));
@@ -340,29 +385,19 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
         }
         __syncthreads();
         const uint32_t c_lo = EMIT ? c_lo_sh : 0;
-        for (uint32_t base = lo; base < hi; base += round) {
-            if (!one_round) load_round(base);
 #pragma unroll
-            for (int j = 0; j < DEDUP_ITEMS; j++) {
-                const uint64_t sign = sg[j];
-                const uint32_t gi = gp[j];
-                if (gi == 0xFFFFFFFFu) continue;
-                uint32_t h = LDS_TABLE;
-                bool found = true;
-                if (sign != EMPTY_KEY) {
-                    h = lds_slot(sign);
-                    int tries = 0;
-                    for (; tries < LDS_TABLE && keys[h] != sign; tries++) h = (h + 1) & (LDS_TABLE - 1);
-                    found = tries < LDS_TABLE;
-                }
-                const uint32_t f = found ? minpos[h] : gi;
-                if (f != gi) first_of[gi] = f;  // k_lds_hist preset first_of[gi] = gi
-                if (f == gi) {
-                    if (!EMIT) cnt_at[gi] = found ? cnts[h] : 1u;  // with EMIT the record carries the count
-                    if (EMIT && found) {  // one lookup per occupied entry gets here
-                        const uint32_t local = group_bucket(sign, nb2) - c_lo;
-                        if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
-                    }
+        for (int j = 0; j < DEDUP_ITEMS; j++) {
+            const uint32_t gi = gp[j];
+            if (gi == 0xFFFFFFFFu) continue;
+            const uint32_t h = hs[j];
+            const uint32_t f = minpos[h];
+            if (f != gi) {
+                first_of[gi] = f;  // k_tile_dedup left first_of[gi] = gi
+            } else {
+                if (!EMIT) cnt_at[gi] = cnts[h];  // with EMIT the record carries the count
+                if (EMIT) {  // one record per occupied entry gets here
+                    const uint32_t local = group_bucket(sg[j], nb2) - c_lo;
+                    if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
                 }
             }
         }
@@ -401,11 +436,29 @@ __device__ __forceinline__ uint32_t rank_of(const uint8_t* __restrict__ flag8, c
     return wordpre[gi >> 6] + (uint32_t)__popcll(word & ((1ull << (gi & 63)) - 1ull));
 }
 
-// Tile counts of first occurrences; a lookup is one iff first_of[gi] == gi.
+// Tile counts of first occurrences; a lookup is one iff first_of[gi] == gi.  The first workgroups also add up
+// what the first-level buckets of every slot were handed: status->tile_share_q16 = the largest share
+// records / lookups among the slots with more than one bucket's worth of lookups, in 1 / 65536 (the host sizes
+// the next call's buckets from it).
 __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const uint32_t* __restrict__ first_of,
                                                              uint8_t* __restrict__ flag8,
-                                                             uint32_t* __restrict__ tilesum) {
+                                                             uint32_t* __restrict__ tilesum,
+                                                             const SlotDesc* __restrict__ descs, int N,
+                                                             const uint32_t* __restrict__ bcursor,
+                                                             DevStatus* status) {
     __shared__ uint32_t red[4];
+    for (int sl = blockIdx.x; sl < N; sl += gridDim.x) {
+        const SlotDesc& d = descs[sl];
+        if (d.len <= (uint32_t)L1_ROOM) continue;  // (the same for the whole workgroup)
+        uint32_t mine = 0;
+        for (uint32_t b = threadIdx.x; b < d.tcap; b += REMAP_THREADS) mine += bcursor[(size_t)(d.tbase + b) * CURSOR_STRIDE];
+        const uint32_t all = block_sum_256(mine, red);
+        if (threadIdx.x == 0) {
+            const uint64_t q = ((uint64_t)all << 16) / d.len + 1;
+            atomicMax(&status->tile_share_q16, (uint32_t)(q < 65536 ? q : 65536));
+        }
+        __syncthreads();
+    }
     const uint32_t base = blockIdx.x * REMAP_TILE + threadIdx.x * REMAP_ITEMS;
     uint32_t bits = 0;
     static_assert(REMAP_ITEMS == 8, "a thread's lookups are two 16-byte loads");
@@ -532,6 +585,11 @@ __global__ __launch_bounds__(256) void k_lds_mapped(const SlotDesc* __restrict__
 #pragma unroll
             for (int j = 0; j < 4; j++) f[j] = g0 + j < L ? first_of[g0 + j] : 0u;
         }
+        // A lookup points at the first occurrence inside its tile, which points at the first one in the slot
+        // (itself, if it is that): the second hop stays inside the lookup's own tile for a repeat within a
+        // tile, and is the identity for a first occurrence.
+#pragma unroll
+        for (int j = 0; j < 4; j++) f[j] = first_of[f[j]];
 #pragma unroll
         for (int j = 0; j < 4; j++) u[j] = rank_of(flag8, wordpre, f[j]);
         if (g0 + 4 <= L) {

@@ -126,6 +126,7 @@ __global__ void k_reset_status(DevStatus* status, uint32_t n_unique, uint32_t gc
         status->mismatch = 0;
         status->abort = 0;
         status->n_big = 0;
+        status->tile_share_q16 = 0;
     }
 }
 
@@ -166,6 +167,7 @@ __global__ __launch_bounds__(256) void k_stage_in(const uint32_t* __restrict__ h
             status->gcap = 0;
             status->n_members = 0;
             status->n_big = 0;
+            status->tile_share_q16 = 0;
         }
     }
 }
@@ -1282,8 +1284,9 @@ __global__ __launch_bounds__(256) void k_member_grads(PushSrc src, const DevStat
 // check: every push analyses its batch from scratch, sparse_table_ops.cc:274-297.)
 struct Fingerprint {
     uint64_t a = 0, b = 0;
-    __device__ __forceinline__ void add(uint32_t gi, uint64_t sign) {
-        const uint64_t m = mix64(sign);
+    __device__ __forceinline__ void add(uint32_t gi, uint64_t sign) { add_mixed(gi, mix64(sign)); }
+    // m = mix64(sign), for a caller that has it already
+    __device__ __forceinline__ void add_mixed(uint32_t gi, uint64_t m) {
         const uint32_t w = (gi * 0x9E3779B1u) | 1u;
         a += m * w;
         b += ((m << 32) | (m >> 32)) * w;

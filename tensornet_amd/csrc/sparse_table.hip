@@ -35,6 +35,10 @@ constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 
 constexpr size_t ONE_STREAM_LOOKUPS = 3u << 20;
 constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to which no scan kernel runs between its launches
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
+#ifndef TN_TILE_GRID
+#define TN_TILE_GRID (256 * 3)
+#endif
+constexpr int TILE_GRID = TN_TILE_GRID;                 // workgroups of k_tile_dedup
 constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS wins: it also takes fewer launches (cfg1, 8 k lookups: 0.154 -> 0.136 ms)
 
 // Up to this many lookups a batch whose slots each fit one workgroup (SMALL_SLOT_MAX lookups, SMALL_SLOTS slots)
@@ -144,6 +148,10 @@ struct SparseTable {
     // sizes the number of second-level buckets, whose room is fixed.  A batch with more distinct
     // records than expected overflows a bucket and takes the fallback path once; the estimate is then reset.
     double distinct_est = 1.0;
+    // Records a tile of the remap through LDS hands to the first-level buckets per lookup (1 = no sign repeats
+    // inside a tile, the safe start), for the slot where that share is largest: sizes the first-level buckets,
+    // whose room is fixed, with the same fallback as above.
+    double tile_est = 1.0;
     uint64_t pull_lookups = 0;  // lookups of the pull whose status is pending
     bool stage_pending = false;
     bool push_pending = false;      // hpush holds an unchecked status
@@ -400,6 +408,10 @@ void harvest(SparseTable* t) {
         if (t->pull_lookups > 0) {  // rises at once, falls within about ten pulls
             const double now = (double)h.ubase[N] / (double)t->pull_lookups;
             t->distinct_est = std::min(1.0, std::max(now, 0.75 * t->distinct_est + 0.25 * now));
+            if (h.st.tile_share_q16 != 0) {  // (a pull through LDS with a slot of more than one bucket)
+                const double share = (double)h.st.tile_share_q16 / 65536.0;
+                t->tile_est = std::min(1.0, std::max(share, 0.75 * t->tile_est + 0.25 * share));
+            }
         }
         latch(t, dev_err_code(h.st.err), std::string("sparse pull: ") + dev_err_text(h.st.err));
         for (int s = 0; s < N && s < (int)t->pending_rows.size(); s++)
@@ -531,11 +543,9 @@ struct Scratch {
     uint32_t ntiles;
     // LDS remap
     uint32_t nbuckets;
-    uint32_t span_cap;  // buckets the widest tile touches (entries of the partition kernels' LDS histogram)
-    uint32_t* bcount;
-    uint32_t* bstart;
-    uint32_t* bcursor;
-    ulonglong2* prec;    // lookups by bucket: {sign, position}
+    uint32_t span_cap;   // first-level buckets the widest tile touches (LDS counters of k_tile_dedup)
+    uint32_t* bcursor;   // per first-level bucket: records handed in
+    ulonglong2* prec;    // the tiles' records by bucket, L1_ROOM each: {sign, position | occurrences | slot}
     uint32_t* first_of;
     uint32_t* cnt_at;
     uint32_t* wordpre;  // first occurrences before every 64-lookup word
@@ -605,7 +615,17 @@ uint32_t second_level_buckets(size_t L, double distinct_est) {
 }
 
 // dt_entries: entries of the global dedup table, or (use_lds) the number of buckets.
-size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds, double distinct_est = 1.0) {
+// First-level buckets of a slot of `len` lookups whose tiles hand on `share` records per lookup: L1_FILL records
+// each on average (L1_ROOM is the room of a bucket); a slot that fits one bucket whatever its signs has one.
+constexpr size_t L1_FILL = 1150;
+constexpr double L1_MARGIN = 1.15;
+size_t first_level_buckets(size_t len, double share) {
+    if (len <= (size_t)L1_ROOM) return 1;
+    return ((size_t)((double)len * std::min(1.0, share * L1_MARGIN)) + L1_FILL - 1) / L1_FILL;
+}
+
+size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool use_lds, double distinct_est = 1.0,
+                     int N = 0) {
     Carver c{base};
     if (use_lds) {
         w.nbuckets = (uint32_t)dt_entries;
@@ -613,9 +633,9 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         // room for the buckets of a batch of distinct signs only: a call that overflows is repeated with that
         // many, and must not pay for a larger buffer then (freeing and allocating waits for the whole device)
         const size_t nb2_room = std::max<size_t>(w.nb2, (L + GRP_TARGET - 1) / GRP_TARGET);
-        const size_t nb1_room = std::max<size_t>(dt_entries, L / LDS_BUCKET_TARGET + MAX_SLOTS + 1);
-        w.bcount = c.take<uint32_t>(nb1_room + 1 + nb2_room);  // (the part in use is zeroed together)
-        w.cursor2 = w.bcount + dt_entries + 1;
+        const size_t nb1_room = std::max<size_t>(dt_entries, L / L1_FILL + (size_t)N + 1);
+        w.bcursor = c.take<uint32_t>(nb1_room * CURSOR_STRIDE + 1 + nb2_room);  // (the part in use is zeroed together)
+        w.cursor2 = w.bcursor + dt_entries * CURSOR_STRIDE + 1;
         w.recs = c.take<GroupRec>(nb2_room * GRP_CAP);
         w.aux = c.take<uint2>(nb2_room * GRP_CAP);
         w.rrow = c.take<uint32_t>(nb2_room * GRP_CAP);
@@ -623,9 +643,7 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         w.newcnt = c.take<uint32_t>(nb2_room);
         w.bcounts = c.take<uint4>(nb2_room);
         w.bbase = c.take<uint4>(nb2_room);
-        w.bstart = c.take<uint32_t>(nb1_room + 1);
-        w.bcursor = c.take<uint32_t>(nb1_room + 1);
-        w.prec = c.take<ulonglong2>(L);
+        w.prec = c.take<ulonglong2>(nb1_room * (size_t)L1_ROOM);
         w.first_of = c.take<uint32_t>(L);
         w.cnt_at = c.take<uint32_t>(L);
         w.wordpre = c.take<uint32_t>(L / 64 + 2);
@@ -680,23 +698,21 @@ int stage_slots(SparseTable* t, int N, const int64_t* const* values, const int64
     dt_entries = te;
     if (use_lds && *use_lds) {
         bool ok = l >= LDS_MIN_LOOKUPS;
-        for (int s = 0; s < N && ok; s++) ok = (size_t)lens[s] <= (size_t)LDS_MAX_SUB * LDS_BUCKET_TARGET;
+        for (int s = 0; s < N && ok; s++) ok = (size_t)lens[s] <= (size_t)LDS_MAX_SUB * L1_FILL;
         *use_lds = ok;
         if (ok) {
-            // A bucket's LDS table holds its distinct signs: LDS_BUCKET_TARGET lookups per bucket if all
-            // of them could be distinct, up to twice as many when the recent pulls repeated most signs
-            // (the same estimate, with the same margin and the same fallback, as for the second level).
-            const double share = std::min(1.0, std::max(0.5, t->distinct_est * 1.25));
-            const size_t target = (size_t)((double)LDS_BUCKET_TARGET / share);
+            // The buckets have fixed room for the records the tiles hand in (one per distinct sign of a tile):
+            // sized from the share of such records the recent pulls had, with a margin; a batch that overflows
+            // them is repeated with buckets for a batch without repeats.
             size_t nb = 0;
             for (int s = 0; s < N; s++) {
-                size_t sub = std::max<size_t>(1, ((size_t)lens[s] + target - 1) / target);
+                const size_t sub = first_level_buckets((size_t)lens[s], t->tile_est);
                 descs[s].tbase = (uint32_t)nb;
                 descs[s].tcap = (uint32_t)sub;
                 nb += sub;
             }
             dt_entries = nb;
-            // buckets the widest tile of the partition kernels touches: first bucket of the slot of
+            // buckets the widest tile of the partition kernel touches: first bucket of the slot of
             // its first lookup .. last bucket of the slot of its last lookup
             size_t widest = 1;
             int s0 = 0, s1 = 0;
@@ -798,20 +814,16 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
     // second-level buckets up to which k_group_emit adds up the bucket counts itself (one bucket per workgroup)
     const bool own_offsets = w.nb2 <= (uint32_t)GRID_CAP * 4;
     if (use_lds) {
-        // (a workgroup per tile up to twice what the chip holds at once: the workgroups queued behind the resident ones
-        // start as those end, which evens the tail out better than a second tile for some of them)
-        const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, GRID_CAP * 2);
-        const size_t part_lds = ((size_t)N + 1 + w.span_cap) * sizeof(uint32_t);
-        TN_LAUNCH_LDS(k_lds_hist, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcount,
+        // (as many workgroups as the chip holds of this kernel at once -- three per CU --, each taking its tiles in turn)
+        const int tiles = launch_grid((int64_t)(L + LDS_TILE - 1) / LDS_TILE, 1, TILE_GRID);
+        const size_t tile_lds = tile_dedup_lds(N, w.span_cap);
+        TN_LAUNCH_LDS(k_tile_dedup, dim3(tiles), dim3(TILE_THREADS), tile_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.prec,
                       reinterpret_cast<ulonglong2*>(p.vals_copy), p.vals_exact, w.first_of, ds, w.span_cap);
-        TN_LAUNCH(k_lds_offsets, dim3(1), dim3(1024), st, w.bcount, w.bstart, w.bcursor, w.nbuckets);
-        TN_LAUNCH_LDS(k_lds_scatter, dim3(tiles), dim3(256), part_lds, st, p.descs, p.lbase, N, L, w.bcursor, w.prec,
-                      w.span_cap);
         if (lds_groups)
-            TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
+            TN_LAUNCH((k_lds_dedup<true>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bcursor,
                       w.nbuckets, w.prec, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         else
-            TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bstart,
+            TN_LAUNCH((k_lds_dedup<false>), dim3(launch_grid(w.nbuckets, 1, GRID_CAP * 2)), dim3(DEDUP_THREADS), st, w.bcursor,
                       w.nbuckets, w.prec, w.first_of, w.cnt_at, ds, w.nb2, w.cursor2, w.recs);
         if (lds_groups) {
             // The grouping of the distinct records only needs what the dedup handed over: it runs on
@@ -839,7 +851,8 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
                       make_optdev(t), t->seed, w.recs, w.rrow, w.nb2, w.newrec, w.newcnt, ds, init_parts);
             if (!t->one_stream) TN_HIP(hipEventRecord(t->join2_ev, t->side2));
         }
-        TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum);
+        TN_LAUNCH(k_lds_flags, dim3(w.ntiles), dim3(REMAP_THREADS), st, L, w.first_of, w.flag8, w.tilesum, p.descs, N,
+                  w.bcursor, ds);
         // up to SELF_SCAN_TILES tiles the ranking pass adds up the tile counts itself
         const uint32_t* own_sums = w.ntiles <= SELF_SCAN_TILES ? w.tilesum : nullptr;
         if (!own_sums)
@@ -1644,7 +1657,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
     bool use_lds = !t->async_pull;
     bool small_allowed = true;
     for (int attempt = 0; attempt < 3; attempt++) {
-        const double est_used = t->distinct_est;  // what this attempt's buckets are sized from
+        const double est_used = std::min(t->distinct_est, t->tile_est);  // what this attempt's buckets are sized from
         std::vector<SlotDesc> descs;
         std::vector<uint32_t> lbase;
         size_t L = 0, dt_entries = 0;
@@ -1676,8 +1689,8 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         const bool exact = t->exact_verify && use_lds && !small;
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L, exact)));
         carve_plan((char*)t->plan_buf.p, p, N, L, exact);
-        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, lds_scratch, t->distinct_est)));
-        carve_scratch((char*)t->ws.p, w, L, dt_entries, lds_scratch, t->distinct_est);
+        TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, lds_scratch, t->distinct_est, N)));
+        carve_scratch((char*)t->ws.p, w, L, dt_entries, lds_scratch, t->distinct_est, N);
         w.span_cap = span_cap;
         t->plan_valid = false;
         // Detached updates of the push before read its plan in this same buffer.  A batch of the same slot count
@@ -1752,6 +1765,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                 harvest(t);
                 if (est_used >= 1.0) small_allowed = false;
                 t->distinct_est = 1.0;
+                t->tile_est = 1.0;
                 t->latched = TN_OK;
                 t->latched_msg.clear();
                 continue;
@@ -1769,7 +1783,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         behind_push = false;
         if (hoist && t->tail_recorded) TN_HIP(hipStreamWaitEvent(t->aux, t->tail_ev, 0));  // the gather that read p.descs
         TN_TRY(upload_slots(t, p.descs, p.lbase, t->dplan, descs, lbase, hoist ? t->aux : st, STATUS_NEW_PLAN,
-                            use_lds ? w.bcount : nullptr, use_lds ? w.nbuckets + 1 + w.nb2 : 0));
+                            use_lds ? w.bcursor : nullptr, use_lds ? w.nbuckets * CURSOR_STRIDE + 1 + w.nb2 : 0));
         if (hoist) TN_HIP(hipStreamWaitEvent(st, t->stage_ev, 0));
 
         const Store& s = t->store;
@@ -1837,6 +1851,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
             // the global-table path, which remains for the batch that overflows even then.
             if (est_used >= 1.0) use_lds = false;
             t->distinct_est = 1.0;
+            t->tile_est = 1.0;
             t->latched = TN_OK;
             t->latched_msg.clear();
             continue;

@@ -89,7 +89,8 @@ struct DevStatus {
     uint32_t mismatch;   // a push found other signs than the plan was built from
     uint32_t n_big;      // groups with many records (handled one wavefront each)
     uint32_t abort;      // the call's inputs are unusable (flagged in err): later kernels of the call do nothing
-    uint32_t pad[2];
+    uint32_t tile_share_q16;  // remap through LDS: records handed to the first-level buckets per lookup, largest share of a slot, in 1 / 65536
+    uint32_t pad[1];
 };
 
 // The chip is eight dies, each with an L2 of its own, and the workgroups of a launch go to the dies in turn

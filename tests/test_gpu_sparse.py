@@ -715,23 +715,30 @@ def test_many_slots(tn, oracle, slots):
         pair.assert_rows_match(base)
 
 
+def _hash32(signs):
+    """Upper half of the 64-bit hash that places a sign among its slot's first-level buckets, among the
+    second-level buckets and in the table (numpy restatement)."""
+    x = np.asarray(signs, dtype=np.uint64).copy()
+    with np.errstate(over="ignore"):
+        x ^= x >> np.uint64(33)
+        x *= np.uint64(0xFF51AFD7ED558CCD)
+        x ^= x >> np.uint64(33)
+        x *= np.uint64(0xC4CEB9FE1A85EC53)
+        x ^= x >> np.uint64(33)
+    return (x >> np.uint64(32)).astype(np.uint32)
+
+
 def test_remap_falls_back_when_a_bucket_overflows(tn, oracle):
-    """Large batches are remapped through per-bucket hash tables in LDS; a slot whose
-    signs are crafted to fall into one bucket (more distinct signs than the LDS table
-    holds) must still give the reference's ids and rows (the call is redone on the
-    global-table path)."""
+    """Large batches are remapped through hash tables in LDS: every tile of 2048 lookups hands its distinct signs
+    to first-level buckets of fixed room (1536 records), chosen by a hash of the sign; a slot whose signs are
+    crafted to fall into one bucket must still give the reference's ids and rows (the call is redone with more
+    buckets and, as that cannot help here, on the global-table path)."""
     D = 8
     rng = np.random.default_rng(77)
     n_slot = 40000
-    nb = (n_slot + 767) // 768  # buckets of the slot (768 lookups each on average)
+    nb = (n_slot + 1149) // 1150  # buckets of the slot when no sign repeats inside a tile
     cand = rng.integers(0, 1 << 63, 400000, dtype=np.uint64)
-    x = cand.copy()
-    x ^= x >> np.uint64(33)
-    x *= np.uint64(0xFF51AFD7ED558CCD)
-    x ^= x >> np.uint64(33)
-    x *= np.uint64(0xC4CEB9FE1A85EC53)
-    x ^= x >> np.uint64(33)
-    bucket = ((x >> np.uint64(32)) * np.uint64(nb)) >> np.uint64(32)  # ~ umulhi(mix64(sign), nb)
+    bucket = (_hash32(cand).astype(np.uint64) * np.uint64(nb)) >> np.uint64(32)
     crowd = cand[bucket == 0][:6000]
     assert len(crowd) == 6000
     filler = cand[bucket != 0][: n_slot - 6000]
@@ -756,13 +763,7 @@ def test_grouping_falls_back_when_a_second_level_bucket_overflows(tn, oracle):
     slots, per_slot = 64, 1000
     nb2 = (slots * per_slot + 1023) // 1024
     cand = rng.integers(0, 1 << 63, 600000, dtype=np.uint64)
-    x = cand.copy()
-    x ^= x >> np.uint64(33)
-    x *= np.uint64(0xFF51AFD7ED558CCD)
-    x ^= x >> np.uint64(33)
-    x *= np.uint64(0xC4CEB9FE1A85EC53)
-    x ^= x >> np.uint64(33)
-    bucket = ((x >> np.uint64(32)) * np.uint64(nb2)) >> np.uint64(32)
+    bucket = (_hash32(cand).astype(np.uint64) * np.uint64(nb2)) >> np.uint64(32)
     crowd = cand[bucket == 0][:2560]
     assert len(crowd) == 2560
     filler = cand[bucket != 0]
