@@ -42,10 +42,6 @@
 
 namespace tn {
 
-#ifndef TN_CURSOR_STRIDE
-#define TN_CURSOR_STRIDE 1
-#endif
-constexpr int CURSOR_STRIDE = TN_CURSOR_STRIDE;  // words from one first-level bucket's cursor to the next
 constexpr int LDS_TILE = 2048;          // lookups per tile of the partition kernel
 constexpr int TILE_THREADS = 512;
 constexpr int TILE_ITEMS = LDS_TILE / TILE_THREADS;
@@ -68,7 +64,7 @@ constexpr int EMIT_THREADS = 512;
 constexpr int EMIT_RECS = GRP_CAP / EMIT_THREADS;  // records per thread of k_group_emit
 constexpr int GRP_ITEMS = (GRP_TABLE + 1 + GRP_THREADS - 1) / GRP_THREADS;
 constexpr int GRP_SLOTS = 128;          // slot masks are 128 bits wide
-static_assert((uint64_t)LDS_MAX_SUB * L1_ROOM <= 0xFFFFFFull && GRP_SLOTS <= 256,
+static_assert((uint64_t)LDS_MAX_SUB * L1_ROOM <= 0x7FFFFFull && GRP_SLOTS <= 256,
               "a record's word holds the occurrences of a sign in its slot and the slot");
 
 // Raises DEV_ERR_REMAP_OVERFLOW.  A batch that overflows does so in a million places at once: atomics on the one
@@ -81,9 +77,10 @@ __device__ __forceinline__ void flag_overflow(DevStatus* status) {
 struct GroupRec {
     uint64_t sign;
     uint32_t gi;   // position of its first occurrence
-    uint32_t cnt;  // bits 0-23 occurrences in its slot, 24-31 the slot (< GRP_SLOTS)
+    uint32_t cnt;  // bits 0-22 occurrences in its slot, 23 all of them within one tile, 24-31 the slot (< GRP_SLOTS)
 };
-constexpr uint32_t REC_CNT_MASK = 0xFFFFFFu;
+constexpr uint32_t REC_CNT_MASK = 0x7FFFFFu;
+constexpr uint32_t REC_ONE_TILE = 0x800000u;
 
 
 // [0, n) from a 32-bit hash without a division; grows with the hash
@@ -283,7 +280,7 @@ __global__ __launch_bounds__(TILE_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             for (int q = 0; q < 4; q++) {
                 const uint32_t i = i0 + q * TILE_THREADS + threadIdx.x;
                 const uint32_t cnt = i < span ? hist[i] : 0;
-                got[q] = cnt ? atomicAdd(&bcursor[(size_t)(b0.x + i) * CURSOR_STRIDE], cnt) : 0;
+                got[q] = cnt ? atomicAdd(&bcursor[b0.x + i], cnt) : 0;
             }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
@@ -330,7 +327,7 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
     // positions): on one die they meet in one L2 and leave it as whole lines.
     const DieShare share(nbuckets);
     for (uint32_t b = share.first; b < share.end; b += share.step) {
-        const uint32_t n = min(bcursor[(size_t)b * CURSOR_STRIDE], (uint32_t)L1_ROOM);
+        const uint32_t n = min(bcursor[b], (uint32_t)L1_ROOM);
         if (n == 0) continue;
         const size_t first = (size_t)b * L1_ROOM;
         // The bucket's records sit in registers, all loads issued together and in flight while the tables
@@ -396,6 +393,9 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
             } else {
                 if (!EMIT) cnt_at[gi] = cnts[h];  // with EMIT the record carries the count
                 if (EMIT) {  // one record per occupied entry gets here
+                    // the sign's only record: all its lookups lie in one tile (what a push makes of it: the tile's
+                    // click sum for the sign is the whole sum)
+                    if (cnts[h] == mu[j]) cnts[h] |= REC_ONE_TILE;
                     const uint32_t local = group_bucket(sg[j], nb2) - c_lo;
                     if (local < LDS_SPAN2) atomicAdd(&hist2[local], 1u);
                 }
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(DEDUP_THREADS) void k_lds_dedup(const uint32_t* __r
                 if (hist2[i]) hist2[i] = atomicAdd(&cursor2[c_lo + i], hist2[i]);  // this bucket's slice
             __syncthreads();
             for (int e = threadIdx.x; e <= LDS_TABLE; e += DEDUP_THREADS) {
-                const uint32_t cnt = cnts[e];
+                const uint32_t cnt = cnts[e];  // (with the one-tile mark)
                 if (cnt == 0) continue;
                 GroupRec r;
                 r.sign = (e == LDS_TABLE) ? EMPTY_KEY : (uint64_t)keys[e];
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(REMAP_THREADS) void k_lds_flags(uint32_t L, const u
         const SlotDesc& d = descs[sl];
         if (d.len <= (uint32_t)L1_ROOM) continue;  // (the same for the whole workgroup)
         uint32_t mine = 0;
-        for (uint32_t b = threadIdx.x; b < d.tcap; b += REMAP_THREADS) mine += bcursor[(size_t)(d.tbase + b) * CURSOR_STRIDE];
+        for (uint32_t b = threadIdx.x; b < d.tcap; b += REMAP_THREADS) mine += bcursor[d.tbase + b];
         const uint32_t all = block_sum_256(mine, red);
         if (threadIdx.x == 0) {
             const uint64_t q = ((uint64_t)all << 16) / d.len + 1;
@@ -893,7 +893,8 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
 // (several million per call, which is what the kernel's time was).  So the bucket's part of
 // the arrays is first put together in LDS and then copied out in order; only where_u, indexed
 // by the distinct index of the record, stays a scattered store.  where_u[u] = {place in the member
-// list, table row of the record's sign (rrow, from k_probe_recs)}; the groups get the rows too.
+// list (with WHERE_ONE_TILE if all lookups of the record lie in one tile), table row of the record's sign
+// (rrow, from k_probe_recs)}; the groups get the rows too.
 //
 // SLOT_RANKS: a record carries its rank in its slot instead of the position of its first occurrence
 // (the pull of a small batch); its distinct index is the slot's base plus that rank.
@@ -989,6 +990,7 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             m.slot = sl;
             m.show = (int32_t)(r.cnt & REC_CNT_MASK);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
             m.click = 0;
+            const uint32_t one_tile = (r.cnt & REC_ONE_TILE) ? WHERE_ONE_TILE : 0u;
             if (k == 1) {
                 const uint32_t g = bb.x + idx;
                 s_list[idx] = m;
@@ -996,13 +998,13 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                 s_off[idx] = g;
                 s_cnt[idx] = 1;
                 s_row[idx] = rows[j];
-                where_u[m.u] = make_uint2(g, rows[j]);
+                where_u[m.u] = make_uint2(g | one_tile, rows[j]);
             } else {
                 const uint32_t g = ids_cap - 1 - (bb.y + idx);
                 const uint32_t before = a.y & 0xFFFFu;        // records of the bucket's earlier groups of this kind
                 const uint32_t t = before + k - 1 - place;    // local member: the group's last record first
                 s_list[n1 + t] = m;
-                where_u[m.u] = make_uint2(top - t, rows[j]);
+                where_u[m.u] = make_uint2((top - t) | one_tile, rows[j]);
                 if (place == 0) {
                     s_row[n1 + idx] = rows[j];  // every record of the sign was given the same row
                     s_sign[n1 + idx] = r.sign;

@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void k_small_verify(const SlotDesc* host_descs
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         bad |= now[j] != then[j];
-        if (CLICKS && label[j] != 0) atomicAdd(&list[where_u[u[j]].x].click, label[j]);
+        if (CLICKS && label[j] != 0) atomicAdd(&list[where_u[u[j]].x & WHERE_PLACE].click, label[j]);
     }
     if (bad) {
         atomicOr(&status->mismatch, 1u);

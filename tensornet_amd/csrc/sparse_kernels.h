@@ -71,6 +71,11 @@ struct GroupEntry {
 
 // One record of a push in its group's member list: which distinct sign of which
 // slot, and its batch_show / batch_click (SparsePushSignInfo's counts).
+// where_u[u].x: the record's place in the member list; the top bit marks a record whose lookups all lie in one
+// tile of 2048 consecutive lookups (only the remap through LDS sets it).
+constexpr uint32_t WHERE_ONE_TILE = 0x80000000u;
+constexpr uint32_t WHERE_PLACE = 0x7FFFFFFFu;
+
 struct __attribute__((aligned(16))) Member {
     uint32_t u;
     uint32_t slot;
@@ -877,7 +882,7 @@ __global__ __launch_bounds__(256) void k_count_show(const SlotDesc* __restrict__
         for (int i = threadIdx.x; i < COUNT_SLOTS; i += 256) {
             const uint32_t u = keys[i];
             if (u == 0xFFFFFFFFu) continue;
-            Member* m = &list[where_u[u].x];
+            Member* m = &list[where_u[u].x & WHERE_PLACE];
             if (cnts[i]) atomicAdd(&m->show, cnts[i]);
             if (clks[i]) atomicAdd(&m->click, clks[i]);
         }
@@ -1316,6 +1321,7 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
     extern __shared__ uint32_t lb[];  // lb[N + 1], sized by the launch: more tiles in flight per CU than with a fixed array
     __shared__ uint32_t ckey[CLICKS ? CLICK_TABLE : 1];
     __shared__ int csum[CLICKS ? CLICK_TABLE : 1];
+    __shared__ uint32_t crowded;  // a label of the tile went to memory directly: its record's sum in the table is not all of it
     load_lbase(lb, lbase, N);
     bool bad = false;
     const uint32_t n_members = gaddr ? status->n_members : 0;
@@ -1326,6 +1332,7 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                 ckey[i] = 0xFFFFFFFFu;  // no distinct index: they stay below FIRST_BIT
                 csum[i] = 0;
             }
+            if (threadIdx.x == 0) crowded = 0;
             __syncthreads();
         }
         const uint32_t g0 = tile * VERIFY_TILE;
@@ -1384,7 +1391,10 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                     }
                     h = (h + 1) & (CLICK_TABLE - 1);
                 }
-                if (!placed) atomicAdd(&list[where_u[u[j]].x].click, label[j]);
+                if (!placed) {
+                    crowded = 1;
+                    atomicAdd(&list[where_u[u[j]].x & WHERE_PLACE].click, label[j]);
+                }
             }
         }
         if (CLICKS) {
@@ -1398,9 +1408,17 @@ __global__ __launch_bounds__(256) void k_verify_values(const SlotDesc* __restric
                 sum[j] = csum[e];
                 place[j] = sum[j] != 0 ? where_u[ckey[e]].x : 0u;
             }
+            // A record whose lookups all lie in this tile gets its whole sum here: a plain store (the sums start at
+            // zero), where an atomic would wait for its turn at the memory's atomic unit.
+            const bool plain_ok = crowded == 0;
 #pragma unroll
-            for (int j = 0; j < PER; j++)
-                if (sum[j] != 0) atomicAdd(&list[place[j]].click, sum[j]);
+            for (int j = 0; j < PER; j++) {
+                if (sum[j] == 0) continue;
+                if ((place[j] & WHERE_ONE_TILE) && plain_ok)
+                    list[place[j] & WHERE_PLACE].click = sum[j];
+                else
+                    atomicAdd(&list[place[j] & WHERE_PLACE].click, sum[j]);
+            }
             __syncthreads();
         }
     }
@@ -1608,15 +1626,24 @@ __device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o,
         // issued whether its record exists or not (past the end: the group's last member again, the row in place of
         // a gradient): a load under a condition makes the compiler wait for all loads where the branches join.
         Member m1[AHEAD], m2[AHEAD];
+        const float* a1[AHEAD];  // with ga: the records' gradient addresses, worked out beforehand
+        const float* a2[AHEAD];
         float4 g0[AHEAD], g1[AHEAD];
         int sh0[AHEAD], ck0[AHEAD], sh1[AHEAD], ck1[AHEAD];
         bool ok0[AHEAD], ok1[AHEAD];
-        auto fetch = [&](const Member (&m)[AHEAD], uint32_t first, float4 (&g)[AHEAD], int (&sh)[AHEAD], int (&ck)[AHEAD],
-                         bool (&ok)[AHEAD]) {
+        auto fetch = [&](const Member (&m)[AHEAD], const float* const (&a)[AHEAD], uint32_t first, float4 (&g)[AHEAD],
+                         int (&sh)[AHEAD], int (&ck)[AHEAD], bool (&ok)[AHEAD]) {
 #pragma unroll
             for (int q = 0; q < AHEAD; q++) {
                 const float* gp = nullptr;
-                ok[q] = src_record(src, m[q], gp, sh[q], ck[q]) && first + q < k;
+                if (ga) {
+                    gp = a[q];
+                    sh[q] = m[q].show;
+                    ck[q] = m[q].click;
+                    ok[q] = gp != nullptr && first + q < k;
+                } else {
+                    ok[q] = src_record(src, m[q], gp, sh[q], ck[q]) && first + q < k;
+                }
                 g[q] = reinterpret_cast<const float4*>(ok[q] ? gp : wp)[sub];
             }
         };
@@ -1624,22 +1651,84 @@ __device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o,
         for (int q = 0; q < AHEAD; q++) {
             m1[q] = mem[min((uint32_t)q, k - 1)];
             m2[q] = mem[min((uint32_t)(AHEAD + q), k - 1)];
+            a1[q] = ga ? ga[min((uint32_t)q, k - 1)] : nullptr;
+            a2[q] = ga ? ga[min((uint32_t)(AHEAD + q), k - 1)] : nullptr;
         }
-        fetch(m1, 0, g0, sh0, ck0, ok0);
+        fetch(m1, a1, 0, g0, sh0, ck0, ok0);
 #pragma unroll
-        for (int q = 0; q < AHEAD; q++) m1[q] = m2[q];
+        for (int q = 0; q < AHEAD; q++) {
+            m1[q] = m2[q];
+            a1[q] = a2[q];
+        }
         for (uint32_t c0 = 0; c0 < k; c0 += AHEAD) {
 #pragma unroll
-            for (int q = 0; q < AHEAD; q++) m2[q] = mem[min(c0 + 2 * AHEAD + q, k - 1)];
-            fetch(m1, c0 + AHEAD, g1, sh1, ck1, ok1);
-#pragma unroll
             for (int q = 0; q < AHEAD; q++) {
-                if (c0 + q >= k) break;
-                if (!ok0[q]) {
-                    no_gradient();
-                    continue;
+                m2[q] = mem[min(c0 + 2 * AHEAD + q, k - 1)];
+                a2[q] = ga ? ga[min(c0 + 2 * AHEAD + q, k - 1)] : nullptr;
+            }
+            fetch(m1, a1, c0 + AHEAD, g1, sh1, ck1, ok1);
+            if constexpr (KIND == OPT_ADAGRAD) {
+                // The records of the window depend on each other through g2sum (one rounded addition per record)
+                // and through the row (one subtraction per element and record) only.  Everything else -- the sums of
+                // squares with their hand-over from lane to lane, the square roots, the divisions -- is worked
+                // out for all records of the window side by side; the two chains then run over the results, in
+                // record order.  The same operations on the same operands as record after record.
+                double mq[AHEAD];
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) mq[q] = 0.0;
+                for (int l = 0; l < LPG; l++) {
+#pragma unroll
+                    for (int q = 0; q < AHEAD; q++) {
+                        double cand = mq[q];  // add_g2sum: double accumulator over the float products, element order 0..D-1
+                        cand += (double)(g0[q].x * g0[q].x);
+                        cand += (double)(g0[q].y * g0[q].y);
+                        cand += (double)(g0[q].z * g0[q].z);
+                        cand += (double)(g0[q].w * g0[q].w);
+                        mq[q] = __shfl(cand, lane0 + l);
+                    }
                 }
-                step(g0[q], sh0[q], ck0[q]);
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) mq[q] = mq[q] / (double)D;
+                float g2[AHEAD];
+                bool missing = false;
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) {
+                    if (ok0[q]) {
+                        any = true;
+                        show += (float)sh0[q];
+                        click += (float)ck0[q];
+                        g2sum = (float)((double)g2sum + mq[q]);
+                    } else if (c0 + q < k) {
+                        missing = true;
+                    }
+                    g2[q] = g2sum;
+                }
+                float4 st4[AHEAD];
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) {
+                    const float den = o.eps + sqrtf(g2[q]);
+                    st4[q] = make_float4(o.lr * g0[q].x / den, o.lr * g0[q].y / den, o.lr * g0[q].z / den,
+                                         o.lr * g0[q].w / den);
+                }
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) {
+                    if (!ok0[q]) continue;
+                    w.x -= st4[q].x;
+                    w.y -= st4[q].y;
+                    w.z -= st4[q].z;
+                    w.w -= st4[q].w;
+                }
+                if (missing) no_gradient();
+            } else {
+#pragma unroll
+                for (int q = 0; q < AHEAD; q++) {
+                    if (c0 + q >= k) break;
+                    if (!ok0[q]) {
+                        no_gradient();
+                        continue;
+                    }
+                    step(g0[q], sh0[q], ck0[q]);
+                }
             }
 #pragma unroll
             for (int q = 0; q < AHEAD; q++) {
@@ -1648,6 +1737,7 @@ __device__ __forceinline__ void apply_group_vec(const Store& s, const OptDev& o,
                 ck0[q] = ck1[q];
                 ok0[q] = ok1[q];
                 m1[q] = m2[q];
+                a1[q] = a2[q];
             }
         }
     }
@@ -1688,8 +1778,8 @@ __global__ __launch_bounds__(256) void k_apply_vec(Store s, OptDev o, PushSrc sr
         if (row > s.cap) continue;  // NO_ROW (unknown sign: flagged by the probe), or no row number at all
         const uint32_t k = grp_cnt[g];
         if (is_big(k, big_k)) continue;
-        apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g], gaddr ? gaddr + grp_off[g] : nullptr, sub,
-                                   lane0, c1, c2);
+        apply_group_vec<KIND, LPG>(s, o, src, status, row, k, list + grp_off[g],
+                                                 gaddr ? gaddr + grp_off[g] : nullptr, sub, lane0, c1, c2);
     }
 }
 

@@ -35,10 +35,7 @@ constexpr int PROBE_RECS_GRID = 1024;  // workgroups of k_probe_recs (measured: 
 constexpr size_t ONE_STREAM_LOOKUPS = 3u << 20;
 constexpr uint32_t SELF_SCAN_TILES = 8192;  // tiles of the ranking pass up to which no scan kernel runs between its launches
 constexpr int GRID_CAP = 256 * 8;                       // 256 CUs x 8 workgroups of 256 threads
-#ifndef TN_TILE_GRID
-#define TN_TILE_GRID (256 * 3)
-#endif
-constexpr int TILE_GRID = TN_TILE_GRID;                 // workgroups of k_tile_dedup
+constexpr int TILE_GRID = 256 * 3;                      // workgroups of k_tile_dedup: what the chip holds of it at once
 constexpr size_t LDS_MIN_LOOKUPS = 1024;  // from here on the remap through LDS wins: it also takes fewer launches (cfg1, 8 k lookups: 0.154 -> 0.136 ms)
 
 // Up to this many lookups a batch whose slots each fit one workgroup (SMALL_SLOT_MAX lookups, SMALL_SLOTS slots)
@@ -634,8 +631,8 @@ size_t carve_scratch(char* base, Scratch& w, size_t L, size_t dt_entries, bool u
         // many, and must not pay for a larger buffer then (freeing and allocating waits for the whole device)
         const size_t nb2_room = std::max<size_t>(w.nb2, (L + GRP_TARGET - 1) / GRP_TARGET);
         const size_t nb1_room = std::max<size_t>(dt_entries, L / L1_FILL + (size_t)N + 1);
-        w.bcursor = c.take<uint32_t>(nb1_room * CURSOR_STRIDE + 1 + nb2_room);  // (the part in use is zeroed together)
-        w.cursor2 = w.bcursor + dt_entries * CURSOR_STRIDE + 1;
+        w.bcursor = c.take<uint32_t>(nb1_room + 1 + nb2_room);  // (the part in use is zeroed together)
+        w.cursor2 = w.bcursor + dt_entries + 1;
         w.recs = c.take<GroupRec>(nb2_room * GRP_CAP);
         w.aux = c.take<uint2>(nb2_room * GRP_CAP);
         w.rrow = c.take<uint32_t>(nb2_room * GRP_CAP);
@@ -1783,7 +1780,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         behind_push = false;
         if (hoist && t->tail_recorded) TN_HIP(hipStreamWaitEvent(t->aux, t->tail_ev, 0));  // the gather that read p.descs
         TN_TRY(upload_slots(t, p.descs, p.lbase, t->dplan, descs, lbase, hoist ? t->aux : st, STATUS_NEW_PLAN,
-                            use_lds ? w.bcursor : nullptr, use_lds ? w.nbuckets * CURSOR_STRIDE + 1 + w.nb2 : 0));
+                            use_lds ? w.bcursor : nullptr, use_lds ? w.nbuckets + 1 + w.nb2 : 0));
         if (hoist) TN_HIP(hipStreamWaitEvent(st, t->stage_ev, 0));
 
         const Store& s = t->store;
