@@ -32,7 +32,7 @@ def log(msg):
 # profiles/cfg3_adagrad_dim16_pull_push.md (counters cannot be read from inside this script).
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "cfg3_traffic.json")
 # launched by a step, a few microseconds each, no traffic worth counting
-SMALL_STEP_KERNELS = ("k_stage_in", "k_publish", "k_lds_offsets", "k_init_new_recs", "k_group_offsets", "k_scan_tiles")
+SMALL_STEP_KERNELS = ("k_stage_in", "k_publish", "k_init_new_recs", "k_group_offsets", "k_scan_tiles")
 
 
 def measured_traffic(step_kernels):
@@ -83,10 +83,12 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
         return records * (row + 16) + groups * (2 * row + st)
 
     table = {
-        # remap through LDS
-        "k_lds_hist": 8 * L + L // 32,         # reads every sign, leaves 16 bytes of fingerprint per 64 of them
-        "k_lds_scatter": 20 * L,               # reads every sign, writes {sign, position} by bucket
-        "k_lds_dedup": 16 * L + 16 * U,        # reads {sign, position}, writes first positions and the distinct records
+        # remap through LDS (T: distinct signs per 2048-lookup tile, summed over the tiles)
+        "k_tile_dedup": 12 * L + L // 32 + 16 * shape["T"],  # reads every sign, leaves its first position in the tile,
+                                                             # 16 bytes of fingerprint per 64 signs and a record per
+                                                             # distinct sign of a tile
+        "k_lds_dedup": 16 * shape["T"] + 4 * (shape["T"] - U) + 16 * U,  # the tiles' records in; first positions for the
+                                                                         # tiles' repeats and the distinct records out
         "k_lds_flags": 4 * L,
         "k_lds_assign": 4 * U,
         "k_lds_mapped": 12 * L,                # first position in, mapped id out
@@ -119,10 +121,17 @@ def batch_shape(values):
 
     per_slot = [torch.unique(v) for v in values]
     _, k = torch.unique(torch.cat(per_slot), return_counts=True)
+    # distinct (tile, slot, sign) triples: what the tiles of 2048 consecutive lookups hand on
+    tile_recs, pos = 0, 0
+    for v in values:
+        tiles = (torch.arange(v.numel(), device=v.device) + pos) // 2048
+        tile_recs += int(torch.unique(torch.stack([tiles, v], 1), dim=0).shape[0])
+        pos += v.numel()
     mid = (k > 1) & (k < BIG_GROUP)
     big = k >= BIG_GROUP
     return {
         "L": sum(v.numel() for v in values), "U": sum(u.numel() for u in per_slot), "G": int(k.numel()),
+        "T": tile_recs,
         "G1": int((k == 1).sum()), "Gm": int(mid.sum()), "Rm": int(k[mid].sum()),
         "Gb": int(big.sum()), "Rb": int(k[big].sum()),
     }
@@ -137,6 +146,17 @@ def populate(tn, handle, resident, dim):
     log("populated %d keys in %.1f s" % (resident, time.time() - t0))
 
 
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(cfg, values, grads_sigma):
     """Times the CPU oracle (the reference's data structures, one thread) on one
     full batch: pull op then push op.  The CPU table only holds the keys the batch
@@ -146,6 +166,7 @@ def cpu_baseline(cfg, values, grads_sigma):
     from oracle import cpu as oracle
     from tensornet_amd import synth
 
+    oracle.load(timed=True)  # the build with the reference's Release flags
     kinds = {"AdaGrad": oracle.ADAGRAD, "Adam": oracle.ADAM, "Ftrl": oracle.FTRL}
     dim = cfg["dim"]
     t = oracle.Table(kinds[cfg["opt"]], dim, buckets=15485863, **cfg["hyper"])
@@ -165,15 +186,100 @@ def cpu_baseline(cfg, values, grads_sigma):
     assert rc == 0
     secs = (t1 - t0) + (t3 - t2)
     log("cpu baseline: pull %.2f s, push %.2f s, %d lookups, %d rows" % (t1 - t0, t3 - t2, L, int(counts.sum())))
+    from oracle import cpu as oracle_front
+
     return {
         "value": L / secs,
         "unit": "keys/s",
         "cores": 1,
+        "threads": 1,
+        "cpu_model": host_cpu_model(),
+        "host_cores": os.cpu_count(),
+        "flags": oracle_front.TIMED_FLAGS,
         "kind": "port",
         "sample": "1 full batch (%d lookups, %d per-slot distinct rows), pull op + push op, CPU table "
                   "pre-populated with only the %d keys the batch touches" % (L, int(counts.sum()), len(signs)),
         "pull_s": t1 - t0,
         "push_s": t3 - t2,
+    }
+
+
+# The other configurations the path is stated on: optimizers, dims and resident keys of the tables one step pulls
+# from and pushes to (cfg4: the wide Ftrl weights and the deep AdaGrad embeddings of the same signs).
+OTHER_TABLES = {
+    "cfg1": [("AdaGrad", 8, dict(learning_rate=0.01, initial_g2sum=0.1, epsilon=1e-8))],
+    "cfg2": [("Adam", 16, dict(learning_rate=1e-3, beta1=0.9, beta2=0.999, epsilon=1e-8))],
+    "cfg4": [("Ftrl", 1, dict(learning_rate=0.05, beta=1.0, lambda1=1.0, lambda2=1.0)),
+             ("AdaGrad", 64, dict(learning_rate=0.01, initial_g2sum=0.1, epsilon=1e-8))],
+    "cfg5": [("AdaGrad", 16, dict(learning_rate=0.01, initial_g2sum=0.1, epsilon=1e-8))],
+}
+
+
+def other_config(tn, name, steps=10, warmup=2, small_path=True):
+    """Pull + push steps of one of the other configurations at its stated shape and resident keys, each step on a
+    seeded batch of its own (the new keys of a step are inserted inside it); the tables are given back afterwards."""
+    import torch
+
+    from tensornet_amd import synth
+
+    cfg = synth.CONFIGS[name]
+    rng = torch.Generator(device="cuda")
+    rng.manual_seed(1)
+    tables = []
+    for opt_name, dim, hyper in OTHER_TABLES[name]:
+        h = tn.core.create_sparse_table(getattr(tn.core, opt_name)(**hyper), "", dim, False, "")
+        tn.core.reserve_sparse_table(h, int(cfg["resident"] * 1.02) + (1 << 22))
+        tn.core.set_sparse_table_small_batch_path(h, small_path)
+        synth.populate_table(tn, h, cfg["resident"], dim)
+        tables.append((h, opt_name, dim))
+    bound, Ls, Us = [], [], []
+    for b in range(warmup + steps):
+        hb = synth.make_batch(cfg, b)
+        values = [torch.from_numpy(v).cuda() for v in hb]
+        labels = [torch.from_numpy(l).cuda() for l in synth.make_labels(hb, b)]
+        ops = []
+        for h, opt_name, dim in tables:
+            grads = [torch.randn((len(v), dim), device="cuda", generator=rng) * cfg["grad_sigma"] for v in values]
+            vars_ = [torch.zeros((len(v) + 1, dim), device="cuda") for v in values]
+            ops.append((tn.ops.BoundSparseTablePull(vars_, values, h), tn.ops.BoundSparseTablePush(values, grads, labels, h)))
+        bound.append(ops)
+        Ls.append(sum(v.numel() for v in values))
+        Us.append(sum(int(torch.unique(v).numel()) for v in values))
+
+    def step(i):
+        for pull, push in bound[i]:
+            pull()
+            push()
+
+    for i in range(warmup):
+        step(i)
+    for h, _, _ in tables:
+        tn.ops.sparse_table_sync(h)
+    torch.cuda.synchronize()
+    keys_before = [tn.core.sparse_table_key_count(h) for h, _, _ in tables]
+    t0 = time.perf_counter()
+    for i in range(warmup, warmup + steps):
+        step(i)
+    for h, _, _ in tables:
+        tn.ops.sparse_table_sync(h)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    new_keys = [tn.core.sparse_table_key_count(h) - k for (h, _, _), k in zip(tables, keys_before)]
+    total_L = sum(Ls[warmup:])
+    total_U = sum(Us[warmup:])
+    alg = sum(step_algorithmic_bytes(opt_name, dim, total_L, total_U) for _, opt_name, dim in tables)
+    for h, _, _ in tables:
+        tn.core.clear_sparse_table(h)
+    del bound
+    torch.cuda.empty_cache()
+    return {
+        "tables": ["%s dim %d" % (o, d) for _, o, d in tables],
+        "resident_keys": cfg["resident"],
+        "lookups_per_step": total_L / steps,
+        "ms_per_step": wall * 1e3 / steps,
+        "keys_per_s": total_L / wall,
+        "new_keys_per_step": new_keys[0] / steps,
+        "step_frac_of_hbm_peak": alg / wall / HBM_PEAK,
     }
 
 
@@ -193,6 +299,8 @@ def main():
                     help="leave roofline.traffic out (development runs on kernels newer than the committed profile)")
     ap.add_argument("--no-fallback", action="store_true", help="skip the side measurement of a pull whose buckets overflow")
     ap.add_argument("--no-decay", action="store_true", help="skip the ShowDecay side measurement")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the side measurement of the other configurations (cfg1, cfg2, cfg4, cfg5)")
     ap.add_argument("--detached-updates", action="store_true",
                     help="the timed steps with the push's update kernels detached (tn_sparse_table_set_detached_updates)")
     ap.add_argument("--detached", action="store_true", help="add the side measurement of detached updates")
@@ -615,6 +723,24 @@ def main():
             "traffic_frac_of_hbm_peak": 40 * total / gsec / HBM_PEAK,
         }
         del w, g
+
+    # ---- side measurement: the other configurations, on tables of their own ---------------------------
+    if args.config == "cfg3" and not args.no_others:
+        del bound, batches
+        tn.core.clear_sparse_table(h)  # (cfg5's table takes 176 GB)
+        torch.cuda.empty_cache()
+        others = {}
+        for name in ("cfg1", "cfg2", "cfg4", "cfg5"):
+            t_cfg = time.time()
+            others[name] = other_config(tn, name)
+            if name in ("cfg1", "cfg2"):  # small enough for the path of few launches: the other path beside it
+                others[name]["other_path_ms_per_step"] = other_config(tn, name, small_path=False)["ms_per_step"]
+            log("%s: %.4f ms/step, %.3e keys/s, %.0f new keys per step, %.3f of the HBM roofline (%.1f s)" %
+                (name, others[name]["ms_per_step"], others[name]["keys_per_s"], others[name]["new_keys_per_step"],
+                 others[name]["step_frac_of_hbm_peak"], time.time() - t_cfg))
+        if "dense_adam" in out:  # cfg5's step also applies the dense Adam update measured above
+            others["cfg5"]["with_dense_adam_ms_per_step"] = others["cfg5"]["ms_per_step"] + out["dense_adam"]["ms_per_step"]
+        out["other_configs"] = others
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg, host_batch0, cfg["grad_sigma"])

@@ -11,25 +11,33 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# the same source built with the reference's Release flags: what bench.py times as the CPU baseline
+TIMED_LIB_PATH = os.path.join(_HERE, "liboracle_timed.so")
+TIMED_FLAGS = "g++ -O3 -DNDEBUG -march=x86-64-v2 -mavx -std=c++14 (CMakeLists.txt:224-238 of the reference)"
 
 ADAGRAD, ADAM, FTRL = 0, 1, 2
 
 sign_info_dtype = np.dtype([("sign", "<u8"), ("batch_show", "<i4"), ("batch_click", "<i4")])
 
 _lib = None
+_timed = False
 
 
 def build():
     subprocess.check_call(["make", "-C", _HERE, "-s"])
 
 
-def load():
-    global _lib
-    if _lib is not None:
+def load(timed=False):
+    """The checker's library; timed=True switches every later call of this module to the build with the
+    reference's Release flags (bench.py's CPU baseline; parity tests keep the default build)."""
+    global _lib, _timed
+    if _lib is not None and (not timed or _timed):
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = TIMED_LIB_PATH if timed else LIB_PATH
+    if not os.path.exists(path):
         build()
-    lib = C.CDLL(LIB_PATH)
+    lib = C.CDLL(path)
+    _timed = bool(timed)
     P = C.c_void_p
     lib.orc_table_create.restype = P
     lib.orc_table_create.argtypes = [C.c_int, P, C.c_int, C.c_int, C.c_int, C.c_uint64, C.c_uint64]

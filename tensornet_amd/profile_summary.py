@@ -6,9 +6,9 @@ benchmark's roofline figures rest on:
 
 The runs (MI355X box, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd $GRAFT_REPO_ROOT`):
 
-    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_trace -o t -- python3 bench.py --steps 5 --warmup 2 --no-cpu
-    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o f -- python3 bench.py --steps 2 --warmup 1 --no-cpu
-    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o w -- python3 bench.py --steps 2 --warmup 1 --no-cpu
+    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_trace -o t -- python3 bench.py --steps 5 --warmup 2 --no-cpu --no-others
+    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o f -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others
+    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o w -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others
     python3 bench.py > gpurun_out/bench_full.json
     python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_trace --fetch gpurun_out/prof_fetch \\
         --write gpurun_out/prof_write --bench gpurun_out/bench_full.json --commit <commit of the profiled tree>
