@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void k_lookup_keys(const SlotDesc* __restrict_
 // svals[seg_off[u] .. seg_off[u + 1]).  The example ids of a slot ascend with the position and two lookups of
 // one sign in one example carry the same value, so "position order" is "ascending value" and ties do not
 // matter: no stable sort is needed.
-//   k_place_lookups  one workgroup per slot (the distinct indices of a slot's lookups fill a window of their
+//   k_place_lookups  a few workgroups per slot (the distinct indices of a slot's lookups fill a window of their
 //                    own, ascending with the slots): counts the lookups of every index in an LDS array, scans
 //                    the counts into seg_off, and puts every lookup into its index's segment -- in the order the
 //                    atomics arrive; indices with ORDER_MID lookups or more are listed for the kernels below
@@ -181,25 +181,37 @@ constexpr int PLACE_ITEMS = 8;
 constexpr uint32_t ORDER_MID = 64;
 constexpr uint32_t ORDER_HUGE = 1024;
 
+// `parts` workgroups per slot: each of them streams all lookups of the slot (they come out of L2 after the first)
+// and takes those whose distinct index lies in its share of the slot's window of distinct indices -- a workgroup
+// per slot leaves most of the device idle, and what bounds it are the LDS atomics and the stores that depend on
+// them, which a share divides.  The lookups of the indices below its share, which it counts on the way, come
+// before its own in svals.
 __global__ __launch_bounds__(PLACE_THREADS) void k_place_lookups(
     const uint32_t* __restrict__ lbase, const uint32_t* __restrict__ ubase, int N, uint32_t L,
     const uint32_t* __restrict__ u_of_gi, const uint64_t* __restrict__ vals, uint32_t* __restrict__ tkey,
     uint64_t* __restrict__ tval, uint32_t* __restrict__ seg_off, uint32_t* __restrict__ gcur, uint32_t lds_cap,
-    uint32_t* __restrict__ mid_list, uint32_t* __restrict__ huge_list, uint32_t* counts, const DevStatus* status) {
+    uint32_t* __restrict__ mid_list, uint32_t* __restrict__ huge_list, uint32_t* counts, const DevStatus* status,
+    uint32_t parts) {
     extern __shared__ uint32_t lcur[];
     __shared__ uint32_t red[PLACE_THREADS / 64];
     __shared__ uint32_t carry_sh;
     if (status->abort) return;
-    const int sl = blockIdx.x;
+    const int sl = blockIdx.x / parts;
+    const uint32_t part = blockIdx.x % parts;
     const uint32_t l0 = lbase[sl], len = lbase[sl + 1] - l0;
     const uint32_t ub = ubase[sl], us = ubase[sl + 1] - ub;
-    if (sl == N - 1 && threadIdx.x == 0) seg_off[ubase[N]] = L;
+    if (sl == N - 1 && part == 0 && threadIdx.x == 0) seg_off[ubase[N]] = L;
     if (len == 0) return;
-    uint32_t* const cur = us <= lds_cap ? lcur : gcur + ub;
+    // my share of the slot's distinct indices (relative to ub)
+    const uint32_t r0 = (uint32_t)((uint64_t)us * part / parts), r1 = (uint32_t)((uint64_t)us * (part + 1) / parts);
+    const uint32_t mine = r1 - r0;
+    if (mine == 0) return;
+    uint32_t* const cur = mine <= lds_cap ? lcur : gcur + ub + r0;
     const uint32_t* const keys = u_of_gi + l0;
-    for (uint32_t i = threadIdx.x; i < us; i += PLACE_THREADS) cur[i] = 0;
+    for (uint32_t i = threadIdx.x; i < mine; i += PLACE_THREADS) cur[i] = 0;
     __syncthreads();
-    // (eight lookups per thread at a time, their loads in flight together: one workgroup streams the whole slot)
+    // (eight lookups per thread at a time, their loads in flight together)
+    uint32_t below = 0;  // lookups of the indices before my share
     for (uint32_t i0 = threadIdx.x; i0 < len; i0 += PLACE_THREADS * PLACE_ITEMS) {
         uint32_t k[PLACE_ITEMS];
 #pragma unroll
@@ -208,23 +220,31 @@ __global__ __launch_bounds__(PLACE_THREADS) void k_place_lookups(
             k[j] = i < len ? (keys[i] & ~FIRST_BIT) - ub : 0xFFFFFFFFu;
         }
 #pragma unroll
-        for (int j = 0; j < PLACE_ITEMS; j++)
-            if (k[j] != 0xFFFFFFFFu) atomicAdd(&cur[k[j]], 1u);
+        for (int j = 0; j < PLACE_ITEMS; j++) {
+            if (k[j] < r0)
+                below++;
+            else if (k[j] < r1)
+                atomicAdd(&cur[k[j] - r0], 1u);
+        }
     }
-    if (threadIdx.x == 0) carry_sh = l0;  // the lookups of the slots before come first
+    {
+        uint32_t total;
+        block_excl_scan<uint32_t, PLACE_THREADS / 64>(below, red, &total);
+        if (threadIdx.x == 0) carry_sh = l0 + total;  // the lookups of the slots before, and of the shares before, come first
+    }
     __syncthreads();
-    for (uint32_t i0 = 0; i0 < us; i0 += PLACE_THREADS) {
+    for (uint32_t i0 = 0; i0 < mine; i0 += PLACE_THREADS) {
         const uint32_t i = i0 + threadIdx.x;
-        const uint32_t cnt = i < us ? ld_relaxed(cur + i) : 0u;  // (counted by atomics: not through the L1 cache)
+        const uint32_t cnt = i < mine ? ld_relaxed(cur + i) : 0u;  // (counted by atomics: not through the L1 cache)
         uint32_t total;
         const uint32_t at = carry_sh + block_excl_scan<uint32_t, PLACE_THREADS / 64>(cnt, red, &total);
-        if (i < us) {
+        if (i < mine) {
             cur[i] = at;
-            seg_off[ub + i] = at;
+            seg_off[ub + r0 + i] = at;
             if (cnt >= ORDER_HUGE)
-                huge_list[atomicAdd(&counts[2], 1u)] = ub + i;
+                huge_list[atomicAdd(&counts[2], 1u)] = ub + r0 + i;
             else if (cnt >= ORDER_MID)
-                mid_list[atomicAdd(&counts[1], 1u)] = ub + i;
+                mid_list[atomicAdd(&counts[1], 1u)] = ub + r0 + i;
         }
         __syncthreads();
         if (threadIdx.x == 0) carry_sh += total;
@@ -237,12 +257,12 @@ __global__ __launch_bounds__(PLACE_THREADS) void k_place_lookups(
         for (int j = 0; j < PLACE_ITEMS; j++) {
             const uint32_t i = i0 + j * PLACE_THREADS;
             k[j] = i < len ? (keys[i] & ~FIRST_BIT) - ub : 0xFFFFFFFFu;
-            v[j] = i < len ? vals[l0 + i] : 0ull;
+            v[j] = (k[j] >= r0 && k[j] < r1) ? vals[l0 + i] : 0ull;
         }
 #pragma unroll
         for (int j = 0; j < PLACE_ITEMS; j++) {
-            if (k[j] == 0xFFFFFFFFu) continue;
-            const uint32_t at = atomicAdd(&cur[k[j]], 1u);
+            if (k[j] < r0 || k[j] >= r1) continue;
+            const uint32_t at = atomicAdd(&cur[k[j] - r0], 1u);
             tkey[at] = ub + k[j];
             tval[at] = v[j];
         }
@@ -364,15 +384,14 @@ __device__ __forceinline__ void add_lookup_share(const float* __restrict__ poole
 
 // Step 3: one group of `chunks` threads per distinct index sums its lookups' shares of the
 // pooled gradient rows, in position order.  A distinct index with long_min lookups or more (a
-// frequent sign) is only noted in long_list: one workgroup each sums those (k_reduce_long).
+// frequent sign) is left out: k_place_lookups has listed those, one workgroup each sums them (k_reduce_long).
 template <int VEC>
 __global__ __launch_bounds__(256) void k_reduce_pooled(const SlotDesc* __restrict__ descs,
                                                        const uint32_t* __restrict__ ubase, int N, int dim,
                                                        int combiner, const DevStatus* status,
                                                        const uint32_t* __restrict__ seg_off,
                                                        const uint64_t* __restrict__ svals, float* __restrict__ flat,
-                                                       uint32_t long_min, uint32_t* __restrict__ long_list,
-                                                       uint32_t* long_count) {
+                                                       uint32_t long_min) {
     if (status->abort) return;
     __shared__ uint32_t ub[MAX_SLOTS + 1];
     load_lbase(ub, ubase, N);
@@ -383,10 +402,7 @@ __global__ __launch_bounds__(256) void k_reduce_pooled(const SlotDesc* __restric
         const uint32_t u = (uint32_t)(t / chunks);
         const int c = (int)(t - (int64_t)u * chunks);
         const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
-        if (hi - lo >= long_min) {
-            if (c == 0) long_list[atomicAdd(long_count, 1u)] = u;
-            continue;
-        }
+        if (hi - lo >= long_min) continue;  // (listed by k_place_lookups: k_reduce_long sums those)
         float acc[VEC];
 #pragma unroll
         for (int q = 0; q < VEC; q++) acc[q] = 0.f;
@@ -416,16 +432,18 @@ __global__ __launch_bounds__(256) void k_reduce_long(const SlotDesc* __restrict_
                                                      const uint32_t* __restrict__ ubase, int N, int dim, int combiner,
                                                      const uint32_t* __restrict__ seg_off,
                                                      const uint64_t* __restrict__ svals, float* __restrict__ flat,
-                                                     const uint32_t* __restrict__ long_list,
-                                                     const uint32_t* long_count, const DevStatus* status) {
+                                                     const uint32_t* __restrict__ mid_list,
+                                                     const uint32_t* __restrict__ huge_list,
+                                                     const uint32_t* counts, const DevStatus* status) {
     if (status->abort) return;
     __shared__ float part[LONG_PART_FLOATS];
     const int chunks = dim / VEC;
     const int groups = 256 / chunks;
     const int q = threadIdx.x / chunks, c = threadIdx.x - q * chunks;
-    const uint32_t n_long = *long_count;
+    // the frequent ones: the two lists k_place_lookups left (ORDER_MID lookups or more)
+    const uint32_t n_mid = counts[1], n_long = n_mid + counts[2];
     for (uint32_t k = blockIdx.x; k < n_long; k += gridDim.x) {
-        const uint32_t u = long_list[k];
+        const uint32_t u = k < n_mid ? mid_list[k] : huge_list[k - n_mid];
         const uint32_t lo = seg_off[u], hi = seg_off[u + 1];
         const float* pooled = descs[find_slot(ubase, N, u)].grads;
         float acc[VEC];

@@ -1956,12 +1956,11 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         const bool huge_in_lds = (size_t)batch * sizeof(uint32_t) <= t->huge_lds;
         const int huge_grid = huge_in_lds ? GRID_CAP : 64;
         Carver c{nullptr};
-        uint32_t *long_list, *long_count, *gcur, *seg_off, *tkey, *mid_list, *huge_list, *gcnt;
+        uint32_t *long_count, *gcur, *seg_off, *tkey, *mid_list, *huge_list, *gcnt;
         uint64_t *vals, *svals, *tval;
         float* flat;
         auto carve = [&](Carver& cv) {
-            long_count = cv.take<uint32_t>(4);  // lists of k_reduce_pooled, k_place_lookups (mid, huge)
-            long_list = cv.take<uint32_t>(L / LONG_SEGMENT + 1);
+            long_count = cv.take<uint32_t>(4);  // [1], [2]: entries of the lists of k_place_lookups (mid, huge)
             mid_list = cv.take<uint32_t>(L / ORDER_MID + 1);
             huge_list = cv.take<uint32_t>(L / ORDER_HUGE + 1);
             gcur = cv.take<uint32_t>(L);
@@ -1979,34 +1978,60 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         carve(c2);
         TN_LAUNCH(k_lookup_keys, dim3(lblocks), dim3(256), st, pd, p.lbase, N, (uint32_t)L, batch, vals, ds, long_count);
         // The lookups of every distinct sign side by side, ascending by example (= by position): into their
-        // sign's segment first, then ordered inside it.
-        const uint32_t place_cap = (uint32_t)(t->place_lds / sizeof(uint32_t));
-        TN_LAUNCH_LDS(k_place_lookups, dim3(N), dim3(PLACE_THREADS), t->place_lds, st, p.lbase, p.ubase, N, (uint32_t)L,
-                      p.u_of_gi, vals, tkey, tval, seg_off, gcur, place_cap, mid_list, huge_list, long_count, ds);
+        // sign's segment first, then ordered inside it.  A few workgroups per slot, each with an LDS counter per
+        // distinct index of its share of the slot (a slot has at most as many as lookups).
+        size_t max_len = 0;
+        for (int s = 0; s < N; s++) max_len = std::max<size_t>(max_len, (size_t)value_lens[s]);
+        // (one workgroup per slot: with several, each streaming the slot for its share of the distinct indices,
+        // the kernel took longer -- 0.20 against 0.17 ms with five, 0.16 with two -- as did a split by position,
+        // which needs a matrix of counts)
+        const uint32_t parts = 1;
+        const size_t place_bytes = std::min(t->place_lds, align_up((max_len / parts + 2) * sizeof(uint32_t), 256));
+        const uint32_t place_cap = (uint32_t)(place_bytes / sizeof(uint32_t));
+        TN_LAUNCH_LDS(k_place_lookups, dim3(N * parts), dim3(PLACE_THREADS), place_bytes, st, p.lbase, p.ubase, N, (uint32_t)L,
+                      p.u_of_gi, vals, tkey, tval, seg_off, gcur, place_cap, mid_list, huge_list, long_count, ds, parts);
+        // The three kernels that order the segments work on segments of their own (short, middle, huge), the two
+        // that sum them likewise (those below LONG_SEGMENT lookups, those from it on): a large batch runs them side
+        // by side on the table's streams.
+        const bool fork = !t->one_stream;
+        hipStream_t s_mid = fork ? t->side : st, s_huge = fork ? t->side2 : st;
+        if (fork) {
+            TN_HIP(hipEventRecord(t->fork_ev, st));
+            TN_HIP(hipStreamWaitEvent(t->side, t->fork_ev, 0));
+            TN_HIP(hipStreamWaitEvent(t->side2, t->fork_ev, 0));
+        }
         TN_LAUNCH(k_rank_short, dim3(launch_grid(L, 256, GRID_CAP * 4)), dim3(256), st, (uint32_t)L, tkey, tval, seg_off,
                   svals, ds);
-        TN_LAUNCH(k_rank_mid, dim3(launch_grid((int64_t)L / ORDER_MID + 1, 1, GRID_CAP * 2)), dim3(256), st, mid_list,
+        TN_LAUNCH(k_rank_mid, dim3(launch_grid((int64_t)L / ORDER_MID + 1, 1, GRID_CAP * 2)), dim3(256), s_mid, mid_list,
                   long_count, seg_off, tval, svals, ds);
         TN_LAUNCH_LDS(k_order_huge, dim3(launch_grid((int64_t)L / ORDER_HUGE + 1, 1, huge_grid)), dim3(256),
-                      huge_in_lds ? (size_t)batch * sizeof(uint32_t) : 0, st, huge_list, long_count, seg_off, tval, svals,
+                      huge_in_lds ? (size_t)batch * sizeof(uint32_t) : 0, s_huge, huge_list, long_count, seg_off, tval, svals,
                       (uint32_t)batch, huge_in_lds ? 1 : 0, gcnt, ds);
         // signs with LONG_SEGMENT lookups or more get a workgroup each instead of one thread group
+        static_assert(LONG_SEGMENT == ORDER_MID, "the lists of k_place_lookups are the frequent signs of k_reduce_long");
         const int chunks = vec ? grad_dim / 4 : grad_dim;
         const uint32_t long_min = chunks <= 256 ? LONG_SEGMENT : 0xFFFFFFFFu;
         const int long_blocks = launch_grid((int64_t)L / LONG_SEGMENT + 1, 1, GRID_CAP);
+        if (fork) {
+            // the frequent signs are summed on the side stream, behind the two kernels that ordered their segments
+            TN_HIP(hipEventRecord(t->join2_ev, t->side2));
+            TN_HIP(hipStreamWaitEvent(t->side, t->join2_ev, 0));
+        }
         if (vec) {
             TN_LAUNCH((k_reduce_pooled<4>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
-                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
-                      long_count);
-            TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), st, pd, p.ubase, N, grad_dim, combiner,
-                      seg_off, svals, flat, long_list, long_count, ds);
+                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min);
+            TN_LAUNCH((k_reduce_long<4>), dim3(long_blocks), dim3(256), s_mid, pd, p.ubase, N, grad_dim, combiner,
+                      seg_off, svals, flat, mid_list, huge_list, long_count, ds);
         } else {
             TN_LAUNCH((k_reduce_pooled<1>), dim3(launch_grid((int64_t)L * chunks, 256, GRID_CAP * 4)), dim3(256), st,
-                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min, long_list,
-                      long_count);
+                      pd, p.ubase, N, grad_dim, combiner, ds, seg_off, svals, flat, long_min);
             if (long_min != 0xFFFFFFFFu)
-                TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), st, pd, p.ubase, N, grad_dim,
-                          combiner, seg_off, svals, flat, long_list, long_count, ds);
+                TN_LAUNCH((k_reduce_long<1>), dim3(long_blocks), dim3(256), s_mid, pd, p.ubase, N, grad_dim,
+                          combiner, seg_off, svals, flat, mid_list, huge_list, long_count, ds);
+        }
+        if (fork) {
+            TN_HIP(hipEventRecord(t->join_ev, t->side));
+            TN_HIP(hipStreamWaitEvent(st, t->join_ev, 0));
         }
         src.flat = flat;
         return TN_OK;
