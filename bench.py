@@ -66,7 +66,7 @@ def step_algorithmic_bytes(opt, dim, L, U):
 
 # Launched on the table's side stream, concurrently with kernels of the caller's stream (the
 # other apply kernels; the ranking kernels of the remap): not on the step's critical path.
-SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_vec", "k_group_count", "k_group_offsets", "k_probe_recs")
+SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_big_adagrad", "k_apply_vec", "k_group_count", "k_group_offsets", "k_probe_recs")
 BIG_GROUP = 16  # records from which a sign is applied by k_apply_big (sparse_table.hip)
 
 
@@ -110,6 +110,7 @@ def kernel_algorithmic_bytes(name, opt, dim, shape):
         "k_apply_single": apply_bytes(shape["G1"], shape["G1"]),
         "k_apply_vec": apply_bytes(shape["Rm"], shape["Gm"]),
         "k_apply_big": apply_bytes(shape["Rb"], shape["Gb"]),
+        "k_apply_big_adagrad": apply_bytes(shape["Rb"], shape["Gb"]),
         "k_apply_scalar": apply_bytes(U, G),
     }
     return table.get(name.split("<")[0], 0)

@@ -894,7 +894,8 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
 // the arrays is first put together in LDS and then copied out in order; only where_u, indexed
 // by the distinct index of the record, stays a scattered store.  where_u[u] = {place in the member
 // list (with WHERE_ONE_TILE if all lookups of the record lie in one tile), table row of the record's sign
-// (rrow, from k_probe_recs)}; the groups get the rows too.
+// (rrow, from k_probe_recs)}; the groups get the rows too.  A group with big_k records or more is listed in
+// big_list and, with {row, first member, records, group}, in big_desc.
 //
 // SLOT_RANKS: a record carries its rank in its slot instead of the position of its first occurrence
 // (the pull of a small batch); its distinct index is the slot's base plus that rank.
@@ -907,8 +908,8 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                                                     const uint32_t* __restrict__ wordpre, uint32_t ids_cap,
                                                     uint32_t big_k, uint64_t* __restrict__ grp_sign,
                                                     uint32_t* __restrict__ grp_off, uint32_t* __restrict__ grp_cnt,
-                                                    uint32_t* __restrict__ big_list, Member* __restrict__ list,
-                                                    uint2* __restrict__ where_u,
+                                                    uint32_t* __restrict__ big_list, uint4* __restrict__ big_desc,
+                                                    Member* __restrict__ list, uint2* __restrict__ where_u,
                                                     const uint32_t* __restrict__ rrow,
                                                     uint32_t* __restrict__ grp_row, DevStatus* status,
                                                     const uint32_t* __restrict__ ubase, uint32_t n_slots) {
@@ -1010,7 +1011,11 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                     s_sign[n1 + idx] = r.sign;
                     s_off[n1 + idx] = top - (before + k - 1);
                     s_cnt[n1 + idx] = (uint16_t)k;
-                    if (is_big(k, big_k)) big_list[bb.w + bigidx] = g;
+                    if (is_big(k, big_k)) {
+                        big_list[bb.w + bigidx] = g;
+                        // (what k_apply_big would otherwise fetch through g: one round trip less per sign)
+                        big_desc[bb.w + bigidx] = make_uint4(rows[j], top - (before + k - 1), k, g);
+                    }
                 }
             }
         }

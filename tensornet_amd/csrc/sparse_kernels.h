@@ -2034,6 +2034,150 @@ __global__ __launch_bounds__(64) void k_apply_big(Store s, OptDev o, PushSrc src
                            gshow, gok, den, (int)threadIdx.x, blockIdx.x, gridDim.x, [] { __syncthreads(); });
 }
 
+// k_apply_big for AdaGrad rows of D elements, D a power of two from 4 to 64, on a plan whose big_desc lists
+// {row, first member, records, group} of every sign with many records (written by k_group_emit): one wavefront
+// per sign, its records up to BigTile<D>::CHUNK at a time.  The lanes tile (record, element) as
+// lane = record * D + element, 64 / D records a round, and keep the gradients of their rounds in registers, so
+// every gradient load of a chunk is in flight at once; the sign's description is asked for together with the
+// status, the row together with the first records.  The staging in LDS only turns the tile round -- a lane per
+// record for the sum of squares (double, in element order), a lane per element for the subtractions (in record
+// order) -- and every loop over it fetches several entries before it uses the first, so that no step of a chain
+// waits for LDS.  Operation for operation the arithmetic of apply_big_groups.
+template <int D>
+struct BigTile {
+    static constexpr int R = 64 / D;                                            // records a round
+    static constexpr int MOST = D == 32 ? 8 : 16;                               // (what the register file takes without spilling)
+    static constexpr int ROUNDS = BIG_CHUNK / R < MOST ? BIG_CHUNK / R : MOST;  // gradient registers of a lane
+    static constexpr int CHUNK = R * ROUNDS;
+    static constexpr int DP = D + 1;  // padded staging row: lanes walking down a column hit different banks
+};
+template <int D>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 8))) void k_apply_big_adagrad(
+    Store s, OptDev o, PushSrc src, DevStatus* status, const uint4* __restrict__ big_desc, uint32_t desc_cap,
+    const Member* __restrict__ list, const float* const* __restrict__ gaddr) {
+    using T = BigTile<D>;
+    constexpr int R = T::R, DP = T::DP;
+    __shared__ float gbuf[T::CHUNK * DP];
+    __shared__ const float* gptr[T::CHUNK];
+    __shared__ float den[T::CHUNK];
+    const int lane = (int)threadIdx.x;
+    const int li = lane & (D - 1), lm = lane / D;
+    uint4 head = big_desc[blockIdx.x < desc_cap ? blockIdx.x : desc_cap - 1];  // (before the status is known)
+    // a push launched on a plan that turned out not to be its batch's (the host redoes it), or whose inputs are unusable
+    if (status->mismatch | status->abort) return;
+    const uint32_t n_big = status->n_big;
+    constexpr double inv_d = 1.0 / (double)D;  // exact: D is a power of two
+    for (uint32_t bi = blockIdx.x; bi < n_big; bi += gridDim.x) {
+        if (bi != blockIdx.x) head = big_desc[bi];
+        const uint32_t row = head.x, off = head.y, k = head.z;
+        if (row > s.cap) continue;  // NO_ROW, or no row number at all: never address the table with it
+        float* wp = s.w + (uint64_t)row * s.wstride;
+        float* sp = s.st + (uint64_t)row * s.sstride;
+        float w = lane < D ? wp[lane] : 0.f;
+        float g2sum = sp[0], show = sp[1], click = sp[2];
+        bool any = false;
+        for (uint32_t c0 = 0; c0 < k; c0 += T::CHUNK) {
+            const int cn = (int)((k - c0) < (uint32_t)T::CHUNK ? (k - c0) : (uint32_t)T::CHUNK);
+            bool ok = false;
+            int sh = 0, ck = 0;
+            if (lane < cn) {
+                const float* gp = nullptr;
+                ok = record_at(src, list + off + c0, gaddr ? gaddr + off + c0 : nullptr, lane, gp, sh, ck);
+                gptr[lane] = gp;
+            }
+            const unsigned long long okmask = __ballot(ok);
+            const unsigned long long chunk_mask = cn == 64 ? ~0ull : (1ull << cn) - 1ull;
+            __syncthreads();
+            {
+                float v[T::ROUNDS];
+#pragma unroll
+                for (int q = 0; q < T::ROUNDS; q++) {
+                    const int m = lm + q * R;
+                    v[q] = (m < cn && ((okmask >> m) & 1ull)) ? gptr[m][li] : 0.f;
+                }
+#pragma unroll
+                for (int q = 0; q < T::ROUNDS; q++) gbuf[(lm + q * R) * DP + li] = v[q];
+            }
+            __syncthreads();
+            // add_g2sum / dim of record `lane`: double sum of float products in element order
+            double mq = 0.0;
+            if (lane < cn) {
+                const float* gr = gbuf + lane * DP;
+                constexpr int AT_ONCE = D < 16 ? D : 16;
+                double tot = 0.0;
+#pragma unroll
+                for (int i0 = 0; i0 < D; i0 += AT_ONCE) {
+                    float a[AT_ONCE];
+#pragma unroll
+                    for (int i = 0; i < AT_ONCE; i++) a[i] = gr[i0 + i];
+#pragma unroll
+                    for (int i = 0; i < AT_ONCE; i++) tot += (double)(a[i] * a[i]);
+                }
+                mq = tot * inv_d;
+            }
+            // g2sum after every record (float += double, rounded each time), show and click in record order:
+            // every lane runs the same chain on values read out of the records' lanes, lane m keeps the g2sum
+            // its record meets
+            const float fsh = (float)sh, fck = (float)ck;
+            float myg2 = 0.f;
+            if (okmask == chunk_mask) {
+                for (int m = 0; m < cn; m++) {
+                    show += lane_value(fsh, m);
+                    click += lane_value(fck, m);
+                    g2sum = (float)((double)g2sum + lane_value(mq, m));
+                    if (lane == m) myg2 = g2sum;
+                }
+            } else {
+                for (int m = 0; m < cn; m++) {
+                    if (!((okmask >> m) & 1ull)) continue;
+                    show += lane_value(fsh, m);
+                    click += lane_value(fck, m);
+                    g2sum = (float)((double)g2sum + lane_value(mq, m));
+                    if (lane == m) myg2 = g2sum;
+                }
+            }
+            if (lane < cn) den[lane] = o.eps + sqrtf(myg2);
+            __syncthreads();
+            // the steps lr * g / den of all records and elements (independent divisions, the operands of a few
+            // rounds fetched together); a record without a gradient row steps by zero, which leaves the weights
+            // as they are
+#pragma unroll 4
+            for (int m = lm; m < cn; m += R) {
+                const float gv = gbuf[m * DP + li], dn = den[m];
+                gbuf[m * DP + li] = ((okmask >> m) & 1ull) ? o.lr * gv / dn : 0.f;
+            }
+            __syncthreads();
+            // per element the subtractions in record order
+            if (lane < D) {
+                for (int m0 = 0; m0 < cn; m0 += 8) {
+                    float t[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) t[j] = m0 + j < cn ? gbuf[(m0 + j) * DP + lane] : 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) w -= t[j];
+                }
+            }
+            if (okmask) any = true;
+            if (lane == 0 && okmask != chunk_mask) atomicOr(&status->err, DEV_ERR_GRAD_ROWS);
+            __syncthreads();
+        }
+        if (any) {
+            if (lane < D) wp[lane] = w;
+            if (lane == 0) {
+                sp[0] = g2sum;
+                sp[1] = show;
+                sp[2] = click;
+                sp[3] = 0.f;  // no_show_days = 0
+                if (o.use_cvm) {
+                    wp[D] = show;
+                    wp[D + 1] = logf(click + 1) - logf(show + 1);
+                }
+            }
+        }
+    }
+}
+
+
 // Any dim / alignment: one thread per distinct sign, scalar loops.
 template <int KIND>
 __global__ __launch_bounds__(256) void k_apply_scalar(Store s, OptDev o, PushSrc src, DevStatus* status,

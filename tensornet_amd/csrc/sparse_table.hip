@@ -107,6 +107,7 @@ struct SparseTable {
     bool exact_verify = false; // pulls that leave fingerprints keep a copy of the signs as well, pushes compare that
     bool plan_exact = false;   // the plan holds such a copy
     uint32_t plan_big_k = BIG_GROUP_DEFAULT;  // records from which the plan lists a sign as one for k_apply_big
+    bool plan_big_desc = false;               // the plan's big_desc goes with its big_list (a pull grouped through LDS)
     hipStream_t side = nullptr;     // the signs with many records are applied here, beside the others
     hipStream_t side2 = nullptr;    // a pull probes the table here, beside the grouping of its distinct records
     // The slot descriptors of a call reach the device here while the caller's stream still runs the tail of the
@@ -525,6 +526,8 @@ struct Plan {
     Member* list;          // members of every group, ascending (with their show / click counts)
     uint2* where_u;        // record -> {its place in `list`, its group}
     uint32_t* big_list;    // groups with BIG_GROUP records or more
+    uint4* big_desc;       // {row, first member, records, group} of those groups (k_group_emit writes it, the other groupings do not)
+    uint32_t big_cap;      // entries of big_list / big_desc
     const float** gaddr;   // gradient row of every record of the groups with several records (a push fills it)
     uint64_t* vals_exact;  // copy of the signs beside their fingerprints (tn_sparse_table_set_exact_verify), else nullptr
 };
@@ -576,7 +579,9 @@ void carve_groups(Carver& c, Plan& p, size_t n) {
     p.grp_cnt = c.take<uint32_t>(n);
     p.list = c.take<Member>(n);
     p.where_u = c.take<uint2>(n);
-    p.big_list = c.take<uint32_t>(n / std::min<uint32_t>(BIG_GROUP, SMALL_BIG_GROUP) + 64);  // (the lowest threshold a plan may use)
+    p.big_cap = (uint32_t)(n / std::min<uint32_t>(BIG_GROUP, SMALL_BIG_GROUP) + 64);  // (the lowest threshold a plan may use)
+    p.big_list = c.take<uint32_t>(p.big_cap);
+    p.big_desc = c.take<uint4>(p.big_cap);
     p.gaddr = c.take<const float*>(n);
 }
 
@@ -886,8 +891,9 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
         }
         TN_LAUNCH((k_group_emit<false>), dim3(bblocks), dim3(EMIT_THREADS), st, w.nb2, w.cursor2, w.recs, w.aux,
                   own_offsets ? nullptr : w.bbase, w.bcounts, w.flag8, w.wordpre, L, big_threshold(s),
-                  p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow, p.grp_row, ds,
+                  p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.big_desc, p.list, p.where_u, w.rrow, p.grp_row, ds,
                   (const uint32_t*)nullptr, 0u);
+        t->plan_big_desc = true;
         return TN_OK;  // the rows were found beside the grouping
     } else if (N <= MASK_SLOTS)
         launch_mask_grouping(p, w, (int64_t)L, big_threshold(s), ushow, ds, st);
@@ -911,7 +917,8 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
 // auxiliary stream; the caller of this function records their end (see SparseTable::upd_ev).
 template <int KIND>
 int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, const PushSrc& src, DevStatus* ds,
-                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready, uint32_t big_k, bool detach) {
+                      const Plan& p, int64_t n_upper, hipStream_t st, bool addr_ready, uint32_t big_k, bool detach,
+                      bool big_desc) {
     const uint32_t ids_cap = (uint32_t)n_upper;
     const bool with_big = big_k != 0xFFFFFFFFu;
     const float* const* gaddr = (with_big && !src.infos && !src.flat) ? p.gaddr : nullptr;
@@ -930,9 +937,22 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
     }
     if (with_big) {
         const int gfloats = big_gbuf_floats(s.D);
-        TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(launch_grid(n_upper / BIG_GROUP + 1, 1, 16384)), dim3(64),
-                      big_lds_bytes(s.D), t->one_stream ? st : t->side, s, o, src, ds, p.big_list, p.grp_row, p.grp_off, p.grp_cnt,
-                      p.list, gfloats, gaddr);
+        const int big_blocks = launch_grid(n_upper / BIG_GROUP + 1, 1, 16384);
+        hipStream_t bst = t->one_stream ? st : t->side;
+#define TN_LAUNCH_BIG_ADAGRAD(DIM)                                                                                  \
+    TN_LAUNCH((k_apply_big_adagrad<DIM>), dim3(big_blocks), dim3(64), bst, s, o, src, ds, (const uint4*)p.big_desc, \
+              p.big_cap, p.list, gaddr)
+        // AdaGrad rows of a power-of-two dim on a plan that describes its frequent signs: the kernel made for them
+        const bool tiled = KIND == OPT_ADAGRAD && big_desc;
+        if (tiled && s.D == 4) TN_LAUNCH_BIG_ADAGRAD(4);
+        else if (tiled && s.D == 8) TN_LAUNCH_BIG_ADAGRAD(8);
+        else if (tiled && s.D == 16) TN_LAUNCH_BIG_ADAGRAD(16);
+        else if (tiled && s.D == 32) TN_LAUNCH_BIG_ADAGRAD(32);
+        else if (tiled && s.D == 64) TN_LAUNCH_BIG_ADAGRAD(64);
+        else
+            TN_LAUNCH_LDS((k_apply_big<KIND>), dim3(big_blocks), dim3(64), big_lds_bytes(s.D), bst, s, o, src, ds,
+                          p.big_list, p.grp_row, p.grp_off, p.grp_cnt, p.list, gfloats, gaddr);
+#undef TN_LAUNCH_BIG_ADAGRAD
     }
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
@@ -971,16 +991,17 @@ int lanes_per_group(const Store& s, bool vec_ok) {
 // Applies the grouped records; n_upper bounds the number of records.
 // addr_ready: p.gaddr already holds the gradient addresses of the multi-record groups' records.
 // big_k: the number of records from which the plan's grouping listed a sign for k_apply_big (0: the table's default).
+// big_desc: p.big_desc describes the signs of p.big_list (the plan of a pull that grouped through LDS).
 int launch_apply(SparseTable* t, const Plan& p, const PushSrc& src, DevStatus* ds, int64_t n_upper, bool vec_ok,
-                 hipStream_t st, bool addr_ready = false, uint32_t big_k = 0, bool detach = false) {
+                 hipStream_t st, bool addr_ready = false, uint32_t big_k = 0, bool detach = false, bool big_desc = false) {
     const Store& s = t->store;
     const OptDev o = make_optdev(t);
     const int lpg = lanes_per_group(s, vec_ok);
     if (big_k == 0) big_k = big_threshold(s);
     switch (o.kind) {
-        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
-        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
-        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach);
+        case OPT_ADAGRAD: return launch_apply_kind<OPT_ADAGRAD>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach, big_desc);
+        case OPT_ADAM: return launch_apply_kind<OPT_ADAM>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach, big_desc);
+        default: return launch_apply_kind<OPT_FTRL>(t, lpg, s, o, src, ds, p, n_upper, st, addr_ready, big_k, detach, big_desc);
     }
 }
 
@@ -1722,6 +1743,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                           t->small_state, parts);
             const uint32_t big_k = N <= SMALL_NO_BIG_SLOTS || big_threshold(s) == 0xFFFFFFFFu ? 0xFFFFFFFFu : SMALL_BIG_GROUP;
             t->plan_big_k = big_k;
+            t->plan_big_desc = false;  // (the small push's update kernel goes through big_list)
             // the grouping's first pass (one workgroup per second-level bucket) and, beside it, a thread per
             // (lookup position, part of a row) for the variables
             const int finish_blocks = (int)(((uint64_t)L * (uint64_t)(vec ? wdim / 4 : wdim) + GRP_THREADS - 1) / GRP_THREADS);
@@ -1735,7 +1757,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
                           t->small_state, parts, ds, reinterpret_cast<uint32_t*>(t->hpull), t->hseq + 0, seq);
             TN_LAUNCH((k_group_emit<true>), dim3(w.nb2), dim3(EMIT_THREADS), st, w.nb2, cur, w.recs, w.aux,
                       (const uint4*)nullptr, w.bcounts, (const uint8_t*)nullptr, (const uint32_t*)nullptr, (uint32_t)L,
-                      big_k, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.list, p.where_u, w.rrow,
+                      big_k, p.grp_sign, p.grp_off, p.grp_cnt, p.big_list, p.big_desc, p.list, p.where_u, w.rrow,
                       p.grp_row, ds, p.ubase, (uint32_t)N);
             TN_HIP(hipGetLastError());
             // the call returns when the second launch has reported: what follows is complete in stream order
@@ -1773,6 +1795,7 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         }
         t->plan_small = false;
         t->plan_big_k = big_threshold(t->store);
+        t->plan_big_desc = false;
         // Behind a push of the training loop the descriptors go in on the auxiliary stream, beside that push's
         // updates: those read the push's own descriptors and status block, and nothing of the scratch buffer.
         // (Same slot count: the arrays at the head of the plan buffer keep their places.)
@@ -2140,7 +2163,7 @@ int push_op_impl(uint32_t table_handle, int N, const int64_t* const* values, con
         if (!t->plan_has_show) TN_TRY(launch_counts());
         TN_TRY(prepare_src());
         TN_TRY(launch_apply(t, p, src, ds, (int64_t)L, vec, st, addr_in_verify, t->plan_big_k,
-                            t->detach_updates && !pooled));
+                            t->detach_updates && !pooled, t->plan_big_desc));
         if (t->detached_now) {
             // their end, for whoever touches the table next; the status goes out behind them (below)
             TN_HIP(hipEventRecord(t->apply_ev, t->aux));
