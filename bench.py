@@ -600,13 +600,14 @@ def main():
             ex = [torch.from_numpy(np.sort(crng.integers(0, cfg["batch"], v.numel()))).cuda() for v in values]
             pooled = [torch.randn((cfg["batch"], dim), device="cuda", generator=rng) * cfg["grad_sigma"] for _ in values]
             pull = tn.ops.BoundSparseTablePull(vars_, values, h)
+            combine = tn.ops.BoundEmbeddingLookupSparse(vars_, pull.mapped, ex, cfg["batch"], h, "mean")
             push = tn.ops.BoundSparseTablePushPooled(values, ex, pooled, labels, h, "mean")
-            cb.append((pull, push, vars_, ex))
+            cb.append((pull, combine, push))
 
         def cstep(i):
-            pull, push, vars_, ex = cb[i % len(cb)]
-            mapped = pull()
-            tn.ops.embedding_lookup_sparse(vars_, mapped, ex, cfg["batch"], h, "mean")
+            pull, combine, push = cb[i % len(cb)]
+            pull()
+            combine()
             push()
 
         for i in range(2):

@@ -148,34 +148,45 @@ def embedding_lookup_sparse(resources, mapped_values, example_ids, batch_size, t
     the rows resources[s][mapped_values[s][i]] of the lookups i of example b.
     example_ids[s][i] is the example of lookup i (SparseTensor.indices[:, 0]).
     Returns N float32 tensors [batch_size, dim]."""
-    n = len(mapped_values)
-    if len(resources) != n or len(example_ids) != n or n == 0:
-        raise ValueError("embedding_lookup_sparse needs one variable, id tensor and example-id tensor per slot")
-    for i in range(n):
-        _require(resources[i], torch.float32, "resources[%d]" % i)
-        _require(mapped_values[i], torch.int64, "mapped_values[%d]" % i)
-        _require(example_ids[i], torch.int64, "example_ids[%d]" % i)
-        if example_ids[i].numel() != mapped_values[i].numel():
-            raise ValueError("example_ids[%d] must have one entry per lookup" % i)
-    dim = resources[0].shape[1]
-    flat = torch.empty((n, batch_size, dim), dtype=torch.float32, device=resources[0].device)
-    out = list(flat.unbind(0))
-    rc = _lib.load().tn_sparse_table_combine_op(
-        table_handle,
-        n,
-        _lib.ptr_array([v.data_ptr() for v in mapped_values]),
-        _lib.i64_array([v.numel() for v in mapped_values]),
-        _lib.ptr_array([e.data_ptr() for e in example_ids]),
-        _lib.ptr_array([r.data_ptr() for r in resources]),
-        _lib.i64_array([r.shape[0] for r in resources]),
-        int(dim),
-        int(batch_size),
-        _combiner(combiner),
-        _lib.ptr_array([o.data_ptr() for o in out]),
-        _stream(),
-    )
-    _lib.check(rc)
-    return out
+    return BoundEmbeddingLookupSparse(resources, mapped_values, example_ids, batch_size, table_handle, combiner)()
+
+
+class BoundEmbeddingLookupSparse:
+    """embedding_lookup_sparse bound to fixed tensors (see BoundSparseTablePull): the variables and mapped ids of a
+    bound pull, the example ids, and outputs allocated once.  Calling it returns the N [batch_size, dim] tensors."""
+
+    def __init__(self, resources, mapped_values, example_ids, batch_size, table_handle, combiner="mean"):
+        n = len(mapped_values)
+        if len(resources) != n or len(example_ids) != n or n == 0:
+            raise ValueError("embedding_lookup_sparse needs one variable, id tensor and example-id tensor per slot")
+        for i in range(n):
+            _require(resources[i], torch.float32, "resources[%d]" % i)
+            _require(mapped_values[i], torch.int64, "mapped_values[%d]" % i)
+            _require(example_ids[i], torch.int64, "example_ids[%d]" % i)
+            if example_ids[i].numel() != mapped_values[i].numel():
+                raise ValueError("example_ids[%d] must have one entry per lookup" % i)
+        dim = resources[0].shape[1]
+        flat = torch.empty((n, batch_size, dim), dtype=torch.float32, device=resources[0].device)
+        self.out = list(flat.unbind(0))
+        self._keep = (list(resources), list(mapped_values), list(example_ids), flat)
+        self._fn = _lib.load().tn_sparse_table_combine_op
+        self._args = (
+            table_handle,
+            n,
+            _lib.ptr_array([v.data_ptr() for v in mapped_values]),
+            _lib.i64_array([v.numel() for v in mapped_values]),
+            _lib.ptr_array([e.data_ptr() for e in example_ids]),
+            _lib.ptr_array([r.data_ptr() for r in resources]),
+            _lib.i64_array([r.shape[0] for r in resources]),
+            int(dim),
+            int(batch_size),
+            _combiner(combiner),
+            _lib.ptr_array([o.data_ptr() for o in self.out]),
+        )
+
+    def __call__(self):
+        _lib.check(self._fn(*self._args, _stream()))
+        return self.out
 
 
 class BoundSparseTablePushPooled:
