@@ -31,7 +31,7 @@ def test_traffic_file_names_known_kernels():
     # the kernels of the cfg3 step all have their figure
     step = ["k_tile_dedup", "k_lds_dedup<true>", "k_lds_flags", "k_lds_assign<false>", "k_lds_mapped",
             "k_group_count", "k_group_emit", "k_probe_recs", "k_gather_vars<4>", "k_verify_values<true, false>",
-            "k_apply_single<KIND, 4>", "k_apply_vec<KIND, 4>", "k_apply_big<KIND>", "k_stage_in", "k_publish"]
+            "k_apply_single<KIND, 4>", "k_apply_vec<KIND, 4>", "k_apply_big_adagrad<DIM>", "k_stage_in", "k_publish"]
     per_launch, source = bench.measured_traffic(step)
     assert source["file"] == "profiles/cfg3_traffic.json" and source["profiled_at_commit"] == t["commit"]
     assert per_launch["k_apply_single"] > bench.kernel_algorithmic_bytes("k_apply_single", "AdaGrad", 16, SHAPE) * 0.5
