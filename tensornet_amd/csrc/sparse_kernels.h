@@ -1280,7 +1280,7 @@ __global__ __launch_bounds__(256) void k_member_grads(PushSrc src, const DevStat
 // entry to memory once.  A label that finds the table crowded goes to memory directly.
 //
 // What the signs are compared with: COPY, the plan's copy of them (the pulls that leave one: the small
-// batches' and the one through the global table); else the fingerprints that k_lds_hist left, one per 64 strided
+// batches' and the one through the global table); else the fingerprints that k_tile_dedup left, one per 64 strided
 // lookups of a tile (the lookups of one wavefront, here as there): 16 bytes to read instead of 512.  A
 // fingerprint is two 64-bit sums over the run, of mix64(sign) and of its halves exchanged, each term times an
 // odd weight drawn from the position.  One changed sign always alters the sums (the hash is a bijection, the
