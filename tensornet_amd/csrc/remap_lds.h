@@ -900,7 +900,7 @@ __global__ __launch_bounds__(256) void k_init_new_recs(Store s, OptDev o, uint64
 // SLOT_RANKS: a record carries its rank in its slot instead of the position of its first occurrence
 // (the pull of a small batch); its distinct index is the slot's base plus that rank.
 template <bool SLOT_RANKS>
-__global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6, 8))) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
+__global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(8, 8))) void k_group_emit(uint32_t nb2, const uint32_t* __restrict__ cursor2,
                                                     const GroupRec* __restrict__ recs, const uint2* __restrict__ aux,
                                                     const uint4* __restrict__ bbase,
                                                     const uint4* __restrict__ bcounts,
@@ -913,12 +913,15 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
                                                     const uint32_t* __restrict__ rrow,
                                                     uint32_t* __restrict__ grp_row, DevStatus* status,
                                                     const uint32_t* __restrict__ ubase, uint32_t n_slots) {
-    // [0, n1): the groups of one record (group = member); from n1 on: in s_list the members of the
-    // other groups, last group first, in s_sign / s_off / s_cnt those groups themselves
-    __shared__ Member s_list[GRP_CAP];
+    // [0, n1): the groups of one record (group = member); from n1 on: in s_mem the members of the other groups,
+    // last group first, in s_sign / s_row those groups themselves, whose offsets and sizes have arrays of their
+    // own (such a group has two records at least, so there are n / 2 of them at most).  A member entry is packed
+    // into eight bytes while it waits here {u | slot << 32 | show << 40}: 35 KB per workgroup, four to a CU.
+    __shared__ unsigned long long s_mem[GRP_CAP];
     __shared__ unsigned long long s_sign[GRP_CAP];
-    __shared__ uint32_t s_off[GRP_CAP], s_row[GRP_CAP];
-    __shared__ uint16_t s_cnt[GRP_CAP];  // at most GRP_SLOTS records per group
+    __shared__ uint32_t s_row[GRP_CAP];
+    __shared__ uint32_t s_off[GRP_CAP / 2];
+    __shared__ uint16_t s_cnt[GRP_CAP / 2];  // at most GRP_SLOTS records per group
     __shared__ uint4 s_part[EMIT_THREADS / 64];
     __shared__ uint32_t s_ub[SLOT_RANKS ? GRP_SLOTS + 1 : 1];  // the slots' bases (a small batch: one round trip less per record)
     if (SLOT_RANKS)
@@ -986,31 +989,27 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             const uint2 a = as[j];
             const uint32_t k = a.x >> 24, idx = a.x & 0xFFFu, bigidx = (a.x >> 12) & 0xFFFu;
             const uint32_t place = (a.y >> 16) & 0xFFu, sl = a.y >> 24;
-            Member m;
-            m.u = us[j];
-            m.slot = sl;
-            m.show = (int32_t)(r.cnt & REC_CNT_MASK);  // batch_show = occurrences (sparse_table_ops.cc:290-293)
-            m.click = 0;
+            // batch_show = occurrences (sparse_table_ops.cc:290-293), batch_click starts at zero
+            const unsigned long long m = (unsigned long long)us[j] | ((unsigned long long)sl << 32) |
+                                         ((unsigned long long)(r.cnt & REC_CNT_MASK) << 40);
             const uint32_t one_tile = (r.cnt & REC_ONE_TILE) ? WHERE_ONE_TILE : 0u;
             if (k == 1) {
                 const uint32_t g = bb.x + idx;
-                s_list[idx] = m;
+                s_mem[idx] = m;
                 s_sign[idx] = r.sign;
-                s_off[idx] = g;
-                s_cnt[idx] = 1;
                 s_row[idx] = rows[j];
-                where_u[m.u] = make_uint2(g | one_tile, rows[j]);
+                where_u[us[j]] = make_uint2(g | one_tile, rows[j]);
             } else {
                 const uint32_t g = ids_cap - 1 - (bb.y + idx);
                 const uint32_t before = a.y & 0xFFFFu;        // records of the bucket's earlier groups of this kind
                 const uint32_t t = before + k - 1 - place;    // local member: the group's last record first
-                s_list[n1 + t] = m;
-                where_u[m.u] = make_uint2((top - t) | one_tile, rows[j]);
+                s_mem[n1 + t] = m;
+                where_u[us[j]] = make_uint2((top - t) | one_tile, rows[j]);
                 if (place == 0) {
                     s_row[n1 + idx] = rows[j];  // every record of the sign was given the same row
                     s_sign[n1 + idx] = r.sign;
-                    s_off[n1 + idx] = top - (before + k - 1);
-                    s_cnt[n1 + idx] = (uint16_t)k;
+                    s_off[idx] = top - (before + k - 1);
+                    s_cnt[idx] = (uint16_t)k;
                     if (is_big(k, big_k)) {
                         big_list[bb.w + bigidx] = g;
                         // (what k_apply_big would otherwise fetch through g: one round trip less per sign)
@@ -1020,20 +1019,28 @@ __global__ __launch_bounds__(EMIT_THREADS) __attribute__((amdgpu_waves_per_eu(6,
             }
         }
         __syncthreads();
+        auto member = [](unsigned long long m) {
+            Member e;
+            e.u = (uint32_t)m;
+            e.slot = (uint32_t)(m >> 32) & 0xFFu;
+            e.show = (int32_t)(m >> 40);
+            e.click = 0;
+            return e;
+        };
         for (uint32_t i = threadIdx.x; i < n1; i += EMIT_THREADS) {
             const uint32_t g = bb.x + i;
-            list[g] = s_list[i];
+            list[g] = member(s_mem[i]);
             grp_sign[g] = s_sign[i];
-            grp_off[g] = s_off[i];
-            grp_cnt[g] = s_cnt[i];
+            grp_off[g] = g;  // (group = member)
+            grp_cnt[g] = 1;
             grp_row[g] = s_row[i];
         }
-        for (uint32_t i = threadIdx.x; i < nr; i += EMIT_THREADS) list[top - i] = s_list[n1 + i];
+        for (uint32_t i = threadIdx.x; i < nr; i += EMIT_THREADS) list[top - i] = member(s_mem[n1 + i]);
         for (uint32_t i = threadIdx.x; i < nm; i += EMIT_THREADS) {
             const uint32_t g = ids_cap - 1 - (bb.y + i);
             grp_sign[g] = s_sign[n1 + i];
-            grp_off[g] = s_off[n1 + i];
-            grp_cnt[g] = s_cnt[n1 + i];
+            grp_off[g] = s_off[i];
+            grp_cnt[g] = s_cnt[i];
             grp_row[g] = s_row[n1 + i];
         }
         __syncthreads();
