@@ -124,12 +124,6 @@ __global__ __launch_bounds__(256) void k_combine_fwd(const SlotDesc* __restrict_
     }
 }
 
-// out[0 .. n) = 0 (a slot without lookups)
-__global__ __launch_bounds__(256) void k_zero_f32(float* __restrict__ out, int64_t n) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = 0.f;
-}
-
 // Backward, step 1: the value of every lookup: its example in the high word, the number of
 // lookups of that example in the low word -- all the reduction needs to know about the lookup, so
 // that it reads them in the order of the distinct signs instead of chasing positions.  The first

@@ -95,11 +95,6 @@ __device__ __forceinline__ uint32_t group_bucket(uint64_t sign, uint32_t nb2) {
     return (uint32_t)__umul64hi(mix64(sign), (uint64_t)nb2);
 }
 
-__global__ __launch_bounds__(256) void k_zero_u32(uint32_t* p, uint32_t n) {
-    const uint32_t stride = gridDim.x * blockDim.x;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
-}
-
 // What a tile hands to a first-level bucket: one record per distinct sign of the tile (per slot, where a tile
 // spans several).  y: bits 0-31 the position of the sign's first occurrence in the tile, 32-43 its occurrences in
 // the tile (1 .. LDS_TILE), 44-55 the slot.
