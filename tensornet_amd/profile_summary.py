@@ -4,31 +4,31 @@ benchmark's roofline figures rest on:
     profiles/cfg3_adagrad_dim16_pull_push.md   kernel durations (kernel trace) and HBM traffic per launch
     profiles/cfg3_traffic.json                 {kernel: HBM bytes per launch}, which bench.py reads
 
-The runs (MI355X box, from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd $GRAFT_REPO_ROOT`):
+The runs (MI355X box, from the repository root, with TMPDIR=/tmp):
 
-    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_trace -o t -- python3 bench.py --steps 5 --warmup 2 --no-cpu --no-others --no-traffic
-    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o f -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic
-    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o w -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic
-    python3 bench.py --no-traffic > gpurun_out/bench_full.json
-    python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_trace --fetch gpurun_out/prof_fetch \\
-        --write gpurun_out/prof_write --bench gpurun_out/bench_full.json --commit <commit of the profiled tree>
+    rocprofv3 --kernel-trace --stats -d prof_out/prof_trace -o t -- python3 bench.py --steps 5 --warmup 2 --no-cpu --no-others --no-traffic
+    rocprofv3 --pmc FETCH_SIZE -d prof_out/prof_fetch -o f -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic
+    rocprofv3 --pmc WRITE_SIZE -d prof_out/prof_write -o w -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic
+    python3 bench.py --no-traffic > prof_out/bench_full.json
+    python3 -m tensornet_amd.profile_summary --trace prof_out/prof_trace --fetch prof_out/prof_fetch \\
+        --write prof_out/prof_write --bench prof_out/bench_full.json --commit <commit of the profiled tree>
 
 With --trace and --title only (no counter runs) it writes a table of kernel durations, e.g. for the small
 configurations, whose steps are a handful of short kernels (one run per configuration):
 
-    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_cfg1 -o t -- python3 bench.py --config cfg1 --steps 50 --warmup 5 \
+    rocprofv3 --kernel-trace --stats -d prof_out/prof_cfg1 -o t -- python3 bench.py --config cfg1 --steps 50 --warmup 5 \
         --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-traffic
-    python3 -m tensornet_amd.profile_summary --trace gpurun_out/prof_cfg1 --title "cfg1 ..." --out profiles/<name>.md [--append]
+    python3 -m tensornet_amd.profile_summary --trace prof_out/prof_cfg1 --title "cfg1 ..." --out profiles/<name>.md [--append]
 
 With --counters (one or more directories of `rocprofv3 --pmc <SQ counters>` runs of the same command, at most 8 SQ
 counters a run) and --title it writes the per-dispatch averages of those counters for the step's kernels and a few
 ratios of them (what share of its wavefronts' time a kernel waits, and on what):
 
     rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_WAIT_ANY SQ_WAIT_INST_ANY SQ_WAIT_INST_LDS SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT \
-        -d gpurun_out/pmc_a -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-others --no-traffic
+        -d prof_out/pmc_a -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-others --no-traffic
     rocprofv3 --pmc SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_LDS SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_ACTIVE_INST_VMEM SQ_ACTIVE_INST_VALU SQ_INST_LEVEL_VMEM \
-        -d gpurun_out/pmc_b -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-others --no-traffic
-    python3 -m tensornet_amd.profile_summary --counters gpurun_out/pmc_a gpurun_out/pmc_b --title "..." --out profiles/<name>.md
+        -d prof_out/pmc_b -o p -- python3 bench.py --steps 3 --warmup 1 --no-cpu --no-dense --no-combiner --no-decay --no-fallback --no-others --no-traffic
+    python3 -m tensornet_amd.profile_summary --counters prof_out/pmc_a prof_out/pmc_b --title "..." --out profiles/<name>.md
 
 FETCH_SIZE / WRITE_SIZE count in KiB per dispatch in units that are not bytes on every ASIC: both are
 scaled by the factor that makes the same counter reproduce the known traffic of the dense Adam stream of
