@@ -157,7 +157,15 @@ def main():
 
     traffic = {}
     out = ["# cfg3 pull+push (dim-16 AdaGrad, 16384 x 100 slots, 5e8 resident keys): rocprofv3 kernel trace and HBM traffic\n",
-           "Written by `python3 -m tensornet_amd.profile_summary` (its docstring holds the five commands) at commit `%s`.\n" % commit,
+           "Written at commit `%s` by (MI355X box, from the repository root, with TMPDIR=/tmp):\n" % commit,
+           "```\n"
+           "rocprofv3 --kernel-trace --stats -d prof_out/prof_trace -o t -- python3 bench.py --steps 5 --warmup 2 --no-cpu --no-others --no-traffic\n"
+           "rocprofv3 --pmc FETCH_SIZE -d prof_out/prof_fetch -o f -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic\n"
+           "rocprofv3 --pmc WRITE_SIZE -d prof_out/prof_write -o w -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-others --no-traffic\n"
+           "python3 bench.py --no-traffic > prof_out/bench_full.json\n"
+           "python3 -m tensornet_amd.profile_summary --trace prof_out/prof_trace --fetch prof_out/prof_fetch --write prof_out/prof_write "
+           "--bench prof_out/bench_full.json --commit %s\n"
+           "```\n" % commit,
            "Durations: per-dispatch `end - start` of the kernel trace, library kernels only. Traffic: FETCH_SIZE / WRITE_SIZE per "
            "dispatch, scaled by the factor the same counter shows for `k_dense_adam_v4` on 2e8 parameters (16 B read and 16 B "
            "written per parameter): FETCH x %.3f, WRITE x %.3f. `alg MB` = algorithmic bytes per launch "
