@@ -1714,8 +1714,12 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         // Detached updates of the push before read its plan in this same buffer.  A batch of the same slot count
         // and about the same size lays its plan out over it array by array, and what this call writes before it
         // orders itself behind them (the per-lookup arrays) stays clear of what they read; any other batch waits.
-        if (t->upd_pending && (N != t->upd_N || (size_t)((const char*)p.grp_sign - (const char*)t->plan_buf.p) >
-                                                    t->upd_groups_off + t->upd_slack))
+        // So does a call that keeps a copy of its signs for the exact comparison: the copy lies behind the group
+        // arrays, where a batch of another size puts it on top of the gradient addresses the updates still read,
+        // and the call's first kernel writes it.
+        if (t->upd_pending && (exact || N != t->upd_N ||
+                               (size_t)((const char*)p.grp_sign - (const char*)t->plan_buf.p) >
+                                   t->upd_groups_off + t->upd_slack))
             TN_TRY(order_after_updates(t, st));
         if (small) {
             TN_TRY(order_after_updates(t, st));

@@ -4,7 +4,8 @@ runs on every step.
 A pull of 3 M lookups or more spreads its work over the table's streams: the table is probed per distinct
 record beside the grouping and the ranking, every second-level bucket lists the rows it inserted, those rows
 are filled by a kernel of their own, and the push's descriptors are staged beside the pull's gather.  Here
-three such batches -- about 1 % of their lookups signs the table has never seen, then 25 % -- go through bound
+three such batches of slightly different sizes -- about 1 % of their lookups signs the table has never seen, then
+25 % -- go through bound
 pull and push ops with no host wait in between but the ones the calls make themselves, and every output is
 compared with the CPU oracle (core/kernels/sparse_table_ops.cc:170-265,317-368,
 core/ps/optimizer/optimizer_kernel.h:299-308): mapped ids and the pulled rows of resident signs bit for bit,
@@ -27,7 +28,7 @@ D = 16
 SCALE = 0.1
 HP = dict(learning_rate=0.01, initial_g2sum=0.1, initial_scale=SCALE, epsilon=1e-8)
 VOCAB = 400000
-SLOTS, PER = 64, 52000  # 3.33 M lookups: above the size from which a call uses the table's side streams
+SLOTS, PER = 64, 53500  # 3.3-3.4 M lookups: above the size from which a call uses the table's side streams
 
 
 def make_batches(pool):
@@ -35,14 +36,15 @@ def make_batches(pool):
     hot = pool[:30]
     batches = []
     next_fresh = 10 ** 9
-    for share in (0.01, 0.012, 0.25):
-        n_fresh = int(share * SLOTS * PER / 3)  # every fresh sign about three times, in one slot or in several
+    # (slots a little longer from batch to batch... and shorter again: every call lays its plan out anew)
+    for share, per in ((0.01, PER), (0.012, PER - 1500), (0.25, PER - 700)):
+        n_fresh = int(share * SLOTS * per / 3)  # every fresh sign about three times, in one slot or in several
         fresh = synth.splitmix64(np.arange(next_fresh, next_fresh + n_fresh, dtype=np.uint64)).view(np.int64)
         next_fresh += n_fresh
         values = []
         for _ in range(SLOTS):
-            v = pool[(rng.random(PER) ** 3 * VOCAB).astype(np.int64)]
-            take = rng.random(PER) < share
+            v = pool[(rng.random(per) ** 3 * VOCAB).astype(np.int64)]
+            take = rng.random(per) < share
             v[take] = fresh[rng.integers(0, n_fresh, int(take.sum()))]
             v[: len(hot)] = hot  # signs with a record in every slot
             values.append(v)
@@ -52,10 +54,12 @@ def make_batches(pool):
     return batches
 
 
-@pytest.mark.parametrize("detached", [False, True])
-def test_large_batches_with_new_signs_back_to_back(tn, oracle, detached):
+@pytest.mark.parametrize("detached,exact", [(False, False), (True, False), (True, True)])
+def test_large_batches_with_new_signs_back_to_back(tn, oracle, detached, exact):
     pair = Pair(tn, oracle, "AdaGrad", D, HP, reserve=3 * 10 ** 6, seed=5)
     tn.core.set_sparse_table_detached_updates(pair.h, detached)
+    # (with the exact comparison of the signs a pull also writes its copy of them, behind the plan's group arrays)
+    tn.core.set_sparse_table_exact_verify(pair.h, exact)
     base = pair.populate(synth.splitmix64(np.arange(1, VOCAB + 1, dtype=np.uint64)))
     pool = base.view(np.int64)
     batches = make_batches(pool)
