@@ -1705,6 +1705,9 @@ int tn_sparse_table_pull_op(uint32_t table_handle, int N, const int64_t* const* 
         Plan p{};
         Scratch w{};
         const bool exact = t->exact_verify && use_lds && !small;
+        // (a plan buffer that has to grow is freed first: not under detached updates that still read it)
+        if (t->upd_pending && carve_plan(nullptr, p, N, L, exact) > t->plan_buf.bytes)
+            TN_HIP(hipEventSynchronize(t->upd_ev));
         TN_TRY(t->plan_buf.ensure(carve_plan(nullptr, p, N, L, exact)));
         carve_plan((char*)t->plan_buf.p, p, N, L, exact);
         TN_TRY(t->ws.ensure(carve_scratch(nullptr, w, L, dt_entries, lds_scratch, t->distinct_est, N)));
