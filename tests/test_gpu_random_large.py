@@ -1,4 +1,4 @@
-"""Seeded random large batches (0.3 to 4.5 M lookups: one stream and several) through pull and push ops queued
+"""Seeded random large batches (1.2 to 4.5 M lookups: one stream and several) through pull and push ops queued
 back to back, three steps a case: the three optimizers, rows of 4 to 64 elements, 40 to 128 slots whose lengths
 differ from step to step (so that every call lays its plan out anew), up to 10 % signs the table has never seen,
 detached updates and the exact comparison of the signs switched on and off at random.  Against the CPU oracle
