@@ -64,9 +64,9 @@ def step_algorithmic_bytes(opt, dim, L, U):
     return 32 * L + U * (8 + 8 * dim + 4 * dim + 8 + 8 * dim + state_bytes(opt, dim))
 
 
-# Launched on the table's side stream, concurrently with kernels of the caller's stream (the
-# other apply kernels; the ranking kernels of the remap): not on the step's critical path.
-SIDE_STREAM_KERNELS = ("k_apply_big", "k_apply_big_adagrad", "k_apply_vec", "k_group_count", "k_group_offsets", "k_probe_recs")
+# Launched on the table's side streams, concurrently with kernels of the caller's stream (the other
+# update kernels; the ranking kernels of the remap).
+SIDE_STREAM_KERNELS = ("k_apply_single", "k_group_count", "k_group_offsets", "k_probe_recs")
 BIG_GROUP = 16  # records from which a sign is applied by k_apply_big (sparse_table.hip)
 
 
@@ -414,12 +414,12 @@ def main():
     lib.tn_profile_reset()
     per_step = {k: (c / psteps, ms / psteps) for k, (c, ms) in prof.items()}
     kernel_ms = sum(ms for _, ms in per_step.values())
-    # the dominant kernel of the step's critical path
+    # the dominant kernel: the one with the largest duration in the step
     shapes = [batch_shape(batches[i][0]) for i in list(prof_range)[:2]]
     G0 = shapes[0]["G"]
     mean_shape = {k: sum(sh[k] for sh in shapes) / len(shapes) for k in shapes[0]}
-    dominant = max((kv for kv in per_step.items() if not kv[0].startswith(SIDE_STREAM_KERNELS)
-                    and kernel_algorithmic_bytes(kv[0], opt_name, dim, mean_shape) > 0), key=lambda kv: kv[1][1])
+    dominant = max((kv for kv in per_step.items() if kernel_algorithmic_bytes(kv[0], opt_name, dim, mean_shape) > 0),
+                   key=lambda kv: kv[1][1])
     dname, (dcount, dms) = dominant
     avg_launch_s = dms / dcount * 1e-3
     mean_L, mean_U = total_L / args.steps, total_U / args.steps

@@ -910,8 +910,10 @@ int launch_build_plan(SparseTable* t, const Plan& p, const Scratch& w, int N, ui
 
 // The three kernels touch disjoint rows.  k_apply_single saturates the memory system (it runs
 // at the device's rate for random row updates); k_apply_big and k_apply_vec are bound by
-// dependent chains and instruction issue, so they run one after the other on the table's side
-// stream beside it, forked from and joined back into the caller's stream by events.
+// dependent chains and instruction issue, so they run one after the other beside it.  The pair is
+// the longer chain: it stays on the caller's stream and k_apply_single goes to the table's side
+// stream, forked from and joined back into the caller's stream by events (a kernel that waits for
+// an event of another stream starts 15-30 us late: better the chain that has the time to spare).
 //
 // detach: none of them on the caller's stream, which does not wait for them either -- k_apply_single on the
 // auxiliary stream; the caller of this function records their end (see SparseTable::upd_ev).
@@ -938,7 +940,7 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
     if (with_big) {
         const int gfloats = big_gbuf_floats(s.D);
         const int big_blocks = launch_grid(n_upper / BIG_GROUP + 1, 1, 16384);
-        hipStream_t bst = t->one_stream ? st : t->side;
+        hipStream_t bst = detach ? t->side : st;
 #define TN_LAUNCH_BIG_ADAGRAD(DIM)                                                                                  \
     TN_LAUNCH((k_apply_big_adagrad<DIM>), dim3(big_blocks), dim3(64), bst, s, o, src, ds, (const uint4*)p.big_desc, \
               p.big_cap, p.list, gaddr)
@@ -957,9 +959,9 @@ int launch_apply_kind(SparseTable* t, int lpg, const Store& s, const OptDev& o, 
 #define TN_LAUNCH_VEC(LPG)                                                                                        \
     do {                                                                                                          \
         TN_LAUNCH((k_apply_single<KIND, LPG>), dim3(launch_grid(n_upper * LPG, 256, GRID_CAP * 4)), dim3(256),    \
-                  detach ? t->aux : st, s, o, src, ds, p.grp_row, p.list);                                        \
+                  detach ? t->aux : (forked ? t->side : st), s, o, src, ds, p.grp_row, p.list);                   \
         TN_LAUNCH((k_apply_vec<KIND, LPG>), dim3(launch_grid(n_upper * LPG / 2, 256, GRID_CAP * 4)), dim3(256),    \
-                  forked ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,  \
+                  detach ? t->side : st, s, o, src, ds, p.grp_row, p.grp_off, p.grp_cnt, p.list, big_k, ids_cap,  \
                   gaddr);                                                                                         \
     } while (0)
     switch (lpg) {
